@@ -1,0 +1,200 @@
+// Entry points and C-ABI bridge of the MLA kernels.
+//
+// The dscuda:: functions validate their arguments before any runtime call
+// (the reference's check_shape, kernels/attention/mla/sm89.cu:20-24, throws
+// std::invalid_argument("MLA requires C=512 and RoPE=64") first thing, which
+// makes the error path testable on a host without a GPU) and then hand over to
+// the kernel translation units.  The extern "C" wrappers follow
+// benchmarks/bindings/mla_bridge.cu:12-73: status 0 / 1 and a thread-local
+// message, exceptions never cross the C boundary.
+#include "../../include/mla.h"
+
+#include "attn_kernels.h"
+#include "hip_common.h"
+
+#include <exception>
+#include <stdexcept>
+#include <string>
+
+namespace dscuda {
+namespace {
+
+void check_shape(int kv_rank, int rope_size) {
+    if (kv_rank != MLA_KV_RANK || rope_size != MLA_ROPE_SIZE) {
+        throw std::invalid_argument("MLA requires C=512 and RoPE=64");
+    }
+}
+
+void check_positive(const char* what, int batch_size, int tokens, int heads) {
+    if (batch_size <= 0 || tokens <= 0 || heads <= 0) {
+        throw std::invalid_argument(std::string(what) + " requires positive batch, sequence and head counts");
+    }
+}
+
+void check_prefill_heads(int qk_head_size, int v_head_size) {
+    const bool ok = (qk_head_size == 192 && v_head_size == 128) || (qk_head_size == 128 && v_head_size == 128) ||
+                    (qk_head_size == 64 && v_head_size == 64);
+    if (!ok) {
+        throw std::invalid_argument("MLA prefill requires (d_qk,d_v) in {(192,128),(128,128),(64,64)}");
+    }
+}
+
+}  // namespace
+
+void mla_compressed_attention_forward_cuda(__hip_bfloat16* output, float* logsumexp,
+                                           const __hip_bfloat16* query_latent, const __hip_bfloat16* query_rope,
+                                           const __hip_bfloat16* kv_latent, const __hip_bfloat16* key_rope,
+                                           int batch_size, int sequence_length, int heads, int kv_rank, int rope_size,
+                                           float scale, hipStream_t stream) {
+    check_shape(kv_rank, rope_size);
+    check_positive("MLA forward", batch_size, sequence_length, heads);
+    mla_absorbed_forward_dispatch(output, logsumexp, query_latent, query_rope, kv_latent, key_rope, batch_size,
+                                  sequence_length, heads, scale, stream);
+}
+
+void mla_compressed_attention_backward_cuda(
+    __hip_bfloat16* query_latent_gradient, __hip_bfloat16* query_rope_gradient, __hip_bfloat16* kv_latent_gradient,
+    __hip_bfloat16* key_rope_gradient, const __hip_bfloat16* output_gradient, const __hip_bfloat16* output,
+    const float* logsumexp, const __hip_bfloat16* query_latent, const __hip_bfloat16* query_rope,
+    const __hip_bfloat16* kv_latent, const __hip_bfloat16* key_rope, int batch_size, int sequence_length, int heads,
+    int kv_rank, int rope_size, float scale, hipStream_t stream) {
+    check_shape(kv_rank, rope_size);
+    check_positive("MLA backward", batch_size, sequence_length, heads);
+    mla_absorbed_backward_dispatch(query_latent_gradient, query_rope_gradient, kv_latent_gradient, key_rope_gradient,
+                                   output_gradient, output, logsumexp, query_latent, query_rope, kv_latent, key_rope,
+                                   batch_size, sequence_length, heads, scale, stream);
+}
+
+std::size_t mla_decode_workspace_elements(int batch_size, int heads, int splits, int kv_rank) {
+    // reference kernels/attention/mla/sm89.cu:539-541
+    return static_cast<std::size_t>(batch_size) * heads * splits * (kv_rank + 2);
+}
+
+void mla_decode_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                             const __hip_bfloat16* paged_kv_cache, const int* block_table, const int* cache_lengths,
+                             float* workspace, int batch_size, int heads, int kv_rank, int rope_size, int page_size,
+                             int pages_per_sequence, int splits, float scale, hipStream_t stream) {
+    check_shape(kv_rank, rope_size);
+    if (batch_size <= 0 || heads <= 0 || page_size <= 0 || pages_per_sequence <= 0 || splits <= 0) {
+        throw std::invalid_argument(
+            "MLA decode requires positive batch, head, page_size, pages_per_sequence and splits");
+    }
+    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
+                        heads, page_size, pages_per_sequence, splits, scale, stream);
+}
+
+void mla_prefill_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                              const __hip_bfloat16* key, const __hip_bfloat16* value, int batch_size,
+                              int sequence_length, int heads, int qk_head_size, int v_head_size, float scale,
+                              hipStream_t stream) {
+    check_prefill_heads(qk_head_size, v_head_size);
+    check_positive("MLA prefill forward", batch_size, sequence_length, heads);
+    attention_forward_dispatch(output, logsumexp, query, key, value, batch_size, sequence_length, heads, heads,
+                               qk_head_size, v_head_size, scale, stream);
+}
+
+std::size_t mla_prefill_backward_workspace_elements(int batch_size, int sequence_length, int heads,
+                                                    int /*qk_head_size*/, int /*v_head_size*/) {
+    return static_cast<std::size_t>(batch_size) * heads * sequence_length;
+}
+
+void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
+                               __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
+                               const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
+                               const __hip_bfloat16* key, const __hip_bfloat16* value, float* workspace,
+                               int batch_size, int sequence_length, int heads, int qk_head_size, int v_head_size,
+                               float scale, hipStream_t stream) {
+    check_prefill_heads(qk_head_size, v_head_size);
+    check_positive("MLA prefill backward", batch_size, sequence_length, heads);
+    if (workspace == nullptr) {
+        throw std::invalid_argument("MLA prefill backward requires a workspace");
+    }
+    attention_backward_dispatch(query_gradient, key_gradient, value_gradient, output_gradient, output, logsumexp, query,
+                                key, value, workspace, batch_size, sequence_length, heads, qk_head_size, v_head_size,
+                                scale, stream);
+}
+
+}  // namespace dscuda
+
+namespace {
+thread_local std::string last_error;
+
+template <typename Call>
+int guarded(Call&& call) {
+    try {
+        call();
+        return 0;
+    } catch (const std::exception& error) {
+        last_error = error.what();
+        return 1;
+    }
+}
+}  // namespace
+
+extern "C" const char* dscuda_mla_last_error() {
+    return last_error.c_str();
+}
+
+extern "C" int dscuda_mla_forward(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
+                                  const __hip_bfloat16* query_rope, const __hip_bfloat16* latent,
+                                  const __hip_bfloat16* key_rope, int batch, int sequence, int heads, int rank,
+                                  int rope, float scale, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_compressed_attention_forward_cuda(output, lse, query, query_rope, latent, key_rope, batch,
+                                                      sequence, heads, rank, rope, scale, stream);
+    });
+}
+
+extern "C" int dscuda_mla_backward(__hip_bfloat16* dquery, __hip_bfloat16* dquery_rope, __hip_bfloat16* dlatent,
+                                   __hip_bfloat16* dkey_rope, const __hip_bfloat16* dout,
+                                   const __hip_bfloat16* output, const float* lse, const __hip_bfloat16* query,
+                                   const __hip_bfloat16* query_rope, const __hip_bfloat16* latent,
+                                   const __hip_bfloat16* key_rope, int batch, int sequence, int heads, int rank,
+                                   int rope, float scale, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_compressed_attention_backward_cuda(dquery, dquery_rope, dlatent, dkey_rope, dout, output, lse,
+                                                       query, query_rope, latent, key_rope, batch, sequence, heads,
+                                                       rank, rope, scale, stream);
+    });
+}
+
+extern "C" std::size_t dscuda_mla_workspace_elements(int batch, int heads, int splits, int rank) {
+    return dscuda::mla_decode_workspace_elements(batch, heads, splits, rank);
+}
+
+extern "C" int dscuda_mla_decode(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
+                                 const __hip_bfloat16* paged_cache, const int* block_table, const int* lengths,
+                                 float* workspace, int batch, int heads, int rank, int rope, int page_size, int pages,
+                                 int splits, float scale, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_decode_forward_cuda(output, lse, query, paged_cache, block_table, lengths, workspace, batch,
+                                        heads, rank, rope, page_size, pages, splits, scale, stream);
+    });
+}
+
+extern "C" int dscuda_mla_prefill_forward(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
+                                          const __hip_bfloat16* key, const __hip_bfloat16* value, int batch,
+                                          int sequence, int heads, int qk_head_size, int v_head_size, float scale,
+                                          hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_prefill_forward_cuda(output, lse, query, key, value, batch, sequence, heads, qk_head_size,
+                                         v_head_size, scale, stream);
+    });
+}
+
+extern "C" std::size_t dscuda_mla_prefill_backward_workspace_elements(int batch, int sequence, int heads,
+                                                                      int qk_head_size, int v_head_size) {
+    return dscuda::mla_prefill_backward_workspace_elements(batch, sequence, heads, qk_head_size, v_head_size);
+}
+
+extern "C" int dscuda_mla_prefill_backward(__hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,
+                                           const __hip_bfloat16* dout, const __hip_bfloat16* output, const float* lse,
+                                           const __hip_bfloat16* query, const __hip_bfloat16* key,
+                                           const __hip_bfloat16* value, float* workspace, int batch, int sequence,
+                                           int heads, int qk_head_size, int v_head_size, float scale,
+                                           hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_prefill_backward_cuda(dquery, dkey, dvalue, dout, output, lse, query, key, value, workspace,
+                                          batch, sequence, heads, qk_head_size, v_head_size, scale, stream);
+    });
+}

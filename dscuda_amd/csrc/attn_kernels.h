@@ -1,0 +1,52 @@
+// Internal launch interface between the public entry points (api_*.hip) and
+// the kernel translation units.  Every function validates nothing: the entry
+// points have already checked shapes.  All of them enqueue on `stream` and
+// return without synchronising.
+#pragma once
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+
+namespace dscuda {
+
+// attn_fwd.hip -- causal forward, per-head K/V (flash attention and MLA prefill).
+// query [B,S,Hq,d_qk], key [B,S,Hkv,d_qk], value [B,S,Hkv,d_v], output
+// [B,S,Hq,d_v], logsumexp [B,Hq,S].
+void attention_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                                const __hip_bfloat16* key, const __hip_bfloat16* value, int batch_size,
+                                int sequence_length, int query_heads, int key_value_heads, int qk_head_size,
+                                int v_head_size, float scale, hipStream_t stream);
+
+// attn_bwd.hip -- recompute backward of the above for Hq == Hkv.
+// delta workspace [B,H,S] fp32.
+void attention_backward_dispatch(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
+                                 __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
+                                 const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
+                                 const __hip_bfloat16* key, const __hip_bfloat16* value, float* delta, int batch_size,
+                                 int sequence_length, int heads, int qk_head_size, int v_head_size, float scale,
+                                 hipStream_t stream);
+
+// mla_absorbed.hip -- absorbed (C=512, R=64) causal forward and backward with
+// one shared latent KV head.
+void mla_absorbed_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query_latent,
+                                   const __hip_bfloat16* query_rope, const __hip_bfloat16* kv_latent,
+                                   const __hip_bfloat16* key_rope, int batch_size, int sequence_length, int heads,
+                                   float scale, hipStream_t stream);
+
+void mla_absorbed_backward_dispatch(__hip_bfloat16* query_latent_gradient, __hip_bfloat16* query_rope_gradient,
+                                    __hip_bfloat16* kv_latent_gradient, __hip_bfloat16* key_rope_gradient,
+                                    const __hip_bfloat16* output_gradient, const __hip_bfloat16* output,
+                                    const float* logsumexp, const __hip_bfloat16* query_latent,
+                                    const __hip_bfloat16* query_rope, const __hip_bfloat16* kv_latent,
+                                    const __hip_bfloat16* key_rope, int batch_size, int sequence_length, int heads,
+                                    float scale, hipStream_t stream);
+
+// mla_decode.hip -- absorbed single-token decode over a paged latent cache.
+void mla_decode_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                         const __hip_bfloat16* paged_kv_cache, const int* block_table, const int* cache_lengths,
+                         float* workspace, int batch_size, int heads, int page_size, int pages_per_sequence,
+                         int splits, float scale, hipStream_t stream);
+
+}  // namespace dscuda

@@ -1,0 +1,109 @@
+// Shared host/device helpers for the gfx950 attention kernels.
+//
+// Host side: HIP_CHECK turns a failing runtime call into a std::runtime_error
+// carrying file:line and the evaluated expression, the same contract as the
+// reference's CUDA_CHECK (include/cuda_common.h:10-25,
+// kernels/common/cuda_common.cu:24-32).  The C-ABI bridges catch it and hand
+// the text back through dscuda_*_last_error().
+//
+// Device side: vector typedefs for the bf16 MFMA builtins and the few
+// cross-lane / conversion primitives every kernel uses.  Lane layouts of the
+// two MFMA shapes used here (wave64, l = lane id):
+//
+//   mfma_f32_32x32x16_bf16   A: row l%32, k = 8*(l/32)+j      (8 bf16 / lane)
+//                            B: col l%32, k = 8*(l/32)+j
+//                            C: col l%32, row 8*(i/4)+4*(l/32)+i%4, i = 0..15
+//   mfma_f32_16x16x32_bf16   A: row l%16, k = 8*(l/16)+j
+//                            B: col l%16, k = 8*(l/16)+j
+//                            C: col l%16, row 4*(l/16)+i, i = 0..3
+//
+// Because the contraction index only has to agree between A and B, any
+// permutation of k that both operands share gives the same product; the
+// kernels use that to feed a C-layout tile straight back in as a B operand.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+
+namespace dscuda {
+
+inline void hip_check(hipError_t result, const char* expression, const char* file, int line) {
+    if (result == hipSuccess) {
+        return;
+    }
+    std::ostringstream message;
+    message << "HIP failure at " << file << ':' << line << " while evaluating " << expression << ": "
+            << hipGetErrorString(result);
+    throw std::runtime_error(message.str());
+}
+
+#define HIP_CHECK(expression) ::dscuda::hip_check((expression), #expression, __FILE__, __LINE__)
+
+using bf16_t = __hip_bfloat16;
+
+#if defined(__HIP_DEVICE_COMPILE__) || defined(__HIPCC__)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+// Value held by the lane 32 places away, combined with the lane's own by a
+// symmetric op.  v_permlane32_swap exchanges the upper half of its first
+// operand with the lower half of its second, so feeding the same register to
+// both leaves {own, other} (in one order or the other) in the two results.
+__device__ __forceinline__ float half_wave_max(float value) {
+    auto swapped = __builtin_amdgcn_permlane32_swap(__float_as_uint(value), __float_as_uint(value), false, false);
+    return fmaxf(__uint_as_float(swapped[0]), __uint_as_float(swapped[1]));
+}
+
+__device__ __forceinline__ float half_wave_sum(float value) {
+    auto swapped = __builtin_amdgcn_permlane32_swap(__float_as_uint(value), __float_as_uint(value), false, false);
+    return __uint_as_float(swapped[0]) + __uint_as_float(swapped[1]);
+}
+
+// Two fp32 -> packed bf16 (round to nearest even, one v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16(float low, float high) {
+    f32x2 pair = {low, high};
+    bf16x2 packed = __builtin_convertvector(pair, bf16x2);
+    return __builtin_bit_cast(uint32_t, packed);
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+    return __uint_as_float(bits16 << 16);
+}
+
+// XCD-aware work-item order.  Workgroups are handed to the 8 XCDs round-robin
+// by linear id; every XCD has a private L2.  Items are grouped so that the
+// `inner` items that share operands (the query blocks of one head) run on one
+// XCD back to back, and `outer` groups (heads) are dealt across XCDs.
+// Returns (outer index, inner index) for a linear workgroup id; falls back to
+// the plain order when `outer` is not a multiple of 8.
+__device__ __forceinline__ void xcd_order(int linear, int outer, int inner, int& outer_index, int& inner_index) {
+    constexpr int XCDS = 8;
+    if (outer % XCDS == 0) {
+        const int xcd = linear % XCDS;
+        const int slot = linear / XCDS;
+        outer_index = xcd + XCDS * (slot / inner);
+        inner_index = slot % inner;
+    } else {
+        outer_index = linear / inner;
+        inner_index = linear % inner;
+    }
+}
+
+#endif  // device helpers
+
+}  // namespace dscuda

@@ -1,0 +1,157 @@
+"""Operator-level callers of the C-ABI entry points.
+
+Each function takes torch tensors that already live on the GPU, allocates the
+outputs with torch (the caller owns every buffer, as in
+``benchmarks/mla.py:56-57,69,111``) and calls one ``dscuda_*`` symbol on
+torch's current stream.  Signatures of the ctypes bindings are the ones the
+reference harness declares (``benchmarks/mla.py:27-32``,
+``benchmarks/flash_attention.py:36-37``).
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .common import F, I, P, bind, checked, library, pointers, stream
+
+
+def _require_cuda(*tensors):
+    for tensor in tensors:
+        if not tensor.is_cuda:
+            raise RuntimeError("dscuda_amd operators need GPU tensors; there is no CPU path")
+        if not tensor.is_contiguous():
+            raise RuntimeError("dscuda_amd operators need contiguous tensors")
+
+
+class _Mla:
+    def __init__(self):
+        lib = library("mla")
+        self.lib = lib
+        self.forward = bind(lib, "dscuda_mla_forward", [P] * 6 + [I] * 5 + [F, P])
+        self.backward = bind(lib, "dscuda_mla_backward", [P] * 11 + [I] * 5 + [F, P])
+        self.decode = bind(lib, "dscuda_mla_decode", [P] * 7 + [I] * 7 + [F, P])
+        self.workspace = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
+        self.prefill_forward = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
+        self.prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
+        self.prefill_workspace = bind(
+            lib, "dscuda_mla_prefill_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
+
+
+class _Flash:
+    def __init__(self):
+        lib = library("flash_attention")
+        self.lib = lib
+        self.forward = bind(lib, "dscuda_flash_forward", [P] * 5 + [I] * 5 + [F, P])
+
+
+_mla = None
+_flash = None
+
+
+def mla_library() -> _Mla:
+    global _mla
+    if _mla is None:
+        _mla = _Mla()
+    return _mla
+
+
+def flash_library() -> _Flash:
+    global _flash
+    if _flash is None:
+        _flash = _Flash()
+    return _flash
+
+
+def flash_forward(query, key, value, scale, out=None, lse=None):
+    """query [B,T,Hq,D], key/value [B,T,Hkv,D] bf16 -> (O [B,T,Hq,D] bf16, LSE [B,Hq,T] fp32)."""
+    _require_cuda(query, key, value)
+    b, t, hq, d = query.shape
+    hkv = key.shape[2]
+    out = torch.empty_like(query) if out is None else out
+    lse = torch.empty(b, hq, t, device=query.device, dtype=torch.float32) if lse is None else lse
+    lib = flash_library()
+    checked(lib.lib, "flash", lib.forward(*pointers((out, lse, query, key, value)), b, t, hq, hkv, d, scale, stream()))
+    return out, lse
+
+
+def mla_prefill_forward(query, key, value, scale, out=None, lse=None):
+    """query/key [B,S,H,d_qk], value [B,S,H,d_v] bf16 -> (O [B,S,H,d_v] bf16, LSE [B,H,S] fp32)."""
+    _require_cuda(query, key, value)
+    b, s, h, dqk = query.shape
+    dv = value.shape[-1]
+    out = torch.empty(b, s, h, dv, device=query.device, dtype=torch.bfloat16) if out is None else out
+    lse = torch.empty(b, h, s, device=query.device, dtype=torch.float32) if lse is None else lse
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.prefill_forward(
+        *pointers((out, lse, query, key, value)), b, s, h, dqk, dv, scale, stream()))
+    return out, lse
+
+
+def mla_prefill_backward(dout, out, lse, query, key, value, scale, workspace=None, grads=None):
+    """-> (dQ, dK [B,S,H,d_qk], dV [B,S,H,d_v]) bf16, overwritten."""
+    _require_cuda(dout, out, lse, query, key, value)
+    b, s, h, dqk = query.shape
+    dv = value.shape[-1]
+    lib = mla_library()
+    if workspace is None:
+        workspace = torch.empty(lib.prefill_workspace(b, s, h, dqk, dv), device=query.device, dtype=torch.float32)
+    if grads is None:
+        grads = (torch.empty_like(query), torch.empty_like(key), torch.empty_like(value))
+    checked(lib.lib, "mla", lib.prefill_backward(
+        *pointers((*grads, dout, out, lse, query, key, value, workspace)), b, s, h, dqk, dv, scale, stream()))
+    return grads
+
+
+def mla_forward(query_latent, query_rope, kv_latent, key_rope, scale, out=None, lse=None):
+    """Absorbed causal MLA forward (dscuda_mla_forward)."""
+    _require_cuda(query_latent, query_rope, kv_latent, key_rope)
+    b, t, h, c = query_latent.shape
+    r = query_rope.shape[-1]
+    out = torch.empty_like(query_latent) if out is None else out
+    lse = torch.empty(b, h, t, device=query_latent.device, dtype=torch.float32) if lse is None else lse
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.forward(
+        *pointers((out, lse, query_latent, query_rope, kv_latent, key_rope)), b, t, h, c, r, scale, stream()))
+    return out, lse
+
+
+def mla_backward(dout, out, lse, query_latent, query_rope, kv_latent, key_rope, scale, grads=None):
+    """Absorbed MLA backward (dscuda_mla_backward) -> (dq_lat, dq_rope, dlatent, dk_rope)."""
+    _require_cuda(dout, out, lse, query_latent, query_rope, kv_latent, key_rope)
+    b, t, h, c = query_latent.shape
+    r = query_rope.shape[-1]
+    if grads is None:
+        grads = tuple(torch.empty_like(x) for x in (query_latent, query_rope, kv_latent, key_rope))
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.backward(
+        *pointers((*grads, dout, out, lse, query_latent, query_rope, kv_latent, key_rope)),
+        b, t, h, c, r, scale, stream()))
+    return grads
+
+
+def mla_decode_workspace(batch, heads, splits, rank=512, device="cuda"):
+    lib = mla_library()
+    return torch.empty(lib.workspace(batch, heads, splits, rank), device=device, dtype=torch.float32)
+
+
+def mla_decode(packed_query, paged_cache, block_table, lengths, scale, splits=8, rank=512,
+               workspace=None, out=None, lse=None):
+    """packed_query [B,1,H,C+R], paged_cache [blocks,page,1,C+R], block_table int32 [B,pages],
+    lengths int32 [B] -> (O [B,1,H,C] bf16, LSE [B,H,1] fp32)."""
+    _require_cuda(packed_query, paged_cache, block_table, lengths)
+    b, _, h, width = packed_query.shape
+    rope = width - rank
+    page_size = paged_cache.shape[1]
+    pages = block_table.shape[1]
+    device = packed_query.device
+    if workspace is None:
+        workspace = mla_decode_workspace(b, h, splits, rank, device)
+    out = torch.empty(b, 1, h, rank, device=device, dtype=torch.bfloat16) if out is None else out
+    lse = torch.empty(b, h, 1, device=device, dtype=torch.float32) if lse is None else lse
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.decode(
+        *pointers((out, lse, packed_query, paged_cache, block_table, lengths, workspace)),
+        b, h, rank, rope, page_size, pages, splits, scale, stream()))
+    return out, lse

@@ -1,0 +1,47 @@
+// Public C++ API and C-ABI of the MI355X (gfx950) causal flash-attention
+// forward.  Keeps the name, argument order and meaning of the reference's
+// include/flash_attention.h:12-24 with the HIP spellings of the platform
+// types.  The caller owns all buffers; the call enqueues on `stream`, does not
+// synchronise and allocates nothing.
+#pragma once
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_runtime.h>
+
+namespace dscuda {
+
+// Fuses causal QK^T, online softmax and PV without materialising the T x T
+// score matrix.  query/output BF16 [B,T,Hq,D], key/value BF16 [B,T,Hkv,D],
+// natural-log logsumexp FP32 [B,Hq,T].  Hq must be divisible by Hkv (query
+// head h reads kv head h / (Hq/Hkv)), T must be a positive multiple of 64
+// (the reference's rule, kernels/attention/flash_attention/sm89_forward.cu:
+// 226-232) and D must be 64 or 128 (the reference accepts 128 only).
+void flash_attention_forward_cuda(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* key,
+    const __hip_bfloat16* value,
+    int batch_size,
+    int sequence_length,
+    int query_heads,
+    int key_value_heads,
+    int head_size,
+    float scale,
+    hipStream_t stream = nullptr);
+
+}  // namespace dscuda
+
+// ---- C ABI (libdscuda_flash_attention_bench.so) -----------------------------
+// Replaces reference benchmarks/bindings/flash_attention_bridge.cu:13-30.
+extern "C" {
+
+const char* dscuda_flash_last_error();  // flash_attention_bridge.cu:13-15
+
+int dscuda_flash_forward(  // flash_attention_bridge.cu:17-30
+    __hip_bfloat16* output, float* logsumexp,
+    const __hip_bfloat16* query, const __hip_bfloat16* key, const __hip_bfloat16* value,
+    int batch, int sequence, int query_heads, int key_value_heads, int dimension,
+    float scale, hipStream_t stream);
+
+}  // extern "C"

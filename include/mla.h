@@ -1,0 +1,212 @@
+// Public C++ API and C-ABI of the MI355X (gfx950) Multi-head Latent Attention
+// kernels.  The first four functions keep the names, argument order and
+// meaning of the reference's include/mla.h:18-81 with the HIP spellings of
+// the two platform types (hipStream_t, __hip_bfloat16: both binary-identical
+// to the reference's for a ctypes / dlsym caller).  The *_prefill_* functions
+// are additive: the per-head (128 nope + 64 rope | 128 value) form has no
+// counterpart in the reference.
+//
+// Conventions shared by every entry point:
+//   * all activation / gradient buffers are BF16, statistics (logsumexp,
+//     workspaces) are FP32, natural-log logsumexp of the *scaled* scores;
+//   * the caller owns every buffer, including workspaces; the library
+//     allocates nothing and keeps no state between calls;
+//   * work is enqueued on `stream` without synchronising, so calls may be
+//     captured into a HIP graph;
+//   * invalid arguments throw std::invalid_argument / std::runtime_error
+//     before anything is launched; the C-ABI wrappers turn that into status 1
+//     plus a thread-local message.
+#pragma once
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+
+namespace dscuda {
+
+constexpr int MLA_KV_RANK = 512;   // reference include/mla.h:10
+constexpr int MLA_ROPE_SIZE = 64;  // reference include/mla.h:11
+
+// Absorbed-query causal MLA forward.  Replaces reference include/mla.h:18-31.
+// query_latent [B,T,H,C], query_rope [B,T,H,R], kv_latent [B,T,C], key_rope
+// [B,T,R], output [B,T,H,C], logsumexp [B,H,T].  C must be 512 and R 64; B, T
+// and H are free, T need not be a multiple of any tile.
+void mla_compressed_attention_forward_cuda(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query_latent,
+    const __hip_bfloat16* query_rope,
+    const __hip_bfloat16* kv_latent,
+    const __hip_bfloat16* key_rope,
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int kv_rank,
+    int rope_size,
+    float scale,
+    hipStream_t stream = nullptr);
+
+// Absorbed-query MLA backward, recomputing probabilities from the saved FP32
+// logsumexp.  Replaces reference include/mla.h:35-53.  The four gradient
+// buffers are overwritten; every gradient row has exactly one writer, so the
+// result is deterministic and needs no workspace (the reference's ownership
+// rule, kernels/attention/mla/sm89.cu:2).
+void mla_compressed_attention_backward_cuda(
+    __hip_bfloat16* query_latent_gradient,
+    __hip_bfloat16* query_rope_gradient,
+    __hip_bfloat16* kv_latent_gradient,
+    __hip_bfloat16* key_rope_gradient,
+    const __hip_bfloat16* output_gradient,
+    const __hip_bfloat16* output,
+    const float* logsumexp,
+    const __hip_bfloat16* query_latent,
+    const __hip_bfloat16* query_rope,
+    const __hip_bfloat16* kv_latent,
+    const __hip_bfloat16* key_rope,
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int kv_rank,
+    int rope_size,
+    float scale,
+    hipStream_t stream = nullptr);
+
+// FP32 elements of decode workspace.  Replaces reference include/mla.h:57-61;
+// same formula, B*H*splits*(C+2), so buffers sized by either library fit.
+std::size_t mla_decode_workspace_elements(
+    int batch_size,
+    int heads,
+    int splits,
+    int kv_rank);
+
+// Absorbed decode of one packed BF16 query [B,1,H,C+R] against a paged cache
+// [blocks,page,1,C+R] with block table [B,pages_per_sequence] and per-sequence
+// lengths (>= 1).  Replaces reference include/mla.h:63-81.  `splits` bounds
+// how finely a sequence may be partitioned (and with it the workspace); the
+// result does not depend on it.
+void mla_decode_forward_cuda(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* paged_kv_cache,
+    const int* block_table,
+    const int* cache_lengths,
+    float* workspace,
+    int batch_size,
+    int heads,
+    int kv_rank,
+    int rope_size,
+    int page_size,
+    int pages_per_sequence,
+    int splits,
+    float scale,
+    hipStream_t stream = nullptr);
+
+// ---- additive: per-head MLA prefill (no counterpart in the reference) ------
+//
+// query/key [B,S,H,d_qk] with the rope slice stored after the nope slice,
+// value/output [B,S,H,d_v], logsumexp [B,H,S]; causal.  Supported head
+// geometries: (d_qk,d_v) = (192,128), (128,128), (64,64).
+void mla_prefill_forward_cuda(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* key,
+    const __hip_bfloat16* value,
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int qk_head_size,
+    int v_head_size,
+    float scale,
+    hipStream_t stream = nullptr);
+
+// FP32 elements of workspace the prefill backward needs (row-wise
+// delta = sum(dO * O), [B,H,S]).
+std::size_t mla_prefill_backward_workspace_elements(
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int qk_head_size,
+    int v_head_size);
+
+// Recompute-based backward of mla_prefill_forward_cuda from the saved BF16
+// output and FP32 logsumexp.  dQ/dK [B,S,H,d_qk] and dV [B,S,H,d_v] are
+// overwritten; every gradient row has exactly one writer (no atomics), dQ is
+// produced by its own pass over the key blocks.
+void mla_prefill_backward_cuda(
+    __hip_bfloat16* query_gradient,
+    __hip_bfloat16* key_gradient,
+    __hip_bfloat16* value_gradient,
+    const __hip_bfloat16* output_gradient,
+    const __hip_bfloat16* output,
+    const float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* key,
+    const __hip_bfloat16* value,
+    float* workspace,
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int qk_head_size,
+    int v_head_size,
+    float scale,
+    hipStream_t stream = nullptr);
+
+}  // namespace dscuda
+
+// ---- C ABI (libdscuda_mla_bench.so) ----------------------------------------
+// Status 0 = ok, 1 = error; the message of the last error on the calling
+// thread is returned by dscuda_mla_last_error() and stays valid until the next
+// error on that thread.  Replaces reference benchmarks/bindings/mla_bridge.cpp
+// symbols (mla_bridge.cu:12-73); argument order is identical.
+extern "C" {
+
+const char* dscuda_mla_last_error();  // mla_bridge.cu:12-14
+
+int dscuda_mla_forward(  // mla_bridge.cu:16-31
+    __hip_bfloat16* output, float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* query_rope,
+    const __hip_bfloat16* latent, const __hip_bfloat16* key_rope,
+    int batch, int sequence, int heads, int rank, int rope, float scale,
+    hipStream_t stream);
+
+int dscuda_mla_backward(  // mla_bridge.cu:33-51
+    __hip_bfloat16* dquery, __hip_bfloat16* dquery_rope,
+    __hip_bfloat16* dlatent, __hip_bfloat16* dkey_rope,
+    const __hip_bfloat16* dout, const __hip_bfloat16* output, const float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* query_rope,
+    const __hip_bfloat16* latent, const __hip_bfloat16* key_rope,
+    int batch, int sequence, int heads, int rank, int rope, float scale,
+    hipStream_t stream);
+
+std::size_t dscuda_mla_workspace_elements(  // mla_bridge.cu:53-56
+    int batch, int heads, int splits, int rank);
+
+int dscuda_mla_decode(  // mla_bridge.cu:58-73
+    __hip_bfloat16* output, float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* paged_cache,
+    const int* block_table, const int* lengths, float* workspace,
+    int batch, int heads, int rank, int rope, int page_size, int pages, int splits,
+    float scale, hipStream_t stream);
+
+// additive (no counterpart in the reference)
+int dscuda_mla_prefill_forward(
+    __hip_bfloat16* output, float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* key, const __hip_bfloat16* value,
+    int batch, int sequence, int heads, int qk_head_size, int v_head_size, float scale,
+    hipStream_t stream);
+
+std::size_t dscuda_mla_prefill_backward_workspace_elements(
+    int batch, int sequence, int heads, int qk_head_size, int v_head_size);
+
+int dscuda_mla_prefill_backward(
+    __hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,
+    const __hip_bfloat16* dout, const __hip_bfloat16* output, const float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* key, const __hip_bfloat16* value,
+    float* workspace,
+    int batch, int sequence, int heads, int qk_head_size, int v_head_size, float scale,
+    hipStream_t stream);
+
+}  // extern "C"

@@ -1,0 +1,78 @@
+"""GPU parity of the causal forward kernels (flash attention and per-head MLA
+prefill) against the fp32 oracle, through the C-ABI."""
+
+import pytest
+import torch
+
+from dscuda_amd.harness import configs, ops
+from oracle import attention_oracle as oracle
+from tests.parity import announce, assert_close_bf16, assert_close_lse
+
+pytestmark = pytest.mark.gpu
+
+
+def _flash_case(cuda, batch, seq, q_heads, kv_heads, dim, seed, factor):
+    q, k, v, scale = configs.flash_forward_inputs(batch, seq, q_heads, kv_heads, dim, seed, factor)
+    announce("flash_forward", dict(B=batch, T=seq, Hq=q_heads, Hkv=kv_heads, D=dim, seed=seed))
+    out, lse = ops.flash_forward(q.to(cuda), k.to(cuda), v.to(cuda), scale)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.causal_attention_forward(q, k, v, scale)
+    assert_close_bf16("O", out, expected)
+    assert_close_lse("LSE", lse, expected_lse)
+
+
+@pytest.mark.parametrize("shape", configs.FLASH_TEST)
+def test_flash_reference_test_shapes(cuda, shape):
+    # benchmarks/flash_attention.py:41-47, inputs scaled by 0.5 as at :61-63
+    _flash_case(cuda, *shape, seed=2026, factor=0.5)
+
+
+def test_flash_workload_1(cuda):
+    # B=1, H=8, S=512, D=64, N(0,1) inputs from seed 0
+    _flash_case(cuda, 1, 512, 8, 8, 64, seed=0, factor=1.0)
+
+
+@pytest.mark.parametrize("shape", [(1, 512, 8, 2, 128), (1, 1024, 8, 1, 128), (2, 2048, 8, 8, 128),
+                                   (1, 512, 8, 2, 64), (1, 4096, 16, 4, 128)])
+def test_flash_more_shapes(cuda, shape):
+    _flash_case(cuda, *shape, seed=11, factor=0.5)
+
+
+@pytest.mark.parametrize("batch,seq,heads", [(1, 1, 1), (2, 17, 3), (1, 65, 4), (1, 128, 8), (2, 257, 4),
+                                             (1, 300, 2), (1, 1024, 16)])
+def test_mla_prefill_forward_small(cuda, batch, seq, heads):
+    # ragged sequence lengths as in the reference's MLA test shapes (benchmarks/mla.py:35-39)
+    q, k, v, scale = configs.mla_prefill_inputs(batch, seq, heads, seed=5)
+    announce("mla_prefill_forward", dict(B=batch, S=seq, H=heads))
+    out, lse = ops.mla_prefill_forward(q.to(cuda), k.to(cuda), v.to(cuda), scale)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.causal_attention_forward(q, k, v, scale)
+    assert_close_bf16("O", out, expected)
+    assert_close_lse("LSE", lse, expected_lse)
+
+
+def test_mla_prefill_forward_invariants(cuda):
+    """Row 0 attends to key 0 only: O[0] = V[0], LSE[0] = scale * q0.k0."""
+    q, k, v, scale = configs.mla_prefill_inputs(1, 256, 4, seed=6)
+    out, lse = ops.mla_prefill_forward(q.to(cuda), k.to(cuda), v.to(cuda), scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out[0, 0].cpu(), v[0, 0])
+    expected = (q[0, 0].float() * k[0, 0].float()).sum(-1) * scale
+    assert (lse[0, :, 0].cpu() - expected).abs().max() <= 1e-4
+
+
+def test_mla_prefill_forward_workload_2(cuda):
+    """S=4096, H=128, 192/192/128 from seed 1 with RoPE; the oracle is run on a
+    sample of heads (first, last and two inner ones) to keep the CPU time bounded."""
+    q, k, v, scale = configs.mla_prefill_inputs()
+    announce("mla_prefill_forward workload 2", tuple(q.shape))
+    out, lse = ops.mla_prefill_forward(q.to(cuda), k.to(cuda), v.to(cuda), scale)
+    torch.cuda.synchronize()
+    out, lse = out.cpu(), lse.cpu()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    heads = [0, 37, 90, 127]
+    expected, expected_lse = oracle.causal_attention_forward(q, k, v, scale, heads=heads)
+    assert_close_bf16("O", out[:, :, heads], expected)
+    assert_close_lse("LSE", lse[:, heads], expected_lse)
+    # size-independent property on every head: row 0 reproduces V[0]
+    assert torch.equal(out[0, 0], v[0, 0])

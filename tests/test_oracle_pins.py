@@ -1,0 +1,279 @@
+"""Pins of the CPU oracle: every function of ``oracle/attention_oracle.py`` is
+checked against something that does not share its formula -- a library routine
+(``scaled_dot_product_attention``, ``autograd``), an fp64 brute-force loop, a
+closed form of the reference's constant-fill profiler inputs, or an invariant
+the mathematics fixes.  A dropped term, a sign error, a transposed operand or a
+wrong mask fails at least one of these."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attention_oracle as oracle
+
+
+def _rand(shape, seed, factor=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float64) * factor).to(dtype)
+
+
+# ---------------------------------------------------------------------------
+# causal attention forward
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dqk,dv,hq,hkv", [(64, 64, 4, 4), (192, 128, 3, 3), (128, 128, 8, 2), (128, 128, 4, 1)])
+def test_forward_matches_sdpa(dqk, dv, hq, hkv):
+    b, s = 2, 97
+    q, k, v = _rand((b, s, hq, dqk), 1), _rand((b, s, hkv, dqk), 2), _rand((b, s, hkv, dv), 3)
+    scale = dqk ** -0.5
+    out, lse = oracle.causal_attention_forward(q, k, v, scale)
+    group = hq // hkv
+    kk, vv = k.repeat_interleave(group, 2), v.repeat_interleave(group, 2)
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), kk.transpose(1, 2), vv.transpose(1, 2),
+                                         is_causal=True, scale=scale).transpose(1, 2)
+    assert (out - ref).abs().max() < 2e-5
+    scores = torch.einsum("bqhd,bkhd->bhqk", q, kk) * scale
+    scores = scores.masked_fill(~torch.ones(s, s, dtype=torch.bool).tril(), -math.inf)
+    assert (lse - torch.logsumexp(scores, -1)).abs().max() < 2e-5
+
+
+def test_forward_brute_force_fp64():
+    """Triple loop in numpy float64, no masking tensor, no softmax routine."""
+    b, s, h, dqk, dv = 1, 9, 2, 6, 5
+    q, k, v = (_rand(shape, seed, dtype=torch.float64) for seed, shape in
+               enumerate([(b, s, h, dqk), (b, s, h, dqk), (b, s, h, dv)], 10))
+    scale = 0.37
+    out, lse = oracle.causal_attention_forward(q, k, v, scale)
+    qn, kn, vn = q.numpy(), k.numpy(), v.numpy()
+    for hh in range(h):
+        for i in range(s):
+            weights = [math.exp(scale * float(np.dot(qn[0, i, hh], kn[0, j, hh]))) for j in range(i + 1)]
+            total = sum(weights)
+            expected = sum(w * vn[0, j, hh] for j, w in enumerate(weights)) / total
+            assert np.allclose(out[0, i, hh].numpy(), expected, atol=1e-12)
+            assert abs(lse[0, hh, i].item() - math.log(total)) < 1e-12
+
+
+def test_forward_invariants():
+    b, s, h, dqk, dv = 1, 33, 2, 192, 128
+    q, k, v = _rand((b, s, h, dqk), 20, 0.5), _rand((b, s, h, dqk), 21, 0.5), _rand((b, s, h, dv), 22, 0.5)
+    scale = dqk ** -0.5
+    out, lse = oracle.causal_attention_forward(q, k, v, scale)
+    # row 0 sees key 0 only
+    assert torch.allclose(out[:, 0], v[:, 0], atol=1e-6)
+    assert torch.allclose(lse[:, :, 0], (q[:, 0] * k[:, 0]).sum(-1) * scale, atol=1e-5)
+    # adding a constant c to every score (extra dimension with q=1, k=c/scale) shifts LSE by c, keeps O
+    shift = 0.75
+    q2 = torch.cat([q, torch.ones(b, s, h, 1)], -1)
+    k2 = torch.cat([k, torch.full((b, s, h, 1), shift / scale)], -1)
+    out2, lse2 = oracle.causal_attention_forward(q2, k2, v, scale)
+    assert torch.allclose(out2, out, atol=1e-5)
+    assert torch.allclose(lse2, lse + shift, atol=1e-5)
+    # constant V passes through untouched (probabilities sum to one)
+    out3, _ = oracle.causal_attention_forward(q, k, torch.full_like(v, 0.3), scale)
+    assert torch.allclose(out3, torch.full_like(out3, 0.3), atol=1e-6)
+    # the head subset selects, it does not change values
+    sub, sub_lse = oracle.causal_attention_forward(q, k, v, scale, heads=[1])
+    assert torch.equal(sub[:, :, 0], out[:, :, 1]) and torch.equal(sub_lse[:, 0], lse[:, 1])
+
+
+# ---------------------------------------------------------------------------
+# attention backward
+# ---------------------------------------------------------------------------
+
+def _autograd_reference(q, k, v, dout, scale):
+    q, k, v = (x.clone().requires_grad_() for x in (q, k, v))
+    s = q.shape[1]
+    scores = torch.einsum("bqhd,bkhd->bhqk", q, k) * scale
+    scores = scores.masked_fill(~torch.ones(s, s, dtype=torch.bool).tril(), -math.inf)
+    out = torch.einsum("bhqk,bkhd->bqhd", scores.softmax(-1), v)
+    return torch.autograd.grad(out, (q, k, v), dout)
+
+
+@pytest.mark.parametrize("dqk,dv", [(192, 128), (64, 64)])
+def test_backward_matches_autograd(dqk, dv):
+    b, s, h = 2, 41, 3
+    q, k, v = (_rand(shape, seed, 0.5, torch.float64) for seed, shape in
+               enumerate([(b, s, h, dqk), (b, s, h, dqk), (b, s, h, dv)], 30))
+    dout = _rand((b, s, h, dv), 33, 1.0, torch.float64)
+    scale = dqk ** -0.5
+    out, lse = oracle.causal_attention_forward(q, k, v, scale)
+    dq, dk, dv_ = oracle.attention_backward(dout, out, lse, q, k, v, scale)
+    rq, rk, rv = _autograd_reference(q, k, v, dout, scale)
+    for name, a, r in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv_, rv)):
+        assert (a - r).abs().max() < 1e-10, name
+
+
+def test_backward_finite_differences():
+    b, s, h, dqk, dv = 1, 7, 1, 4, 3
+    q, k, v = (_rand(shape, seed, 1.0, torch.float64) for seed, shape in
+               enumerate([(b, s, h, dqk), (b, s, h, dqk), (b, s, h, dv)], 40))
+    dout = _rand((b, s, h, dv), 43, 1.0, torch.float64)
+    scale = 0.6
+    out, lse = oracle.causal_attention_forward(q, k, v, scale)
+    grads = oracle.attention_backward(dout, out, lse, q, k, v, scale)
+
+    def loss(qq, kk, vv):
+        return (oracle.causal_attention_forward(qq, kk, vv, scale)[0] * dout).sum().item()
+
+    eps = 1e-6
+    for index, (tensor, grad) in enumerate(zip((q, k, v), grads)):
+        flat = tensor.reshape(-1)
+        for position in range(0, flat.numel(), 3):
+            plus, minus = tensor.clone(), tensor.clone()
+            plus.reshape(-1)[position] += eps
+            minus.reshape(-1)[position] -= eps
+            args_p = [q, k, v]
+            args_m = [q, k, v]
+            args_p[index], args_m[index] = plus, minus
+            numeric = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(numeric - grad.reshape(-1)[position].item()) < 1e-6
+
+
+def test_backward_row_sum_of_dscore_is_zero():
+    """sum_k dS[q,k] = 0  <=>  dQ is orthogonal to nothing in particular but
+    dS K summed against a constant key gives zero: with K constant along the
+    sequence, dQ must vanish."""
+    b, s, h, dqk, dv = 1, 19, 2, 16, 8
+    q = _rand((b, s, h, dqk), 50, 1.0, torch.float64)
+    k = _rand((b, 1, h, dqk), 51, 1.0, torch.float64).expand(b, s, h, dqk).contiguous()
+    v = _rand((b, s, h, dv), 52, 1.0, torch.float64)
+    dout = _rand((b, s, h, dv), 53, 1.0, torch.float64)
+    out, lse = oracle.causal_attention_forward(q, k, v, 0.25)
+    dq, _, _ = oracle.attention_backward(dout, out, lse, q, k, v, 0.25)
+    assert dq.abs().max() < 1e-12
+
+
+# ---------------------------------------------------------------------------
+# absorbed MLA
+# ---------------------------------------------------------------------------
+
+def test_mla_forward_is_mqa_over_concatenated_heads():
+    b, t, h = 2, 37, 5
+    ql, qr = _rand((b, t, h, 512), 60, 0.25), _rand((b, t, h, 64), 61, 0.25)
+    c, kr = _rand((b, t, 512), 62, 0.25), _rand((b, t, 64), 63, 0.25)
+    scale = 576 ** -0.5
+    out, lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, oracle.causal_mask(t))
+    q = torch.cat([ql, qr], -1)
+    k = torch.cat([c, kr], -1)[:, :, None]
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2).expand(b, h, t, 576),
+                                         c[:, None].expand(b, h, t, 512), is_causal=True, scale=scale)
+    assert (out - ref.transpose(1, 2)).abs().max() < 2e-5
+    # and equals the per-head oracle fed with the broadcast KV head
+    out2, lse2 = oracle.causal_attention_forward(q, k, c[:, :, None], scale)
+    assert (out - out2).abs().max() < 2e-5 and (lse - lse2).abs().max() < 2e-5
+    rounded, lse3 = oracle.mla_forward(ql, qr, c, kr, scale, oracle.causal_mask(t))
+    assert rounded.dtype == torch.bfloat16 and torch.equal(rounded, out.bfloat16()) and torch.equal(lse3, lse)
+
+
+def test_mla_constant_fill_closed_form():
+    """Constants of benchmarks/attention/benchmark_mla.cu:38-47 (q_lat=1/8, q_rope=-1/16, c=1/4,
+    k_rope=1/32, dO=1/64, scale=1/24): every score is (16-0.125)/24, O == 0.25,
+    LSE[t] = score + ln(t+1); dP == delta so dS == 0 and only the value path
+    feeds dLatent: dLatent[k] = H * dO * (Harm(T) - Harm(k))."""
+    b, t, h = 1, 24, 3
+    ql = torch.full((b, t, h, 512), 0.125)
+    qr = torch.full((b, t, h, 64), -0.0625)
+    c = torch.full((b, t, 512), 0.25)
+    kr = torch.full((b, t, 64), 0.03125)
+    scale = 1.0 / 24.0
+    mask = oracle.causal_mask(t)
+    out, lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, mask)
+    score = (512 * 0.125 * 0.25 - 64 * 0.0625 * 0.03125) / 24
+    assert abs(score - 0.6614583333) < 1e-9
+    assert torch.allclose(out, torch.full_like(out, 0.25), atol=1e-6)
+    expected_lse = score + torch.log(torch.arange(1, t + 1, dtype=torch.float32))
+    assert torch.allclose(lse, expected_lse[None, None].expand(b, h, t), atol=1e-5)
+    dout = torch.full((b, t, h, 512), 0.015625)
+    dq, dqr, dlat, dkr = oracle.mla_backward_unrounded(dout, out, lse, ql, qr, c, kr, scale, mask)
+    assert dq.abs().max() < 1e-6 and dqr.abs().max() < 1e-6 and dkr.abs().max() < 1e-6
+    harmonic = torch.cumsum(1.0 / torch.arange(1, t + 1, dtype=torch.float64), 0)
+    harm_before = torch.cat([torch.zeros(1, dtype=torch.float64), harmonic[:-1]])
+    expected = (h * 0.015625 * (harmonic[-1] - harm_before)).float()
+    assert torch.allclose(dlat, expected[None, :, None].expand(b, t, 512), atol=1e-5)
+
+
+def test_mla_backward_matches_autograd():
+    """The way the reference builds its expected gradients (benchmarks/mla.py:108-110)."""
+    b, t, h = 2, 17, 3
+    tensors = [_rand(shape, seed, 0.25, torch.float64) for seed, shape in
+               enumerate([(b, t, h, 512), (b, t, h, 64), (b, t, 512), (b, t, 64)], 70)]
+    dout = _rand((b, t, h, 512), 74, 0.2, torch.float64)
+    scale = 576 ** -0.5
+    mask = oracle.causal_mask(t)
+    leaves = [x.clone().requires_grad_() for x in tensors]
+    out, lse = oracle.mla_forward_unrounded(*leaves, scale, mask)
+    expected = torch.autograd.grad(out, leaves, dout)
+    actual = oracle.mla_backward_unrounded(dout, out.detach(), lse.detach(), *tensors, scale, mask)
+    for a, e in zip(actual, expected):
+        assert (a - e).abs().max() < 1e-10
+    rounded = oracle.mla_backward(dout, out.detach(), lse.detach(), *tensors, scale, mask)
+    assert all(r.dtype == torch.bfloat16 for r in rounded)
+
+
+# ---------------------------------------------------------------------------
+# decode
+# ---------------------------------------------------------------------------
+
+def test_decode_matches_sdpa_with_length_mask():
+    b, n, h = 3, 70, 4
+    q = _rand((b, 1, h, 576), 80, 0.5)
+    cache = _rand((b, n, 576), 81, 0.5)
+    lengths = torch.tensor([1, 33, 70])
+    scale = 192 ** -0.5
+    out, lse = oracle.mla_decode_unrounded(q, cache, lengths, scale)
+    assert out.shape == (b, 1, h, 512) and lse.shape == (b, h, 1)
+    for i in range(b):
+        ln = int(lengths[i])
+        keys = cache[i, :ln][None, None].expand(1, h, ln, 576)
+        ref = F.scaled_dot_product_attention(q[i].transpose(0, 1)[None], keys, keys[..., :512], scale=scale)
+        assert (out[i, 0] - ref[0, :, 0]).abs().max() < 2e-5
+        scores = torch.einsum("hd,kd->hk", q[i, 0], cache[i, :ln]) * scale
+        assert (lse[i, :, 0] - torch.logsumexp(scores, -1)).abs().max() < 2e-5
+
+
+def test_decode_full_length_equals_last_prefill_row():
+    b, t, h = 2, 29, 3
+    ql, qr = _rand((b, t, h, 512), 90, 0.25), _rand((b, t, h, 64), 91, 0.25)
+    c, kr = _rand((b, t, 512), 92, 0.25), _rand((b, t, 64), 93, 0.25)
+    scale = 576 ** -0.5
+    out, lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, oracle.causal_mask(t))
+    packed_q = torch.cat([ql[:, -1:], qr[:, -1:]], -1)
+    dec, dec_lse = oracle.mla_decode_unrounded(packed_q, torch.cat([c, kr], -1), torch.tensor([t, t]), scale)
+    assert (dec[:, 0] - out[:, -1]).abs().max() < 1e-5 and (dec_lse[:, :, 0] - lse[:, :, -1]).abs().max() < 1e-5
+
+
+def test_decode_constant_fill_closed_form():
+    """benchmarks/attention/benchmark_mla_decode.cu:42-48: q = 1/8, cache = 1/4,
+    scale = 1/24 -> score 0.75, O == 0.25, LSE = 0.75 + ln(context)."""
+    b, n, h = 2, 100, 4
+    q = torch.full((b, 1, h, 576), 0.125)
+    cache = torch.full((b, n, 576), 0.25)
+    lengths = torch.tensor([100, 37])
+    out, lse = oracle.mla_decode_unrounded(q, cache, lengths, 1.0 / 24.0)
+    assert torch.allclose(out, torch.full_like(out, 0.25), atol=1e-6)
+    expected = 0.75 + torch.log(lengths.float())
+    assert torch.allclose(lse[:, :, 0], expected[:, None].expand(b, h), atol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# page packing, workspace size
+# ---------------------------------------------------------------------------
+
+def test_pack_cache_closed_form():
+    kv = _rand((3, 130, 576), 100).bfloat16()
+    paged, table = oracle.pack_cache(kv, 64)
+    assert paged.shape == (9, 64, 1, 576) and table.dtype == torch.int32
+    assert torch.equal(table, torch.arange(9, dtype=torch.int32).reshape(3, 3))
+    for bi in range(3):
+        for token in (0, 63, 64, 129):
+            assert torch.equal(paged[table[bi, token // 64], token % 64, 0], kv[bi, token])
+        assert paged[table[bi, 2], 2:].abs().max() == 0  # padding is zero
+
+
+def test_workspace_elements():
+    assert oracle.decode_workspace_elements(2, 3, 8, 512) == 2 * 3 * 8 * 514
+    assert oracle.decode_workspace_elements(64, 128, 8, 512) == 64 * 128 * 8 * 514
