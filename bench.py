@@ -1,0 +1,140 @@
+"""Headline benchmark: one MI355X, synthetic DeepSeek-V3-shaped inputs.
+
+``python bench.py --gpus 1 --steps K --warmup W`` prints one JSON line.  A step
+is one MLA prefill forward over the S=4096, H=128, 192/192/128 workload with
+all inputs resident in HBM; ``value`` is its algorithmic TFLOP/s (causal pair
+count S^2/2).  The ``roofline`` object prices the forward kernel against the
+chip's dense bf16 MFMA peak from its own event-timed launches, ``extra`` holds
+the other workloads of the metric (backward TFLOP/s, decode GB/s, flash
+forward time), and ``cpu_baseline`` is the fp32 CPU oracle timed on this
+machine's host cores over a sample of heads of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def event_time_ms(function, steps, warmup):
+    """Average duration of `function` over `steps` launches, from events on torch's
+    current stream (the stream the kernels are enqueued on)."""
+    import torch
+    for _ in range(warmup):
+        function()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        function()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) * 1000.0
+    return start.elapsed_time(stop) / steps, wall / steps
+
+
+def cpu_baseline_forward(q, k, v, scale, gpu_out, gpu_lse, sample_heads):
+    """fp32 oracle on the host cores over `sample_heads` heads; also checks the
+    GPU result of the same heads.  Only this leg touches oracle/."""
+    import torch
+    from dscuda_amd.harness import configs
+    from oracle import attention_oracle as oracle
+
+    heads = list(range(0, q.shape[2], max(1, q.shape[2] // sample_heads)))[:sample_heads]
+    oracle.causal_attention_forward(q[:, :256], k[:, :256], v[:, :256], scale, heads=heads[:1])  # warm threads
+    begin = time.perf_counter()
+    expected, expected_lse = oracle.causal_attention_forward(q, k, v, scale, heads=heads)
+    seconds = time.perf_counter() - begin
+    flops = configs.forward_flops(q.shape[0], len(heads), q.shape[1], q.shape[3], v.shape[3])
+    worst, mean = oracle.error_stats(gpu_out[:, :, heads].float().cpu(), expected)
+    lse_err = (gpu_lse[:, heads].cpu() - expected_lse).abs().max().item()
+    baseline = {
+        "value": flops / seconds / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{len(heads)} of {q.shape[2]} heads of the same workload, unfused fp32 PyTorch oracle, "
+                  f"{seconds:.1f} s, os.cpu_count()={os.cpu_count()}, torch {torch.__version__}",
+    }
+    parity = {"heads_checked": len(heads), "o_max_abs": worst, "o_mean_abs": mean, "lse_max_abs": lse_err,
+              "ok": bool(worst <= 2e-2 and mean <= 2e-3 and lse_err <= 1e-3)}
+    return baseline, parity
+
+
+def main():
+    parser = argparse.ArgumentParser(description=__doc__)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--cpu-heads", type=int, default=32, help="heads in the CPU baseline sample")
+    parser.add_argument("--no-extra", action="store_true", help="skip the backward / decode / flash measurements")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards over heads "
+                 "without communication); run with --gpus 1")
+
+    import torch
+    from dscuda_amd.harness import configs, ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+
+    # ---- headline: MLA prefill forward, S=4096, H=128, 192/192/128, seed 1 + RoPE
+    batch, seq, heads, dqk, dv = 1, 4096, 128, 192, 128
+    q, k, v, scale = configs.mla_prefill_inputs(batch, seq, heads, seed=1)
+    dq, dk, dvv = q.to(device), k.to(device), v.to(device)
+    out = torch.empty(batch, seq, heads, dv, device=device, dtype=torch.bfloat16)
+    lse = torch.empty(batch, heads, seq, device=device, dtype=torch.float32)
+
+    def forward_step():
+        ops.mla_prefill_forward(dq, dk, dvv, scale, out, lse)
+
+    kernel_ms, wall_ms = event_time_ms(forward_step, args.steps, args.warmup)
+    flops = configs.forward_flops(batch, heads, seq, dqk, dv)
+    achieved = flops / kernel_ms / 1e9
+
+    extra = {}
+    if not args.no_extra:
+        from dscuda_amd.harness import extra_workloads
+        extra = extra_workloads.measure(device, event_time_ms, q, k, v, scale, out, lse)
+
+    baseline, parity = cpu_baseline_forward(q, k, v, scale, out, lse, args.cpu_heads)
+
+    line = {
+        "metric": "MLA fwd/bwd TFLOP/s (% bf16 MFMA peak); decode HBM GB/s, 1xMI355X",
+        "value": flops / wall_ms / 1e9,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "MLA prefill forward, B=1 S=4096 H=128, d_qk=128+64, d_v=128, causal, "
+                               "0.5*N(0,1) seed 1, RoPE theta=10000, scale 1/sqrt(192)"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "attention_forward_kernel<192,128,8>", "kernel_ms": kernel_ms,
+                     "flops_per_launch": flops},
+        "cpu_baseline": baseline,
+        "parity": parity,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
