@@ -1,6 +1,5 @@
 #include "attn_kernels.h"
 #include <stdexcept>
 namespace dscuda {
-void mla_absorbed_forward_dispatch(__hip_bfloat16*, float*, const __hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*, int, int, int, float, hipStream_t) { throw std::runtime_error("absorbed forward: not built yet"); }
 void mla_absorbed_backward_dispatch(__hip_bfloat16*, __hip_bfloat16*, __hip_bfloat16*, __hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*, const float*, const __hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*, int, int, int, float, hipStream_t) { throw std::runtime_error("absorbed backward: not built yet"); }
 }

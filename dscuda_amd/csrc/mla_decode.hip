@@ -1,5 +1,890 @@
+// Absorbed-weight MLA over a shared 512+64 latent KV stream for gfx950:
+// single-token decode from a paged cache (split-KV + merge) and the causal
+// absorbed prefill forward.  Takes the place of the reference's
+// mla_decode_split_kernel / mla_decode_combine_kernel
+// (kernels/attention/mla/sm89.cu:413-507) and mla_forward_kernel (:156-291);
+// the decomposition below is built around 64-lane MFMA waves and the 160 KB
+// LDS and shares nothing with their per-head scalar loops.
+//
+// Rows and tiles
+//   A workgroup (4 waves) owns 128 "rows" -- the heads of one sequence in
+//   decode, consecutive (token, head) pairs in prefill -- and walks the key
+//   stream in tiles of 64 tokens.  Every row of a workgroup reads the same
+//   keys, so a 72 KB tile is fetched from HBM once and feeds 128 rows x
+//   (576 + 512) x 2 flop per token: the only way the 242 flop/byte of the
+//   H = 128 decode stays on the HBM roofline.  Each wave owns 32 rows: the
+//   scores are produced transposed, S^T (64 keys x 32 rows) = K_tile Q^T with
+//   Q held in registers (36 k-steps), and O^T (512 x 32 rows) += V^T P^T is
+//   accumulated in 256 accumulator registers per lane.
+//
+// One LDS copy serves K and V
+//   V is the first 512 columns of the same rows.  The tile is stored once,
+//   row-major, and read two ways: 16-byte row reads for the K operand, and
+//   ds_read_b64_tr_b16 (a 4 keys x 16 columns block transposed across 16
+//   lanes) for the V^T operand.  Two stages of 72 KB double-buffer the stream.
+//
+// Global -> LDS without registers
+//   Tiles arrive by global_load_lds (16 bytes per lane, a wave instruction
+//   fills 1 KB of consecutive LDS).  With no padding possible inside that 1 KB
+//   the bank spread comes from a swizzle applied on the global side: the
+//   16-byte chunk c of row r lives at slot 72*r + (c ^ f(r)), f(r) = the three
+//   bits of r>>1 with bits 0 and 2 exchanged.  That makes both the 16-row
+//   column reads (K operand) and the 4-row x 64-byte block reads (V operand)
+//   conflict free, and every LDS address of the inner loops stays a per-lane
+//   base plus an immediate.
+//
+// Scheduling (decode)
+//   The tiles of all sequences form one list that is cut into equal ranges,
+//   one per workgroup (one workgroup per CU), so uneven lengths balance to
+//   within a tile.  A range may start or end inside a sequence; such a segment
+//   leaves (max, sum, unnormalised O) in the caller's workspace at slot
+//   workgroup + sequence -- unique because ranges and sequences both advance
+//   monotonically -- and a second kernel merges the slots of a sequence.
+//   Sequences that fall inside one range are finished in place.  Lengths live
+//   on the device; the cut is computed in-kernel from a block scan, so the
+//   call stays capturable.
 #include "attn_kernels.h"
+#include "hip_common.h"
+
+#include <algorithm>
 #include <stdexcept>
+#include <string>
+
 namespace dscuda {
-void mla_decode_dispatch(__hip_bfloat16*, float*, const __hip_bfloat16*, const __hip_bfloat16*, const int*, const int*, float*, int, int, int, int, int, float, hipStream_t) { throw std::runtime_error("decode: not built yet"); }
+namespace {
+
+constexpr int RANK = 512;
+constexpr int ROPE = 64;
+constexpr int WIDTH = RANK + ROPE;
+constexpr int BN = 64;                      // keys per tile
+constexpr int ROWS = 128;                   // rows per workgroup
+constexpr int THREADS = 256;
+constexpr int CHUNKS = WIDTH / 8;           // 72 16-byte chunks per key row
+constexpr int ROW_BYTES = CHUNKS * 16;      // 1152
+constexpr int STAGE_BYTES = BN * ROW_BYTES; // 73728
+constexpr int LOADS_PER_THREAD = BN * CHUNKS / THREADS;  // 18
+constexpr int KSTEPS = WIDTH / 16;          // 36
+constexpr int DBLOCKS = RANK / 32;          // 16
+constexpr int MAX_SEQUENCES = 3072;         // prefix table that fits beside the two stages
+constexpr int EPILOGUE_PITCH = 1024 + 16;   // bytes per staged output row
+
+typedef __attribute__((address_space(3))) void* lds_pointer;
+typedef const __attribute__((address_space(1))) void* global_pointer;
+
+__device__ __forceinline__ int swizzle_of_row(int row) {
+    const int u = row >> 1;
+    return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
 }
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
+// vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt/lgkmcnt unconstrained).
+template <int COUNT>
+__device__ __forceinline__ void wait_vector_memory() {
+    __builtin_amdgcn_s_waitcnt((COUNT & 15) | ((COUNT >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Workgroup barrier without the full memory fence of __syncthreads(): the fence
+// would wait for every outstanding vector-memory operation, i.e. for the next
+// tile's direct-to-LDS loads that are meant to stay in flight across the
+// barrier.  LDS traffic of this wave is drained; arrival of a tile is ordered
+// separately by wait_vector_memory before the barrier.
+__device__ __forceinline__ void workgroup_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__device__ __forceinline__ unsigned lds_offset_of(const void* pointer) {
+    return (unsigned)(uintptr_t)(lds_pointer)pointer;
+}
+
+// 16 bytes per lane from global memory straight into LDS at
+// lds_base + 16 * lane (lds_base wave-uniform).  Issued as asm so that the
+// compiler's wait-count bookkeeping does not see an LDS writer: it would
+// otherwise drain every outstanding load before each LDS read of the tile
+// being consumed, serialising the prefetch.  Arrival is ordered by hand with
+// wait_vector_memory + workgroup_barrier.
+__device__ __forceinline__ void direct_load_16(const void* source, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(source), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
+struct KeyStream {
+    const bf16_t* latent;      // token t at latent + t*latent_stride, 512 wide
+    const bf16_t* rope;        // token t at rope + t*rope_stride, 64 wide
+    size_t latent_stride;
+    size_t rope_stride;
+    const int* block_table;    // nullptr: tokens are stored contiguously
+    int page_size;
+};
+
+// Issue the direct-to-LDS loads of one 64-token tile.  Tokens past
+// `last_token` are clamped to it (their rows are zeroed afterwards), so no
+// byte outside the visible part of the sequence is ever read.
+__device__ __forceinline__ void issue_tile(unsigned char* stage_base, const KeyStream& keys, int key0, int last_token,
+                                           int wave, int lane) {
+    const bool paged = keys.block_table != nullptr;
+    const bool page_holds_tile = paged && (keys.page_size % BN == 0);
+    long long tile_physical = key0;
+    if (page_holds_tile) {
+        const int page = keys.block_table[key0 / keys.page_size];
+        tile_physical = (long long)page * keys.page_size + key0 % keys.page_size;
+    }
+    // Slot of load i is (4*i + wave)*64 + lane; it advances by 256 = 3*72 + 40
+    // per load, which keeps row / position an add and a compare instead of a
+    // division (and keeps 18 precomputed addresses out of the register file).
+    int row = (wave * 64 + lane) / CHUNKS;
+    int position = (wave * 64 + lane) % CHUNKS;
+    unsigned destination_offset = lds_offset_of(stage_base) + wave * 1024;
+#pragma unroll 1
+    for (int i = 0; i < LOADS_PER_THREAD; ++i) {
+        const int chunk = position ^ swizzle_of_row(row);
+        const int token = min(key0 + row, last_token);
+        long long physical;
+        if (!paged) {
+            physical = token;
+        } else if (page_holds_tile) {
+            physical = tile_physical + (token - key0);
+        } else {
+            const int page = keys.block_table[token / keys.page_size];
+            physical = (long long)page * keys.page_size + token % keys.page_size;
+        }
+        const bf16_t* source = chunk < RANK / 8 ? keys.latent + physical * keys.latent_stride + 8 * chunk
+                                                : keys.rope + physical * keys.rope_stride + 8 * (chunk - RANK / 8);
+        direct_load_16(source, destination_offset);
+        destination_offset += 4 * 1024;
+        row += 3;
+        position += 40;
+        if (position >= CHUNKS) {
+            position -= CHUNKS;
+            row += 1;
+        }
+    }
+}
+
+// Score-chain MFMAs with the accumulator held in ordinary vector registers.
+// The compiler's own MFMAs take accumulator-file destinations in a kernel this
+// large, and that file is fully occupied by the output accumulators.  Issued
+// as asm, the hazard bookkeeping is done here: the first MFMA starts from the
+// inline constant 0 (no producer to wait for), dependent MFMAs accumulating
+// into the very registers they read are interlocked by hardware, and
+// score_mfma_drain spends the wait states a vector-ALU reader of the result
+// needs after the last 8-pass MFMA before the value is handed back.
+__device__ __forceinline__ void score_mfma_first(f32x16& accumulator, const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(accumulator) : "v"(a), "v"(b));
+}
+
+__device__ __forceinline__ void score_mfma(f32x16& accumulator, const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(accumulator) : "v"(a), "v"(b));
+}
+
+__device__ __forceinline__ void score_mfma_drain(f32x16& accumulator) {
+    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(accumulator));
+}
+
+struct RowState {
+    f32x16 o[DBLOCKS];
+    float reference;  // point the exponentials are taken against, in log2 units (score * scale * log2 e)
+    float row_sum;    // this lane's share of the normaliser
+};
+
+// Head room (log2 units) put between the first tile's maximum and the fixed
+// reference of the fast path, and the excess over the reference at which the
+// fast path gives up (2^80 per term leaves 2^47 of fp32 range for the sums).
+constexpr float FAST_HEADROOM = 40.0f;
+constexpr float FAST_LIMIT = 80.0f;
+
+// One tile for one wave: S^T = K Q^T, softmax against `limit` visible keys for
+// this lane's row, O^T += V^T P^T.
+//
+// SAFE == false (the path that normally runs): the reference is fixed once,
+// FAST_HEADROOM above the row maximum of the first tile, so the 256 output
+// accumulators are never rescaled and nothing conditional touches them (a
+// conditional rescale makes the compiler copy the whole accumulator file at
+// the join).  Scores may exceed the reference by up to FAST_LIMIT before a
+// term gets near the top of the fp32 range; `risk` reports a row that came
+// closer than that, in which case the caller discards the result and repeats
+// the walk with SAFE == true.
+// SAFE == true: textbook online softmax, the reference follows the running
+// maximum and the accumulators are rescaled on every half tile.
+template <bool SAFE>
+__device__ __forceinline__ void process_tile(RowState& state, bool& risk, const bf16x8 (&qf)[KSTEPS],
+                                             const unsigned char* stage, int key0, int limit, int wave_min_limit,
+                                             bool first, float c, int lane_id) {
+    // The per-lane LDS offsets below are recomputed for every tile from an
+    // lane id read afresh (volatile, so nothing derived from it is hoisted): kept
+    // live across the loop they would be the registers that no longer fit and
+    // get spilled, and a scratch reload inside the loop stalls on the tile
+    // prefetch.
+    (void)lane_id;
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    const int lq = lane % 32;
+    const int g = lane / 32;
+
+    // K operand: row 32*mb + lq, 16-byte chunk 2*ks + g.  (2*ks+g) ^ f only mixes
+    // the low three bits, i.e. stays inside the 128-byte group ks/4.
+    const int swz = swizzle_of_row(lq);  // rows lq and lq+32 share f (f ignores bits >= 4 of the row)
+    const unsigned char* k_row = stage + lq * ROW_BYTES;
+    const unsigned char* k_lane[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) k_lane[j] = k_row + ((2 * j + g) ^ swz) * 16;
+
+    // V^T operand through transposing reads.  In a block of 16 lanes, lane s
+    // points at row 4*g + s/4 (+8 for the second read), columns 4*(s%4)..+3 of
+    // the 16-column group 16*(block%2); the instruction hands lane i column i
+    // of the four rows.  Together: MFMA row l%32, keys {4g..4g+3, 8+4g..8+4g+3}
+    // of each 16-key step, the k-order P^T carries from the C layout.
+    const int s16 = lane % 16;
+    const int block = lane / 16;
+    const int row1 = 4 * g + s16 / 4;
+    const int f1 = swizzle_of_row(row1);
+    const int chunk_low = (2 * (block % 2) + (s16 % 4) / 2) ^ (f1 & 3);
+    // Bit 2 of f (= bit 1 of the row) moves a row's data by one 64-byte column
+    // block: rows 2,3 (mod 4) keep column block d at position block d ^ 1.  The
+    // lanes addressing those rows therefore read 64 bytes further (even d) or
+    // nearer (odd d), which two base pointers per read turn back into immediates.
+    const int flip = 64 * ((row1 >> 1) & 1);
+    const unsigned char* v_lane1 = stage + row1 * ROW_BYTES + chunk_low * 16 + 8 * (s16 & 1);
+    const unsigned char* v_lane2 = stage + (row1 + 8) * ROW_BYTES + (chunk_low ^ 1) * 16 + 8 * (s16 & 1);
+    const unsigned char* v_base1[2] = {v_lane1 + flip, v_lane1 - flip};
+    const unsigned char* v_base2[2] = {v_lane2 + flip, v_lane2 - flip};
+
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4* tr_pointer;
+
+    // The tile is consumed in two halves of 32 keys so that only 16 score and 8
+    // probability registers are live beside the 256 accumulators and 144 Q
+    // registers.  Operand reads are software-pipelined by hand in groups of four
+    // MFMAs (the scheduler barrier keeps the compiler from hoisting a whole
+    // half's reads, which would push Q out to scratch).
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        // The 256 output accumulators fill the accumulator register file exactly,
+        // and a compiler-issued MFMA would want 16 more of them for the scores.
+        // The score chain is therefore issued by hand with its accumulator in
+        // ordinary registers (score_mfma_*).
+        f32x16 s_acc;
+        {
+            constexpr int GROUPS = KSTEPS / 4;
+            bf16x8 current[4], next[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                current[j] = *reinterpret_cast<const bf16x8*>(k_lane[j] + mb * 32 * ROW_BYTES);
+            }
+#pragma unroll
+            for (int group = 0; group < GROUPS; ++group) {
+                if (group + 1 < GROUPS) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        next[j] = *reinterpret_cast<const bf16x8*>(k_lane[j] + mb * 32 * ROW_BYTES + (group + 1) * 128);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (group == 0 && j == 0) {
+                        score_mfma_first(s_acc, current[j], qf[0]);
+                    } else {
+                        score_mfma(s_acc, current[j], qf[4 * group + j]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) current[j] = next[j];
+            }
+            score_mfma_drain(s_acc);
+        }
+
+        if (key0 + 32 * mb + 32 > wave_min_limit) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int k = key0 + 32 * mb + 8 * (i / 4) + 4 * g + (i % 4);
+                if (k >= limit) s_acc[i] = -INFINITY;
+            }
+        }
+
+        float tile_max = s_acc[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) tile_max = fmaxf(tile_max, s_acc[i]);
+        tile_max = half_wave_max(tile_max) * c;  // log2 units from here on
+
+        if (SAFE) {
+            const float new_reference = fmaxf(state.reference, tile_max);
+            const float alpha = __builtin_amdgcn_exp2f(state.reference - new_reference);
+            state.reference = new_reference;
+            state.row_sum *= alpha;
+#pragma unroll
+            for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) state.o[d][i] *= alpha;
+                __builtin_amdgcn_sched_barrier(0);  // one block at a time through the ordinary registers
+            }
+        } else {
+            if (first && mb == 0) state.reference = tile_max + FAST_HEADROOM;
+            risk = risk || (tile_max - state.reference > FAST_LIMIT);
+        }
+
+        const float offset = state.reference;
+        bf16x8 pf[2];
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            u32x4 packed;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 8 * n + 2 * j;
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -offset));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[i + 1], c, -offset));
+                state.row_sum += p0 + p1;
+                packed[j] = pack_bf16(p0, p1);
+            }
+            pf[n] = __builtin_bit_cast(bf16x8, packed);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        {
+            // 32 MFMAs (2 key steps x 16 column blocks) in 16 groups of two column blocks
+            constexpr int WIDTH_G = 2;
+            constexpr int GROUPS = 2 * DBLOCKS / WIDTH_G;
+            s16x4 cur_lo[WIDTH_G], cur_hi[WIDTH_G], next_lo[WIDTH_G], next_hi[WIDTH_G];
+            auto step_of = [&](int group, int j) {
+                const int n = group / (DBLOCKS / WIDTH_G);
+                const int d = WIDTH_G * (group % (DBLOCKS / WIDTH_G)) + j;
+                return (2 * mb + n) * 16 * ROW_BYTES + d * 64;
+            };
+#pragma unroll
+            for (int j = 0; j < WIDTH_G; ++j) {
+                cur_lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base1[j % 2] + step_of(0, j)));
+                cur_hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base2[j % 2] + step_of(0, j)));
+            }
+#pragma unroll
+            for (int group = 0; group < GROUPS; ++group) {
+                if (group + 1 < GROUPS) {
+#pragma unroll
+                    for (int j = 0; j < WIDTH_G; ++j) {
+                        next_lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base1[j % 2] + step_of(group + 1, j)));
+                        next_hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base2[j % 2] + step_of(group + 1, j)));
+                    }
+                }
+                const int n = group / (DBLOCKS / WIDTH_G);
+#pragma unroll
+                for (int j = 0; j < WIDTH_G; ++j) {
+                    const int d = WIDTH_G * (group % (DBLOCKS / WIDTH_G)) + j;
+                    const s16x8 both = __builtin_shufflevector(cur_lo[j], cur_hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
+                    state.o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n], state.o[d], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < WIDTH_G; ++j) {
+                    cur_lo[j] = next_lo[j];
+                    cur_hi[j] = next_hi[j];
+                }
+            }
+        }
+    }
+}
+
+// Column of the output a lane's accumulator register stands for.
+__device__ __forceinline__ constexpr int output_column(int d, int i4, int g) {
+    return 32 * d + 8 * i4 + 4 * g;
+}
+
+// Normalised bf16 rows -> out_row(row) .. +512, staged through this wave's LDS
+// region so that each store instruction writes one full 1 KB row.
+template <typename RowPointer>
+__device__ __forceinline__ void store_final(const RowState& state, float inverse, unsigned char* wave_lds, int lane,
+                                            RowPointer out_row) {
+    const int lq = lane % 32;
+    const int g = lane / 32;
+#pragma unroll
+    for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            u32x2 packed;
+            packed.x = pack_bf16(state.o[d][4 * i4 + 0] * inverse, state.o[d][4 * i4 + 1] * inverse);
+            packed.y = pack_bf16(state.o[d][4 * i4 + 2] * inverse, state.o[d][4 * i4 + 3] * inverse);
+            *reinterpret_cast<u32x2*>(wave_lds + lq * EPILOGUE_PITCH + 2 * output_column(d, i4, g)) = packed;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+    for (int row = 0; row < 32; ++row) {
+        bf16_t* destination = out_row(row);
+        if (destination != nullptr) {
+            const u32x4 bits = *reinterpret_cast<const u32x4*>(wave_lds + row * EPILOGUE_PITCH + 16 * lane);
+            *reinterpret_cast<u32x4*>(destination + 8 * lane) = bits;
+        }
+    }
+}
+
+// Unnormalised fp32 rows -> partial_row(row) .. +512 floats, in two halves of 256 columns.
+template <typename RowPointer>
+__device__ __forceinline__ void store_partial(const RowState& state, unsigned char* wave_lds, int lane,
+                                              RowPointer partial_row) {
+    const int lq = lane % 32;
+    const int g = lane / 32;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int dd = 0; dd < DBLOCKS / 2; ++dd) {
+            const int d = half * (DBLOCKS / 2) + dd;
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const f32x4 values = {state.o[d][4 * i4 + 0], state.o[d][4 * i4 + 1], state.o[d][4 * i4 + 2],
+                                      state.o[d][4 * i4 + 3]};
+                const int column = output_column(d, i4, g) - 256 * half;
+                *reinterpret_cast<f32x4*>(wave_lds + lq * EPILOGUE_PITCH + 4 * column) = values;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+        for (int row = 0; row < 32; ++row) {
+            float* destination = partial_row(row);
+            if (destination != nullptr) {
+                const f32x4 values = *reinterpret_cast<const f32x4*>(wave_lds + row * EPILOGUE_PITCH + 16 * lane);
+                *reinterpret_cast<f32x4*>(destination + 256 * half + 4 * lane) = values;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// Zero the rows of a landed tile that lie past the end of the sequence, so that
+// stale cache contents (possibly NaN) cannot reach the V operand.
+__device__ __forceinline__ void zero_tail_rows(unsigned char* stage, int first_invalid_row, int tid) {
+    const int chunks = (BN - first_invalid_row) * CHUNKS;
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int index = tid; index < chunks; index += THREADS) {
+        *reinterpret_cast<u32x4*>(stage + first_invalid_row * ROW_BYTES + index * 16) = zero;
+    }
+}
+
+__device__ __forceinline__ void load_query(bf16x8 (&qf)[KSTEPS], const bf16_t* latent_row, const bf16_t* rope_row,
+                                           bool valid, int g) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        u32x4 bits = {0, 0, 0, 0};
+        if (valid) {
+            const bf16_t* source = ks < RANK / 16 ? latent_row + 16 * ks + 8 * g : rope_row + 16 * (ks - RANK / 16) + 8 * g;
+            bits = *reinterpret_cast<const u32x4*>(source);
+        }
+        qf[ks] = __builtin_bit_cast(bf16x8, bits);
+    }
+}
+
+__device__ __forceinline__ void reset(RowState& state) {
+#pragma unroll
+    for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) state.o[d][i] = 0.f;
+    }
+    state.reference = -INFINITY;
+    state.row_sum = 0.f;
+}
+
+// Walk tiles [tile_begin, tile_end) of one key stream for the 128 rows of this
+// workgroup, starting from cleared accumulators.  `limit` is this lane's row's
+// number of visible keys; every row must see at least one key of the first
+// tile.  Every wave processes every tile (rows that see nothing of a tile
+// simply get zero probabilities), so the accumulators never pass through a
+// conditional.  Returns this wave's overflow-risk flag (always false for SAFE).
+template <bool SAFE>
+__device__ __forceinline__ bool walk_tiles(RowState& state, const bf16x8 (&qf)[KSTEPS], unsigned char* lds,
+                                           const KeyStream& keys, int tile_begin, int tile_end, int tokens, int limit,
+                                           float c, int tid) {
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int lane = tid % 64;
+    int wave_min_limit = limit;  // wave-uniform: below it no masking is needed
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, offset));
+    }
+    wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
+    reset(state);
+    bool risk = false;
+    const int last_token = tokens - 1;
+    // Drain the query loads here: a wait for them inside the loop would also
+    // wait for the tile prefetch that is kept in flight there.
+    wait_vector_memory<0>();
+    issue_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, last_token, wave, lane);
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        unsigned char* stage = lds + (tile & 1) * STAGE_BYTES;
+        if (tile + 1 < tile_end) {
+            issue_tile(lds + ((tile + 1) & 1) * STAGE_BYTES, keys, (tile + 1) * BN, last_token, wave, lane);
+            wait_vector_memory<LOADS_PER_THREAD>();
+        } else {
+            wait_vector_memory<0>();
+        }
+        workgroup_barrier();
+        const int key0 = tile * BN;
+        if (key0 + BN > tokens) {
+            zero_tail_rows(stage, tokens - key0, tid);
+            workgroup_barrier();
+        }
+        process_tile<SAFE>(state, risk, qf, stage, key0, limit, wave_min_limit, tile == tile_begin, c, lane);
+        workgroup_barrier();
+    }
+    return risk;
+}
+
+// Fast walk first; the rare workgroup in which some row outran the fixed
+// reference repeats the walk with the rescaling variant.  Each variant loads
+// its own copy of the query fragments so that the register allocation of the
+// fast loop does not have to carry them across the slow one.
+__device__ __forceinline__ void walk_tiles_checked(RowState& state, const bf16_t* query_latent_row,
+                                                   const bf16_t* query_rope_row, bool valid, unsigned char* lds,
+                                                   const KeyStream& keys, int tile_begin, int tile_end, int tokens,
+                                                   int limit, float c, int tid) {
+    const int g = (tid % 64) / 32;
+    bool risk;
+    {
+        bf16x8 qf[KSTEPS];
+        load_query(qf, query_latent_row, query_rope_row, valid, g);
+        risk = walk_tiles<false>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
+    }
+    if (__syncthreads_or(risk)) {
+        bf16x8 qf[KSTEPS];
+        load_query(qf, query_latent_row, query_rope_row, valid, g);
+        walk_tiles<true>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
+    }
+}
+
+__device__ __forceinline__ int tiles_of(int length) {
+    return (max(length, 0) + BN - 1) / BN;
+}
+
+// Inclusive prefix of tiles per sequence into prefix[0..B]; returns the total.
+__device__ __forceinline__ int scan_tiles(int* prefix, int* scratch, const int* lengths, int batch_size, int tid) {
+    const int lane = tid % 64;
+    const int wave = tid / 64;
+    int carry = 0;
+    if (tid == 0) prefix[0] = 0;
+    for (int base = 0; base < batch_size; base += THREADS) {
+        const int index = base + tid;
+        int value = index < batch_size ? tiles_of(lengths[index]) : 0;
+#pragma unroll
+        for (int offset = 1; offset < 64; offset <<= 1) {
+            const int other = __shfl_up(value, offset);
+            if (lane >= offset) value += other;
+        }
+        if (lane == 63) scratch[wave] = value;
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; ++w) {
+            const int t = scratch[w];
+            if (w < wave) before += t;
+            total += t;
+        }
+        if (index < batch_size) prefix[index + 1] = carry + before + value;
+        carry += total;
+        __syncthreads();
+    }
+    return carry;
+}
+
+// ----------------------------------------------------------------------------
+// decode
+// ----------------------------------------------------------------------------
+
+struct DecodeSlots {
+    float* partial_output;   // [slots][H][512]
+    float* partial_stats;    // [slots][H][2]  (max in log2 units, sum)
+};
+
+__global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
+    bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query,
+    const bf16_t* __restrict__ paged_kv_cache, const int* __restrict__ block_table,
+    const int* __restrict__ cache_lengths, float* __restrict__ workspace, int batch_size, int heads, int page_size,
+    int pages_per_sequence, int workgroups, int whole_sequences, float scale) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    int* prefix = reinterpret_cast<int*>(lds + 2 * STAGE_BYTES);
+    int* scratch = prefix + MAX_SEQUENCES + 1;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64;
+    const int wave = tid / 64;
+    const int lq = lane % 32;
+    const int g = lane / 32;
+    const int workgroup = blockIdx.x;
+    const int head0 = blockIdx.y * ROWS;
+    const float c = scale * LOG2E;
+
+    const int total = scan_tiles(prefix, scratch, cache_lengths, batch_size, tid);
+    int range_begin, range_end, sequence;
+    if (whole_sequences) {
+        sequence = workgroup;
+        range_begin = prefix[sequence];
+        range_end = prefix[sequence + 1];
+    } else {
+        const int per = (total + workgroups - 1) / workgroups;
+        range_begin = min(workgroup * per, total);
+        range_end = min(range_begin + per, total);
+        // first sequence whose tiles reach past range_begin
+        int low = 0, high = batch_size;
+        while (low < high) {
+            const int mid = (low + high) / 2;
+            if (prefix[mid + 1] <= range_begin) low = mid + 1; else high = mid;
+        }
+        sequence = low;
+    }
+    if (range_begin >= range_end) return;
+
+    const size_t slots = (size_t)workgroups + batch_size;
+    float* partial_output = workspace;
+    float* partial_stats = workspace + slots * heads * RANK;
+
+    const int head = head0 + 32 * wave + lq;
+    const bool valid = head < heads;
+    const bool wave_active = head0 + 32 * wave < heads;
+    unsigned char* wave_lds = lds + wave * 32 * EPILOGUE_PITCH;
+
+    RowState state;
+    int position = range_begin;
+    while (position < range_end) {
+        const int sequence_begin = prefix[sequence];
+        const int sequence_end = prefix[sequence + 1];
+        const int segment_end = min(range_end, sequence_end);
+        const int tokens = cache_lengths[sequence];
+        const bool whole = position == sequence_begin && segment_end == sequence_end;
+        if (segment_end <= position) {  // a sequence without tiles (length < 1) owns nothing
+            ++sequence;
+            continue;
+        }
+
+        const bf16_t* query_row = query + ((size_t)sequence * heads + (valid ? head : 0)) * WIDTH;
+
+        KeyStream keys;
+        keys.latent = paged_kv_cache;
+        keys.rope = paged_kv_cache + RANK;
+        keys.latent_stride = WIDTH;
+        keys.rope_stride = WIDTH;
+        keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
+        keys.page_size = page_size;
+        walk_tiles_checked(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
+                           segment_end - sequence_begin, tokens, tokens, c, tid);
+
+        const float total_sum = half_wave_sum(state.row_sum);
+        if (wave_active) {
+            if (whole) {
+                const float inverse = 1.0f / total_sum;
+                if (valid && g == 0) {
+                    logsumexp[(size_t)sequence * heads + head] = (state.reference + __builtin_amdgcn_logf(total_sum)) * LN2;
+                }
+                store_final(state, inverse, wave_lds, lane, [&](int row) -> bf16_t* {
+                    const int h = head0 + 32 * wave + row;
+                    return h < heads ? output + ((size_t)sequence * heads + h) * RANK : nullptr;
+                });
+            } else {
+                const size_t slot = (size_t)workgroup + sequence;
+                if (valid && g == 0) {
+                    float* stats = partial_stats + (slot * heads + head) * 2;
+                    stats[0] = state.reference;
+                    stats[1] = total_sum;
+                }
+                store_partial(state, wave_lds, lane, [&](int row) -> float* {
+                    const int h = head0 + 32 * wave + row;
+                    return h < heads ? partial_output + (slot * heads + h) * RANK : nullptr;
+                });
+            }
+        }
+        __syncthreads();  // the staging region is about to be overwritten by the next segment's tiles
+        position = segment_end;
+        ++sequence;
+    }
+}
+
+// Merge the partial results of every sequence that was cut by a range boundary.
+__global__ __launch_bounds__(128) void mla_decode_combine_kernel(
+    bf16_t* __restrict__ output, float* __restrict__ logsumexp, const int* __restrict__ cache_lengths,
+    const float* __restrict__ workspace, int batch_size, int heads, int workgroups) {
+    __shared__ int sums[2][2];
+    const int tid = threadIdx.x;
+    const int sequence = blockIdx.y;
+    const int head = blockIdx.x;
+
+    // tiles before this sequence and in total
+    int before = 0, total = 0;
+    for (int index = tid; index < batch_size; index += 128) {
+        const int t = tiles_of(cache_lengths[index]);
+        total += t;
+        if (index < sequence) before += t;
+    }
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        before += __shfl_xor(before, offset);
+        total += __shfl_xor(total, offset);
+    }
+    if (tid % 64 == 0) {
+        sums[tid / 64][0] = before;
+        sums[tid / 64][1] = total;
+    }
+    __syncthreads();
+    before = sums[0][0] + sums[1][0];
+    total = sums[0][1] + sums[1][1];
+    const int own = tiles_of(cache_lengths[sequence]);
+    if (own == 0) return;
+    const int per = (total + workgroups - 1) / workgroups;
+    const int first = before / per;
+    const int last = (before + own - 1) / per;
+    if (first == last) return;  // finished in place by the split kernel
+
+    const size_t slots = (size_t)workgroups + batch_size;
+    const float* partial_output = workspace;
+    const float* partial_stats = workspace + slots * heads * RANK;
+
+    float reference = -INFINITY;
+    for (int w = first; w <= last; ++w) {
+        reference = fmaxf(reference, partial_stats[(((size_t)w + sequence) * heads + head) * 2]);
+    }
+    float normaliser = 0.f;
+    f32x4 accumulator = {0.f, 0.f, 0.f, 0.f};
+    for (int w = first; w <= last; ++w) {
+        const size_t row = ((size_t)w + sequence) * heads + head;
+        const float weight = __builtin_amdgcn_exp2f(partial_stats[row * 2] - reference);
+        normaliser += weight * partial_stats[row * 2 + 1];
+        const f32x4 values = *reinterpret_cast<const f32x4*>(partial_output + row * RANK + 4 * tid);
+        accumulator += values * weight;
+    }
+    const float inverse = 1.0f / normaliser;
+    u32x2 packed;
+    packed.x = pack_bf16(accumulator[0] * inverse, accumulator[1] * inverse);
+    packed.y = pack_bf16(accumulator[2] * inverse, accumulator[3] * inverse);
+    const size_t out_row = (size_t)sequence * heads + head;
+    *reinterpret_cast<u32x2*>(output + out_row * RANK + 4 * tid) = packed;
+    if (tid == 0) {
+        logsumexp[out_row] = (reference + __builtin_amdgcn_logf(normaliser)) * LN2;
+    }
+}
+
+// ----------------------------------------------------------------------------
+// absorbed causal prefill forward
+// ----------------------------------------------------------------------------
+
+__global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
+    bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent,
+    const bf16_t* __restrict__ query_rope, const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope,
+    int sequence_length, int heads, int row_blocks, float scale) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid % 64;
+    const int wave = tid / 64;
+    const int lq = lane % 32;
+    const int g = lane / 32;
+    const float c = scale * LOG2E;
+
+    // heaviest (latest) row blocks first
+    const int batch = blockIdx.x / row_blocks;
+    const int row_block = row_blocks - 1 - blockIdx.x % row_blocks;
+    const long long rows = (long long)sequence_length * heads;   // (token, head) pairs of one batch element
+    const long long row0 = (long long)row_block * ROWS;
+    const long long row = row0 + 32 * wave + lq;
+    const bool valid = row < rows;
+    const bool wave_active = row0 + 32 * wave < rows;
+    const int token = valid ? (int)(row / heads) : 0;
+    const int head = valid ? (int)(row % heads) : 0;
+    const long long global_row = (long long)batch * rows + (valid ? row : 0);
+
+    RowState state;
+
+    const long long last_row = min(rows, row0 + ROWS) - 1;
+    const int visible = (int)(last_row / heads) + 1;  // keys any row of this block may see
+    KeyStream keys;
+    keys.latent = kv_latent + (size_t)batch * sequence_length * RANK;
+    keys.rope = key_rope + (size_t)batch * sequence_length * ROPE;
+    keys.latent_stride = RANK;
+    keys.rope_stride = ROPE;
+    keys.block_table = nullptr;
+    keys.page_size = 0;
+    walk_tiles_checked(state, query_latent + global_row * RANK, query_rope + global_row * ROPE, valid, lds, keys, 0,
+                       tiles_of(visible), visible, token + 1, c, tid);
+
+    if (!wave_active) return;
+    const float total_sum = half_wave_sum(state.row_sum);
+    if (valid && g == 0) {
+        logsumexp[((size_t)batch * heads + head) * sequence_length + token] =
+            (state.reference + __builtin_amdgcn_logf(total_sum)) * LN2;
+    }
+    unsigned char* wave_lds = lds + wave * 32 * EPILOGUE_PITCH;
+    store_final(state, 1.0f / total_sum, wave_lds, lane, [&](int r) -> bf16_t* {
+        const long long rr = row0 + 32 * wave + r;
+        return rr < rows ? output + ((long long)batch * rows + rr) * RANK : nullptr;
+    });
+}
+
+constexpr int LDS_BYTES = 2 * STAGE_BYTES + (MAX_SEQUENCES + 1 + 8) * 4;
+
+template <typename Kernel>
+void allow_large_lds(Kernel kernel) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  LDS_BYTES));
+}
+
+int compute_units() {
+    static thread_local int cached = 0;
+    if (cached == 0) {
+        int device = 0;
+        HIP_CHECK(hipGetDevice(&device));
+        HIP_CHECK(hipDeviceGetAttribute(&cached, hipDeviceAttributeMultiprocessorCount, device));
+    }
+    return cached;
+}
+
+}  // namespace
+
+void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, const bf16_t* paged_kv_cache,
+                         const int* block_table, const int* cache_lengths, float* workspace, int batch_size,
+                         int heads, int page_size, int pages_per_sequence, int splits, float scale,
+                         hipStream_t stream) {
+    if (batch_size > MAX_SEQUENCES) {
+        throw std::invalid_argument("MLA decode supports at most " + std::to_string(MAX_SEQUENCES) +
+                                    " sequences per call");
+    }
+    static thread_local bool prepared = false;
+    if (!prepared) {
+        allow_large_lds(mla_decode_split_kernel);
+        prepared = true;
+    }
+    // Slots workgroups + batch must fit the B*H*splits*(C+2) workspace: with
+    // splits == 1 every sequence is finished by one workgroup and no slot is used.
+    const int whole_sequences = splits == 1 ? 1 : 0;
+    int workgroups = batch_size;
+    if (!whole_sequences) {
+        const long long by_workspace = (long long)batch_size * (splits - 1);
+        workgroups = (int)std::min<long long>(compute_units(), by_workspace);
+    }
+    const int head_groups = (heads + ROWS - 1) / ROWS;
+    hipLaunchKernelGGL(mla_decode_split_kernel, dim3(workgroups, head_groups), dim3(THREADS), LDS_BYTES, stream,
+                       output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
+                       heads, page_size, pages_per_sequence, workgroups, whole_sequences, scale);
+    HIP_CHECK(hipGetLastError());
+    if (!whole_sequences) {
+        hipLaunchKernelGGL(mla_decode_combine_kernel, dim3(heads, batch_size), dim3(128), 0, stream, output,
+                           logsumexp, cache_lengths, workspace, batch_size, heads, workgroups);
+        HIP_CHECK(hipGetLastError());
+    }
+}
+
+void mla_absorbed_forward_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query_latent,
+                                   const bf16_t* query_rope, const bf16_t* kv_latent, const bf16_t* key_rope,
+                                   int batch_size, int sequence_length, int heads, float scale, hipStream_t stream) {
+    static thread_local bool prepared = false;
+    if (!prepared) {
+        allow_large_lds(mla_absorbed_forward_kernel);
+        prepared = true;
+    }
+    const long long rows = (long long)sequence_length * heads;
+    const long long row_blocks = (rows + ROWS - 1) / ROWS;
+    if (row_blocks * batch_size > 0x7fffffffLL) {
+        throw std::invalid_argument("MLA forward: batch*tokens*heads exceeds the grid limit");
+    }
+    hipLaunchKernelGGL(mla_absorbed_forward_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS), LDS_BYTES,
+                       stream, output, logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length, heads,
+                       (int)row_blocks, scale);
+    HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace dscuda

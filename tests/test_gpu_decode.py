@@ -1,0 +1,146 @@
+"""GPU parity of the absorbed MLA decode (paged latent cache, split-KV) and of
+the absorbed causal prefill forward against the fp32 oracle, through the C-ABI."""
+
+import pytest
+import torch
+
+from dscuda_amd.harness import configs, ops
+from oracle import attention_oracle as oracle
+from tests.parity import announce, assert_close_bf16, assert_close_lse
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_case(cuda, batch, tokens, heads, lengths, splits=8, page_size=64, seed=2026, factor=0.25,
+                 permute_pages=False, scale=None):
+    g = torch.Generator().manual_seed(seed)
+    query = (torch.randn(batch, 1, heads, 576, generator=g) * factor).bfloat16()
+    cache = (torch.randn(batch, tokens, 576, generator=g) * factor).bfloat16()
+    scale = configs.c_float(576 ** -0.5) if scale is None else scale
+    paged, table = configs.pack_cache(cache, page_size)
+    if permute_pages:
+        order = torch.randperm(paged.shape[0], generator=g)
+        inverse = torch.empty_like(order)
+        inverse[order] = torch.arange(order.numel())
+        paged = paged[order].contiguous()      # new block i holds old block order[i]
+        table = inverse[table.long()].to(torch.int32)
+    lengths_t = torch.tensor(lengths, dtype=torch.int32)
+    announce("mla_decode", dict(B=batch, KV=tokens, H=heads, lengths=lengths, splits=splits, page=page_size,
+                                permuted=permute_pages))
+    out, lse = ops.mla_decode(query.to(cuda), paged.to(cuda), table.to(cuda), lengths_t.to(cuda), scale,
+                              splits=splits)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths_t, scale)
+    assert_close_bf16("O", out, expected)
+    assert_close_lse("LSE", lse, expected_lse)
+    return out, lse
+
+
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_DECODE)
+def test_decode_reference_test_shapes(cuda, batch, tokens, heads):
+    # benchmarks/mla.py:36-39 with the test-mode lengths (1, ..., T) of :58-61
+    _decode_case(cuda, batch, tokens, heads, configs.harness_decode_lengths(batch, tokens, test=True))
+
+
+@pytest.mark.parametrize("batch,tokens,heads", [(2, 1024, 16), (1, 256, 16), (4, 4096, 32), (4, 4096, 128)])
+def test_decode_reference_benchmark_shapes(cuda, batch, tokens, heads):
+    _decode_case(cuda, batch, tokens, heads, configs.harness_decode_lengths(batch, tokens, test=False))
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 8, 32])
+def test_decode_is_split_invariant(cuda, splits):
+    _decode_case(cuda, 5, 700, 128, [1, 63, 64, 65, 700], splits=splits, seed=7)
+
+
+def test_decode_permuted_block_table(cuda):
+    _decode_case(cuda, 3, 333, 64, [333, 17, 200], permute_pages=True, seed=8)
+
+
+@pytest.mark.parametrize("page_size", [16, 48, 128])
+def test_decode_other_page_sizes(cuda, page_size):
+    _decode_case(cuda, 3, 300, 32, [300, 1, 129], page_size=page_size, seed=9)
+
+
+def test_decode_many_heads(cuda):
+    _decode_case(cuda, 2, 200, 160, [200, 77], seed=10)
+
+
+def test_decode_large_scores_take_the_rescaling_path(cuda):
+    """Scores that outgrow the first tile's maximum by far more than the fast
+    path's head room: late keys are aligned with the query, early ones are not."""
+    batch, tokens, heads = 2, 300, 8
+    g = torch.Generator().manual_seed(12)
+    query = (torch.randn(batch, 1, heads, 576, generator=g)).bfloat16()
+    cache = (torch.randn(batch, tokens, 576, generator=g) * 0.05).bfloat16()
+    cache[:, 200:260] = (query[:, 0, :1].float() * 4.0).bfloat16()  # huge positive scores late in the stream
+    lengths = torch.tensor([300, 250], dtype=torch.int32)
+    paged, table = configs.pack_cache(cache, 64)
+    scale = 1.0
+    announce("mla_decode rescaling path")
+    out, lse = ops.mla_decode(query.to(cuda), paged.to(cuda), table.to(cuda), lengths.to(cuda), scale, splits=1)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths, scale)
+    assert expected_lse.max() > 500  # really is far outside the fast path's range
+    assert_close_bf16("O", out, expected, max_abs=6e-2, mean_abs=6e-3)  # values are O(4): bf16 spacing 3e-2
+    worst = ((lse.cpu() - expected_lse).abs() / expected_lse.abs().clamp_min(1)).max().item()
+    assert worst <= 1e-5
+
+
+def test_decode_closed_form_constant_fill(cuda):
+    """benchmarks/attention/benchmark_mla_decode.cu:42-48: O == 0.25, LSE = 0.75 + ln(context)."""
+    batch, context, heads = 2, 1024, 16
+    query = torch.full((batch, 1, heads, 576), 0.125).bfloat16()
+    cache = torch.full((batch, context, 576), 0.25).bfloat16()
+    paged, table = configs.pack_cache(cache, 64)
+    lengths = torch.full((batch,), context, dtype=torch.int32)
+    out, lse = ops.mla_decode(query.to(cuda), paged.to(cuda), table.to(cuda), lengths.to(cuda), 1.0 / 24.0)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().float(), torch.full((batch, 1, heads, 512), 0.25))
+    assert (lse.cpu() - (0.75 + torch.log(torch.tensor(float(context))))).abs().max() <= 1e-4
+
+
+def test_decode_workload_4(cuda):
+    """B=64, H=128, lengths ~ U[1024, 8192] from seed 3: oracle on a sample of
+    sequences (shortest, longest, first), every output checked for finiteness."""
+    data = configs.mla_decode_inputs()
+    lengths = data["lengths"]
+    announce("mla_decode workload 4", dict(total_tokens=int(lengths.sum())))
+    out, lse = ops.mla_decode(data["query"].to(cuda), data["paged"].to(cuda), data["table"].to(cuda),
+                              lengths.to(cuda), data["scale"], splits=8)
+    torch.cuda.synchronize()
+    out, lse = out.cpu(), lse.cpu()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    sample = sorted({0, int(lengths.argmin()), int(lengths.argmax()), 31, 63})
+    for b in sample:
+        n = int(lengths[b])
+        expected, expected_lse = oracle.mla_decode_unrounded(
+            data["query"][b:b + 1], data["cache"][b:b + 1, :n], lengths[b:b + 1], data["scale"])
+        assert_close_bf16(f"O[{b}]", out[b:b + 1], expected)
+        assert_close_lse(f"LSE[{b}]", lse[b:b + 1], expected_lse)
+
+
+# ---- absorbed causal prefill forward (dscuda_mla_forward) ----------------------
+
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 200, 128)])
+def test_absorbed_forward(cuda, batch, tokens, heads):
+    ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
+    announce("mla_forward", dict(B=batch, T=tokens, H=heads))
+    out, lse = ops.mla_forward(ql.to(cuda), qr.to(cuda), c.to(cuda), kr.to(cuda), scale)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, oracle.causal_mask(tokens))
+    assert_close_bf16("O", out, expected)
+    assert_close_lse("LSE", lse, expected_lse)
+
+
+def test_absorbed_forward_closed_form_constant_fill(cuda):
+    """benchmarks/attention/benchmark_mla.cu:38-47: O == 0.25, LSE[t] = 0.6614583 + ln(t+1)."""
+    batch, tokens, heads = 1, 128, 8
+    ql = torch.full((batch, tokens, heads, 512), 0.125).bfloat16()
+    qr = torch.full((batch, tokens, heads, 64), -0.0625).bfloat16()
+    c = torch.full((batch, tokens, 512), 0.25).bfloat16()
+    kr = torch.full((batch, tokens, 64), 0.03125).bfloat16()
+    out, lse = ops.mla_forward(ql.to(cuda), qr.to(cuda), c.to(cuda), kr.to(cuda), 1.0 / 24.0)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().float(), torch.full((batch, tokens, heads, 512), 0.25))
+    expected = 0.6614583333 + torch.log(torch.arange(1, tokens + 1, dtype=torch.float32))
+    assert (lse.cpu() - expected[None, None]).abs().max() <= 1e-4
