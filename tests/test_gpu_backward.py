@@ -1,0 +1,85 @@
+"""GPU parity of the recompute-based backward of the per-head MLA prefill
+against the fp32 oracle (analytic formulas pinned to autograd), through the
+C-ABI.  As in the reference harness (benchmarks/mla.py:68,113-117) the
+backward is fed the oracle's own bf16-rounded O and fp32 LSE, so forward and
+backward are tested independently."""
+
+import pytest
+import torch
+
+from dscuda_amd.harness import configs, ops
+from oracle import attention_oracle as oracle
+from tests.parity import announce, assert_close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _backward_case(cuda, batch, seq, heads, nope, rope, dv, seed, heads_checked=None, dout_factor=1.0):
+    q, k, v, scale = configs.mla_prefill_inputs(batch, seq, heads, nope=nope, rope=rope, dv=dv, seed=seed,
+                                                rotate=rope > 0)
+    dout = configs.mla_prefill_dout(batch, seq, heads, dv, seed=seed + 100, factor=dout_factor)
+    heads_checked = list(range(heads)) if heads_checked is None else heads_checked
+    out_f, lse_f = oracle.causal_attention_forward(q, k, v, scale, heads=heads_checked)
+    # saved tensors: bf16 O and fp32 LSE for every head (unchecked heads get zeros: their gradients are not compared)
+    out = torch.zeros(batch, seq, heads, dv, dtype=torch.bfloat16)
+    lse = torch.zeros(batch, heads, seq, dtype=torch.float32)
+    out[:, :, heads_checked] = out_f.bfloat16()
+    lse[:, heads_checked] = lse_f
+    announce("mla_prefill_backward", dict(B=batch, S=seq, H=heads, dqk=nope + rope, dv=dv))
+    dq, dk, dvg = ops.mla_prefill_backward(dout.to(cuda), out.to(cuda), lse.to(cuda), q.to(cuda), k.to(cuda),
+                                           v.to(cuda), scale)
+    torch.cuda.synchronize()
+    sub = lambda t: t[:, :, heads_checked]
+    eq, ek, ev = oracle.attention_backward(sub(dout), sub(out), lse[:, heads_checked], sub(q), sub(k), sub(v), scale)
+    assert_close_bf16("dQ", sub(dq.cpu()), eq)
+    assert_close_bf16("dK", sub(dk.cpu()), ek)
+    assert_close_bf16("dV", sub(dvg.cpu()), ev)
+
+
+@pytest.mark.parametrize("batch,seq,heads", [(1, 1, 1), (2, 17, 3), (1, 65, 4), (1, 128, 8), (2, 257, 4), (1, 512, 8),
+                                             (1, 1000, 2)])
+def test_backward_small(cuda, batch, seq, heads):
+    # ragged lengths as in benchmarks/mla.py:35-39,44, per-head 192/128 geometry
+    _backward_case(cuda, batch, seq, heads, 128, 64, 128, seed=21)
+
+
+@pytest.mark.parametrize("dqk,dv", [(128, 128), (64, 64)])
+def test_backward_square_heads(cuda, dqk, dv):
+    _backward_case(cuda, 1, 320, 4, dqk, 0, dv, seed=22)
+
+
+def test_backward_constant_key_gives_zero_dq(cuda):
+    """With K constant along the sequence every score of a row is equal, dS sums to zero
+    over the row and dQ = dS K vanishes."""
+    batch, seq, heads = 1, 192, 2
+    q, k, v, scale = configs.mla_prefill_inputs(batch, seq, heads, seed=23)
+    k = k[:, :1].expand(batch, seq, heads, 192).contiguous()
+    dout = configs.mla_prefill_dout(batch, seq, heads, 128, seed=24)
+    out_f, lse = oracle.causal_attention_forward(q, k, v, scale)
+    dq, dk, dvg = ops.mla_prefill_backward(dout.to(cuda), out_f.bfloat16().to(cuda), lse.to(cuda), q.to(cuda),
+                                           k.to(cuda), v.to(cuda), scale)
+    torch.cuda.synchronize()
+    assert dq.float().abs().max().item() <= 2e-2
+
+
+def test_backward_workload_3(cuda):
+    """S=4096, H=128 from seed 1 (+RoPE), dO ~ N(0,1) from seed 2; saved O / LSE and expected
+    gradients from the oracle on a sample of heads."""
+    batch, seq, heads = 1, 4096, 128
+    q, k, v, scale = configs.mla_prefill_inputs(batch, seq, heads, seed=1)
+    dout = configs.mla_prefill_dout(batch, seq, heads, 128, seed=2)
+    checked = [0, 64, 127]
+    out_f, lse_f = oracle.causal_attention_forward(q, k, v, scale, heads=checked)
+    out = torch.zeros(batch, seq, heads, 128, dtype=torch.bfloat16)
+    lse = torch.zeros(batch, heads, seq)
+    out[:, :, checked] = out_f.bfloat16()
+    lse[:, checked] = lse_f
+    announce("mla_prefill_backward workload 3")
+    dq, dk, dvg = ops.mla_prefill_backward(dout.to(cuda), out.to(cuda), lse.to(cuda), q.to(cuda), k.to(cuda),
+                                           v.to(cuda), scale)
+    torch.cuda.synchronize()
+    sub = lambda t: t[:, :, checked]
+    eq, ek, ev = oracle.attention_backward(sub(dout), sub(out), lse[:, checked], sub(q), sub(k), sub(v), scale)
+    assert_close_bf16("dQ", sub(dq.cpu()), eq)
+    assert_close_bf16("dK", sub(dk.cpu()), ek)
+    assert_close_bf16("dV", sub(dvg.cpu()), ev)
