@@ -83,3 +83,45 @@ def test_backward_workload_3(cuda):
     assert_close_bf16("dQ", sub(dq.cpu()), eq)
     assert_close_bf16("dK", sub(dk.cpu()), ek)
     assert_close_bf16("dV", sub(dvg.cpu()), ev)
+
+
+# ---- absorbed backward (dscuda_mla_backward) ------------------------------------
+
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 96, 20)])
+def test_absorbed_backward(cuda, batch, tokens, heads):
+    """Shapes of benchmarks/mla.py:34-45; dO = 0.2 * N(0,1) as at :108; saved O (bf16) and LSE
+    come from the oracle forward as at :68,113-117."""
+    ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
+    g = torch.Generator().manual_seed(77)
+    dout = (torch.randn(batch, tokens, heads, 512, generator=g) * 0.2).bfloat16()
+    mask = oracle.causal_mask(tokens)
+    out, lse = oracle.mla_forward(ql, qr, c, kr, scale, mask)
+    announce("mla_backward", dict(B=batch, T=tokens, H=heads))
+    grads = ops.mla_backward(dout.to(cuda), out.to(cuda), lse.to(cuda), ql.to(cuda), qr.to(cuda), c.to(cuda),
+                             kr.to(cuda), scale)
+    torch.cuda.synchronize()
+    expected = oracle.mla_backward_unrounded(dout, out, lse, ql, qr, c, kr, scale, mask)
+    for name, actual, reference in zip(("dq_latent", "dq_rope", "dlatent", "dk_rope"), grads, expected):
+        assert_close_bf16(name, actual.cpu(), reference)
+
+
+def test_absorbed_backward_closed_form_constant_fill(cuda):
+    """benchmarks/attention/benchmark_mla.cu:38-47 with dO = 2**-6: dS == 0, so dq_latent = dq_rope =
+    dk_rope = 0 and dLatent[k] = H * dO * (Harm(T) - Harm(k))."""
+    batch, tokens, heads = 1, 96, 4
+    ql = torch.full((batch, tokens, heads, 512), 0.125).bfloat16()
+    qr = torch.full((batch, tokens, heads, 64), -0.0625).bfloat16()
+    c = torch.full((batch, tokens, 512), 0.25).bfloat16()
+    kr = torch.full((batch, tokens, 64), 0.03125).bfloat16()
+    dout = torch.full((batch, tokens, heads, 512), 0.015625).bfloat16()
+    scale = 1.0 / 24.0
+    out, lse = oracle.mla_forward(ql, qr, c, kr, scale, oracle.causal_mask(tokens))
+    grads = ops.mla_backward(dout.to(cuda), out.to(cuda), lse.to(cuda), ql.to(cuda), qr.to(cuda), c.to(cuda),
+                             kr.to(cuda), scale)
+    torch.cuda.synchronize()
+    dq, dqr, dlat, dkr = (x.cpu().float() for x in grads)
+    assert dq.abs().max() <= 1e-3 and dqr.abs().max() <= 1e-3 and dkr.abs().max() <= 1e-3
+    harmonic = torch.cumsum(1.0 / torch.arange(1, tokens + 1, dtype=torch.float64), 0)
+    before = torch.cat([torch.zeros(1, dtype=torch.float64), harmonic[:-1]])
+    expected = (heads * 0.015625 * (harmonic[-1] - before)).float()
+    assert (dlat - expected[None, :, None]).abs().max() <= 4e-3  # bf16 rounding of values up to 0.32
