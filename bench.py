@@ -106,7 +106,7 @@ def main():
     extra = {}
     if not args.no_extra:
         from dscuda_amd.harness import extra_workloads
-        extra = extra_workloads.measure(device, event_time_ms, q, k, v, scale, out, lse)
+        extra = extra_workloads.measure(device, event_time_ms, dq, dk, dvv, scale, out, lse)
 
     baseline, parity = cpu_baseline_forward(q, k, v, scale, out, lse, args.cpu_heads)
 

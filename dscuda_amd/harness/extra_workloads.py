@@ -1,16 +1,56 @@
 """The other workloads of the headline metric, timed beside the forward one by
 ``bench.py``: backward TFLOP/s, decode GB/s and the flash-attention forward
-time.  Each entry is skipped (with the reason) while its kernel is missing."""
+time.  All inputs are resident in HBM before the timed region."""
 
 from __future__ import annotations
 
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
 
-def measure(device, event_time_ms, q, k, v, scale, out, lse):
+
+def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3):
+    """q, k, v: the S=4096 H=128 prefill inputs already on `device`; out / lse: the
+    forward's results for them (the backward's saved tensors)."""
     import torch
 
     from . import configs, ops
 
     results = {}
+    batch, seq, heads, dqk = q.shape
+    dv = v.shape[-1]
+
+    # MLA backward, same shape, dO ~ N(0,1) seed 2
+    dout = configs.mla_prefill_dout(batch, seq, heads, dv, seed=2).to(device)
+    grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    workspace = torch.empty(batch * heads * seq, device=device, dtype=torch.float32)
+    ms, _ = event_time_ms(lambda: ops.mla_prefill_backward(dout, out, lse, q, k, v, scale, workspace, grads),
+                          steps, warmup)
+    flops = configs.backward_flops(batch, heads, seq, dqk, dv)
+    results["mla_backward_S4096_H128"] = {
+        "ms": ms, "tflops": flops / ms / 1e9, "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS,
+        "flops": flops, "kernels": "attention_delta + attention_key_gradient + attention_query_gradient"}
+    del dout, grads, workspace
+
+    # absorbed decode, B=64 H=128, lengths ~ U[1024,8192] seed 3, 64-token pages
+    data = configs.mla_decode_inputs()
+    lengths = data["lengths"]
+    total = int(lengths.sum())
+    dq = data["query"].to(device)
+    paged = data["paged"].to(device)
+    table = data["table"].to(device)
+    dl = lengths.to(device)
+    b, h = dq.shape[0], dq.shape[2]
+    workspace = ops.mla_decode_workspace(b, h, 8, 512, device)
+    dout_o = torch.empty(b, 1, h, 512, device=device, dtype=torch.bfloat16)
+    dlse = torch.empty(b, h, 1, device=device, dtype=torch.float32)
+    ms, _ = event_time_ms(lambda: ops.mla_decode(dq, paged, table, dl, data["scale"], splits=8, workspace=workspace,
+                                                 out=dout_o, lse=dlse), 3 * steps, warmup)
+    nbytes = configs.decode_bytes(total, b, h)
+    results["mla_decode_B64_H128"] = {
+        "us": ms * 1000.0, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
+        "bytes": nbytes, "total_tokens": total, "tflops": configs.decode_flops(total, h) / ms / 1e9,
+        "kernels": "mla_decode_split + mla_decode_combine"}
+    del paged, workspace
 
     # flash attention forward, B=1 H=8 S=512 D=64 (latency bound: report time)
     fq, fk, fv, fscale = configs.flash_forward_inputs()

@@ -1,0 +1,119 @@
+"""Host-only checks of the drop-in boundary: both libraries load, export every
+symbol include/*.h declares, and turn invalid arguments into status 1 plus the
+reference's message without touching a GPU (validation precedes any runtime
+call, as in the reference: kernels/attention/mla/sm89.cu:20-24,514)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from dscuda_amd.harness.common import F, I, P, ROOT, bind, checked, library, library_path
+
+
+def _declared_symbols(header):
+    text = (ROOT / "include" / header).read_text()
+    block = text[text.index('extern "C" {'):]
+    return sorted(set(re.findall(r"\b(dscuda_\w+)\s*\(", block)))
+
+
+def test_libraries_exist_under_build():
+    # file names are part of the contract (benchmarks/common.py:19-20)
+    assert library_path("mla").name == "libdscuda_mla_bench.so"
+    assert library_path("flash_attention").name == "libdscuda_flash_attention_bench.so"
+    assert library_path("mla").exists() and library_path("flash_attention").exists()
+
+
+@pytest.mark.parametrize("name,header", [("mla", "mla.h"), ("flash_attention", "flash_attention.h")])
+def test_every_declared_symbol_is_exported(name, header):
+    lib = library(name)
+    symbols = _declared_symbols(header)
+    assert symbols, header
+    for symbol in symbols:
+        assert getattr(lib, symbol) is not None, symbol
+    if name == "mla":
+        assert {"dscuda_mla_forward", "dscuda_mla_backward", "dscuda_mla_decode", "dscuda_mla_workspace_elements",
+                "dscuda_mla_last_error", "dscuda_mla_prefill_forward", "dscuda_mla_prefill_backward",
+                "dscuda_mla_prefill_backward_workspace_elements"} <= set(symbols)
+    else:
+        assert {"dscuda_flash_forward", "dscuda_flash_last_error"} <= set(symbols)
+
+
+def test_workspace_elements_match_the_reference_formula():
+    lib = library("mla")
+    size = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
+    assert size(2, 3, 8, 512) == 2 * 3 * 8 * 514          # kernels/attention/mla/sm89.cu:539-541
+    assert size(64, 128, 8, 512) == 64 * 128 * 8 * 514
+    assert size(4096, 128, 64, 512) == 4096 * 128 * 64 * 514  # needs size_t
+    prefill = bind(lib, "dscuda_mla_prefill_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
+    assert prefill(1, 4096, 128, 192, 128) == 4096 * 128
+
+
+def _status_and_message(lib, prefix, status):
+    with pytest.raises(RuntimeError) as info:
+        checked(lib, prefix, status)
+    return str(info.value)
+
+
+def test_mla_shape_errors_round_trip_without_a_gpu():
+    lib = library("mla")
+    forward = bind(lib, "dscuda_mla_forward", [P] * 6 + [I] * 5 + [F, P])
+    backward = bind(lib, "dscuda_mla_backward", [P] * 11 + [I] * 5 + [F, P])
+    decode = bind(lib, "dscuda_mla_decode", [P] * 7 + [I] * 7 + [F, P])
+    null = [None]
+    assert _status_and_message(lib, "mla", forward(*null * 6, 1, 8, 2, 256, 64, 1.0, None)) == \
+        "MLA requires C=512 and RoPE=64"
+    assert _status_and_message(lib, "mla", backward(*null * 11, 1, 8, 2, 512, 32, 1.0, None)) == \
+        "MLA requires C=512 and RoPE=64"
+    assert _status_and_message(lib, "mla", decode(*null * 7, 1, 8, 128, 64, 64, 4, 8, 1.0, None)) == \
+        "MLA requires C=512 and RoPE=64"
+    assert "positive" in _status_and_message(lib, "mla", forward(*null * 6, 0, 8, 2, 512, 64, 1.0, None))
+    assert "positive" in _status_and_message(lib, "mla", decode(*null * 7, 1, 8, 512, 64, 64, 4, 0, 1.0, None))
+    prefill = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
+    assert "(d_qk,d_v)" in _status_and_message(lib, "mla", prefill(*null * 5, 1, 8, 2, 96, 96, 1.0, None))
+    prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
+    assert "workspace" in _status_and_message(
+        lib, "mla", prefill_backward(*null * 10, 1, 8, 2, 192, 128, 1.0, None))
+
+
+def test_flash_errors_round_trip_without_a_gpu():
+    lib = library("flash_attention")
+    forward = bind(lib, "dscuda_flash_forward", [P] * 5 + [I] * 5 + [F, P])
+    null = [None]
+    # messages of kernels/attention/flash_attention/sm89_forward.cu:226-232 (head-size rule widened to 64 | 128)
+    assert _status_and_message(lib, "flash", forward(*null * 5, 1, 64, 2, 2, 96, 1.0, None)) == \
+        "flash attention requires head_size = 64 or 128"
+    assert _status_and_message(lib, "flash", forward(*null * 5, 1, 65, 2, 2, 128, 1.0, None)) == \
+        "flash attention requires T to be a positive multiple of 64"
+    assert _status_and_message(lib, "flash", forward(*null * 5, 1, 0, 2, 2, 128, 1.0, None)) == \
+        "flash attention requires T to be a positive multiple of 64"
+    assert _status_and_message(lib, "flash", forward(*null * 5, 1, 64, 3, 2, 128, 1.0, None)) == \
+        "flash attention requires query_heads to be divisible by key_value_heads"
+
+
+def test_last_error_is_per_thread_and_sticky():
+    import threading
+    lib = library("mla")
+    forward = bind(lib, "dscuda_mla_forward", [P] * 6 + [I] * 5 + [F, P])
+    last = bind(lib, "dscuda_mla_last_error", [], ctypes.c_char_p)
+    assert forward(*[None] * 6, 1, 8, 2, 100, 64, 1.0, None) == 1
+    first = last().decode()
+    seen = {}
+
+    def other():
+        seen["before"] = last().decode()   # a fresh thread has no error yet
+
+    thread = threading.Thread(target=other)
+    thread.start()
+    thread.join()
+    assert first == "MLA requires C=512 and RoPE=64" and seen["before"] == ""
+    assert last().decode() == first        # still there until the next error on this thread
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from dscuda_amd.harness import ops
+    q = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.flash_forward(q, q, q, 1.0)
