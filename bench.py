@@ -75,7 +75,7 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
-    parser.add_argument("--cpu-heads", type=int, default=32, help="heads in the CPU baseline sample")
+    parser.add_argument("--cpu-heads", type=int, default=128, help="heads in the CPU baseline sample")
     parser.add_argument("--no-extra", action="store_true", help="skip the backward / decode / flash measurements")
     args = parser.parse_args()
     if args.gpus != 1:

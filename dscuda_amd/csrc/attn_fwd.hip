@@ -22,21 +22,25 @@
 //   directly the B operand of O^T += V^T P^T (k index = key), so P never
 //   moves between lanes or through LDS.
 //
-// LDS layout (per stage, two stages)
-//   K  : [64 keys][d_qk] bf16, row pitch 2*d_qk + 16 bytes.  A fragment read
-//        is 16 lanes x 16 B down a column of rows; the odd multiple of 16 B in
-//        the pitch spreads those over all 64 banks.
-//   V^T: [d_v][64 keys] bf16, 128-byte rows, 16-byte chunk index XORed with
-//        (row >> 1) & 7.  V arrives row-major (d_v contiguous) but MFMA wants
-//        the contraction index (key) contiguous per lane, so each thread
-//        transposes a 4 keys x 4 d_v block in registers on the way in.  Inside
-//        each group of 16 keys the two middle groups of four are swapped so
-//        that the eight keys a lane needs (the C-layout row set
-//        {4g..4g+3, 8+4g..8+4g+3}) are one aligned 16-byte read.
-//
-// Global -> LDS goes through registers: the next tile's loads are issued
-// before the current tile's math and written to the other stage after it,
-// one workgroup barrier per tile.
+// Tiles: global -> LDS without registers
+//   K and V tiles arrive by global_load_lds (16 bytes per lane, 1 KB of
+//   consecutive LDS per wave instruction), both row-major, two stages.  No
+//   thread holds tile data in registers and nothing is written to LDS with
+//   store instructions.  With no padding possible inside the 1 KB a wave
+//   instruction fills, bank spread comes from a swizzle applied on the global
+//   side (which 16-byte chunk a lane fetches):
+//     K  : chunk c of row r sits at position c ^ fK(r).  A fragment read is 16
+//          lanes x 16 B down a column of rows; fK(r) = (r>>1)&7 for rows that
+//          are 128 (mod 256) bytes long, r&15 for rows that are 0 (mod 256).
+//     V  : MFMA wants the contraction index (key) contiguous per lane, V has
+//          d_v contiguous.  ds_read_b64_tr_b16 transposes a 4 keys x 16 columns
+//          block across 16 lanes while reading, so the row-major tile is used
+//          as it is.  Such a read touches 4 rows x 64 bytes; rows are 64*NG
+//          bytes long (NG = d_v/32 column groups), so the 64-byte group index
+//          of row r is XORed with r&3 (NG = 4) or (r>>1)&1 (NG = 2), and the
+//          lane that addresses row r undoes it in its own address.
+//   A tile is requested while the previous one is consumed; arrival is ordered
+//   by s_waitcnt vmcnt + one workgroup barrier per tile.
 #include "attn_kernels.h"
 #include "hip_common.h"
 
@@ -52,22 +56,35 @@ struct FwdConfig {
     static constexpr int BN = 64;
     static constexpr int BM = 32 * NWAVES;
     static constexpr int THREADS = 64 * NWAVES;
-    static constexpr int K_PITCH = DQK * 2 + 16;           // bytes
-    static constexpr int K_BYTES = BN * K_PITCH;
-    static constexpr int VT_PITCH = BN * 2;                 // bytes, swizzled
-    static constexpr int VT_BYTES = DV * VT_PITCH;
-    static constexpr int STAGE_BYTES = K_BYTES + VT_BYTES;
-    static constexpr int K_CHUNKS = BN * (DQK / 8);         // 16-byte chunks per K tile
-    static constexpr int K_PER_THREAD = K_CHUNKS / THREADS;
-    static constexpr int V_UNITS = (BN / 4) * (DV / 4);     // 4 keys x 4 d_v blocks per V tile
-    static constexpr int V_PER_THREAD = V_UNITS / THREADS;
-    static constexpr int O_PITCH = DV * 2 + 16;             // epilogue staging, bytes
+    static constexpr int K_ROW = DQK * 2;                  // bytes
+    static constexpr int K_CHUNKS = DQK / 8;               // 16-byte chunks per row
+    static constexpr int K_BYTES = BN * K_ROW;
+    static constexpr int V_ROW = DV * 2;
+    static constexpr int V_CHUNKS = DV / 8;
+    static constexpr int V_GROUPS = DV / 32;               // 64-byte column groups per row
+    static constexpr int V_BYTES = BN * V_ROW;
+    static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
+    static constexpr int K_LOADS_PER_WAVE = K_BYTES / 1024 / NWAVES;   // wave instructions
+    static constexpr int V_LOADS_PER_WAVE = V_BYTES / 1024 / NWAVES;
+    static constexpr int O_PITCH = DV * 2 + 16;            // epilogue staging, bytes
     static constexpr int O_BYTES = BM * O_PITCH;
     static constexpr int LDS_BYTES = (2 * STAGE_BYTES > O_BYTES) ? 2 * STAGE_BYTES : O_BYTES;
-    static_assert(K_CHUNKS % THREADS == 0, "K tile must divide evenly over the workgroup");
-    static_assert(V_UNITS % THREADS == 0, "V tile must divide evenly over the workgroup");
-    static_assert(DQK % 16 == 0 && DV % 32 == 0, "head sizes must fit the MFMA tile");
+    static_assert(K_BYTES % (1024 * NWAVES) == 0 && V_BYTES % (1024 * NWAVES) == 0,
+                  "tile loads must divide evenly over the waves");
+    static_assert(K_ROW % 128 == 0, "K rows must be a multiple of 128 bytes");
+    static_assert(V_GROUPS == 2 || V_GROUPS == 4, "d_v must be 64 or 128");
+
+    __device__ static constexpr int k_swizzle(int row) {
+        return (K_ROW % 256 == 0) ? (row & 15) : ((row >> 1) & 7);
+    }
+    __device__ static constexpr int v_flip(int row) {
+        return V_GROUPS == 4 ? (row & 3) : ((row >> 1) & 1);
+    }
 };
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4* transposing_read_pointer;
 
 template <int DQK, int DV, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
@@ -82,7 +99,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
@@ -102,11 +119,13 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
     const int q_row = wave_q0 + lq;
 
     const size_t q_stride = (size_t)query_heads * DQK;
-    const size_t k_stride = (size_t)key_value_heads * DQK;
-    const size_t v_stride = (size_t)key_value_heads * DV;
+    const unsigned k_stride_bytes = (unsigned)key_value_heads * DQK * 2;
+    const unsigned v_stride_bytes = (unsigned)key_value_heads * DV * 2;
     const bf16_t* q_base = query + ((size_t)b * S * query_heads + h) * DQK;
-    const bf16_t* k_base = key + ((size_t)b * S * key_value_heads + hk) * DQK;
-    const bf16_t* v_base = value + ((size_t)b * S * key_value_heads + hk) * DV;
+    const unsigned char* k_base =
+        reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * key_value_heads + hk) * DQK);
+    const unsigned char* v_base =
+        reinterpret_cast<const unsigned char*>(value + ((size_t)b * S * key_value_heads + hk) * DV);
 
     // ---- Q fragments (B operand: column = query lq, k = 16*ks + 8*g + j)
     bf16x8 qf[KSTEPS];
@@ -125,73 +144,34 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
 
     const int last_key = min(S, q0 + C::BM) - 1;
     const int tiles = last_key / BN + 1;
+    const unsigned lds_base = lds_offset_of(lds);
 
-    u32x4 k_stage[C::K_PER_THREAD];
-    u32x2 v_stage[C::V_PER_THREAD][4];
-
-    auto load_tile = [&](int tile) {
+    // Requests this wave's share of tile `tile` into `stage`.  Rows past the end
+    // of the sequence are clamped to the last one: such keys are invisible to
+    // every stored query, the data only has to be finite.
+    auto request_tile = [&](int tile, int stage) {
         const int key0 = tile * BN;
+        const int row_limit = S - 1 - key0;
+        const unsigned char* k_tile = k_base + (size_t)key0 * k_stride_bytes;
+        const unsigned char* v_tile = v_base + (size_t)key0 * v_stride_bytes;
+        const unsigned stage_base = lds_base + stage * C::STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < C::K_PER_THREAD; ++i) {
-            const int id = tid + C::THREADS * i;
-            const int row = id / (DQK / 8);
-            const int col = id % (DQK / 8);
-            const int k = key0 + row;
-            u32x4 bits = {0, 0, 0, 0};
-            if (k < S) {
-                bits = *reinterpret_cast<const u32x4*>(k_base + (size_t)k * k_stride + 8 * col);
-            }
-            k_stage[i] = bits;
+        for (int i = 0; i < C::K_LOADS_PER_WAVE; ++i) {
+            const int load = wave * C::K_LOADS_PER_WAVE + i;
+            const int slot = 64 * load + lane;
+            const int row = slot / C::K_CHUNKS;
+            const int chunk = (slot % C::K_CHUNKS) ^ C::k_swizzle(row);
+            const unsigned offset = (unsigned)min(row, row_limit) * k_stride_bytes + 16u * chunk;
+            direct_load_16_offset(k_tile, offset, stage_base + load * 1024);
         }
 #pragma unroll
-        for (int i = 0; i < C::V_PER_THREAD; ++i) {
-            const int unit = tid + C::THREADS * i;
-            const int c4 = unit % (DV / 4);
-            const int kg = unit / (DV / 4);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = key0 + 4 * kg + j;
-                u32x2 bits = {0, 0};
-                if (k < S) {
-                    bits = *reinterpret_cast<const u32x2*>(v_base + (size_t)k * v_stride + 4 * c4);
-                }
-                v_stage[i][j] = bits;
-            }
-        }
-    };
-
-    auto store_tile = [&](int stage) {
-        unsigned char* k_lds = lds + stage * C::STAGE_BYTES;
-        unsigned char* vt_lds = k_lds + C::K_BYTES;
-#pragma unroll
-        for (int i = 0; i < C::K_PER_THREAD; ++i) {
-            const int id = tid + C::THREADS * i;
-            const int row = id / (DQK / 8);
-            const int col = id % (DQK / 8);
-            *reinterpret_cast<u32x4*>(k_lds + row * C::K_PITCH + 16 * col) = k_stage[i];
-        }
-#pragma unroll
-        for (int i = 0; i < C::V_PER_THREAD; ++i) {
-            const int unit = tid + C::THREADS * i;
-            const int c4 = unit % (DV / 4);
-            const int kg = unit / (DV / 4);
-            // keys 4*kg .. 4*kg+3 = 16*n + 8*a + 4*g' + (0..3)  ->  position 16*n + 8*g' + 4*a
-            const int n = kg / 4;
-            const int a = (kg % 4) / 2;
-            const int gp = kg % 2;
-            const int chunk = 2 * n + gp;
-            const u32x2 r0 = v_stage[i][0], r1 = v_stage[i][1], r2 = v_stage[i][2], r3 = v_stage[i][3];
-            u32x2 t[4];
-            t[0] = u32x2{(r0.x & 0xffffu) | (r1.x << 16), (r2.x & 0xffffu) | (r3.x << 16)};
-            t[1] = u32x2{(r0.x >> 16) | (r1.x & 0xffff0000u), (r2.x >> 16) | (r3.x & 0xffff0000u)};
-            t[2] = u32x2{(r0.y & 0xffffu) | (r1.y << 16), (r2.y & 0xffffu) | (r3.y << 16)};
-            t[3] = u32x2{(r0.y >> 16) | (r1.y & 0xffff0000u), (r2.y >> 16) | (r3.y & 0xffff0000u)};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int dv = 4 * c4 + e;
-                const int swz = chunk ^ ((dv >> 1) & 7);
-                *reinterpret_cast<u32x2*>(vt_lds + dv * C::VT_PITCH + 16 * swz + 8 * a) = t[e];
-            }
+        for (int i = 0; i < C::V_LOADS_PER_WAVE; ++i) {
+            const int load = wave * C::V_LOADS_PER_WAVE + i;
+            const int slot = 64 * load + lane;
+            const int row = slot / C::V_CHUNKS;
+            const int chunk = (slot % C::V_CHUNKS) ^ (C::v_flip(row) << 2);
+            const unsigned offset = (unsigned)min(row, row_limit) * v_stride_bytes + 16u * chunk;
+            direct_load_16_offset(v_tile, offset, stage_base + C::K_BYTES + load * 1024);
         }
     };
 
@@ -205,20 +185,27 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
     float row_sum = 0.f;        // this lane's share (its 32 keys per tile) of the normaliser
     const float c = scale * LOG2E;
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
+    // Per-lane pieces of the LDS read addresses.
+    const int k_swz = C::k_swizzle(lq);                        // rows lq and lq+32 share it
+    const int s16 = lane % 16;
+    const int v_row = 4 * g + s16 / 4;                          // + 16*n, + 8 for the second read
+    const int v_in_group = 32 * ((lane / 16) % 2) + 8 * (s16 % 4);
+    const int v_flip = C::v_flip(v_row);                        // rows v_row + 8*m share it
+
+    wait_vector_memory<0>();   // the query loads: no wait for them may remain inside the loop
+    request_tile(0, 0);
 
     for (int tile = 0; tile < tiles; ++tile) {
         const int stage = tile & 1;
-        const bool more = tile + 1 < tiles;
-        if (more) {
-            load_tile(tile + 1);
+        wait_vector_memory<0>();   // this wave's share of the tile has landed
+        workgroup_barrier();       // ... and everybody's; every wave has left the previous tile
+        if (tile + 1 < tiles) {
+            request_tile(tile + 1, stage ^ 1);
         }
         const int key0 = tile * BN;
         if (key0 <= wave_q0 + 31) {  // otherwise every key of the tile is in this wave's future
             const unsigned char* k_lds = lds + stage * C::STAGE_BYTES;
-            const unsigned char* vt_lds = k_lds + C::K_BYTES;
+            const unsigned char* v_lds = k_lds + C::K_BYTES;
 
             f32x16 s_acc[2];
 #pragma unroll
@@ -228,10 +215,11 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
             }
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
+                const int position = (2 * ks + g) ^ k_swz;
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) {
-                    const bf16x8 a = *reinterpret_cast<const bf16x8*>(
-                        k_lds + (32 * mb + lq) * C::K_PITCH + 32 * ks + 16 * g);
+                    const bf16x8 a =
+                        *reinterpret_cast<const bf16x8*>(k_lds + (32 * mb + lq) * C::K_ROW + 16 * position);
                     s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s_acc[mb], 0, 0, 0);
                 }
             }
@@ -287,24 +275,31 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
                 pf[n] = __builtin_bit_cast(bf16x8, packed);
             }
 
+            // V^T operand through transposing reads.  In a block of 16 lanes, lane s
+            // points at key row 16n + 4g + s/4 (+8 for the second read) and columns
+            // 4*(s%4)..+3 of the 16-column half (block%2) of column group d; the
+            // instruction hands lane i column i of the four rows.  Together: MFMA row
+            // lane%32, keys {4g..4g+3, 8+4g..8+4g+3} of the 16-key step, the k-order
+            // P^T carries from the C layout.
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
 #pragma unroll
                 for (int d = 0; d < DBLOCKS; ++d) {
-                    const int dv = 32 * d + lq;
-                    const int swz = (2 * n + g) ^ ((dv >> 1) & 7);
-                    const bf16x8 a = *reinterpret_cast<const bf16x8*>(vt_lds + dv * C::VT_PITCH + 16 * swz);
-                    o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[n], o_acc[d], 0, 0, 0);
+                    const unsigned char* first =
+                        v_lds + (16 * n + v_row) * C::V_ROW + 64 * (d ^ v_flip) + v_in_group;
+                    const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)first);
+                    const s16x4 high =
+                        __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(first + 8 * C::V_ROW));
+                    const s16x8 both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n],
+                                                                       o_acc[d], 0, 0, 0);
                 }
             }
         }
-        if (more) {
-            store_tile(stage ^ 1);
-        }
-        __syncthreads();
     }
 
     // ---- epilogue: normalise, stage O through LDS for 16-byte row stores
+    workgroup_barrier();   // every wave is done reading the tile stages
     const float total = half_wave_sum(row_sum);
     const float inverse = 1.0f / total;
     if (g == 0 && q_row < S) {
@@ -349,6 +344,10 @@ void launch_forward(bf16_t* output, float* logsumexp, const bf16_t* query, const
     const long long grid = groups * query_blocks;
     if (grid > 0x7fffffffLL) {
         throw std::invalid_argument("attention forward: batch*heads*query_blocks exceeds the grid limit");
+    }
+    // per-lane byte offsets inside a key tile are 32-bit
+    if ((long long)key_value_heads * (DQK > DV ? DQK : DV) * 2 * C::BN > 0x7fffffffLL) {
+        throw std::invalid_argument("attention forward: key_value_heads * head size is too large");
     }
     auto kernel = attention_forward_kernel<DQK, DV, NWAVES>;
     if (C::LDS_BYTES > 64 * 1024) {

@@ -85,6 +85,62 @@ __device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
     return __uint_as_float(bits16 << 16);
 }
 
+// ---- direct global -> LDS loads and the synchronisation that goes with them ----
+//
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight
+// into LDS at (M0 base) + 16 * lane; a wave instruction fills 1 KB of
+// consecutive LDS.  The loads are issued as asm so that the compiler's
+// wait-count bookkeeping does not see an LDS writer: it would otherwise drain
+// every outstanding load before each LDS read of the tile being consumed and
+// serialise the prefetch.  Arrival is ordered by hand: wait_vector_memory
+// (per wave) followed by workgroup_barrier (all waves).
+
+typedef __attribute__((address_space(3))) void* lds_pointer;
+
+__device__ __forceinline__ unsigned lds_offset_of(const void* pointer) {
+    return (unsigned)(uintptr_t)(lds_pointer)pointer;
+}
+
+// source = per-lane 64-bit address; lds_base wave-uniform
+__device__ __forceinline__ void direct_load_16(const void* source, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(source), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
+// source = uniform 64-bit base + per-lane 32-bit byte offset; lds_base wave-uniform
+__device__ __forceinline__ void direct_load_16_offset(const void* uniform_base, unsigned byte_offset, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(uniform_base), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
+// vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt/lgkmcnt unconstrained).
+template <int COUNT>
+__device__ __forceinline__ void wait_vector_memory() {
+    __builtin_amdgcn_s_waitcnt((COUNT & 15) | ((COUNT >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Workgroup barrier without the full memory fence of __syncthreads(): the fence
+// would wait for every outstanding vector-memory operation, i.e. for loads that
+// are meant to stay in flight across the barrier.  LDS traffic of this wave is
+// drained.
+__device__ __forceinline__ void workgroup_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Lane id read afresh.  Being volatile, nothing computed from it is hoisted out
+// of a loop: per-lane addresses are recomputed where they are used (a handful
+// of integer ops) instead of being carried in registers.
+__device__ __forceinline__ int fresh_lane_id() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
 // XCD-aware work-item order.  Workgroups are handed to the 8 XCDs round-robin
 // by linear id; every XCD has a private L2.  Items are grouped so that the
 // `inner` items that share operands (the query blocks of one head) run on one

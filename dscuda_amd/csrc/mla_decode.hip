@@ -68,7 +68,6 @@ constexpr int DBLOCKS = RANK / 32;          // 16
 constexpr int MAX_SEQUENCES = 3072;         // prefix table that fits beside the two stages
 constexpr int EPILOGUE_PITCH = 1024 + 16;   // bytes per staged output row
 
-typedef __attribute__((address_space(3))) void* lds_pointer;
 typedef const __attribute__((address_space(1))) void* global_pointer;
 
 __device__ __forceinline__ int swizzle_of_row(int row) {
@@ -76,37 +75,8 @@ __device__ __forceinline__ int swizzle_of_row(int row) {
     return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
 }
 
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
-// vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt/lgkmcnt unconstrained).
-template <int COUNT>
-__device__ __forceinline__ void wait_vector_memory() {
-    __builtin_amdgcn_s_waitcnt((COUNT & 15) | ((COUNT >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// Workgroup barrier without the full memory fence of __syncthreads(): the fence
-// would wait for every outstanding vector-memory operation, i.e. for the next
-// tile's direct-to-LDS loads that are meant to stay in flight across the
-// barrier.  LDS traffic of this wave is drained; arrival of a tile is ordered
-// separately by wait_vector_memory before the barrier.
-__device__ __forceinline__ void workgroup_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-__device__ __forceinline__ unsigned lds_offset_of(const void* pointer) {
-    return (unsigned)(uintptr_t)(lds_pointer)pointer;
-}
-
-// 16 bytes per lane from global memory straight into LDS at
-// lds_base + 16 * lane (lds_base wave-uniform).  Issued as asm so that the
-// compiler's wait-count bookkeeping does not see an LDS writer: it would
-// otherwise drain every outstanding load before each LDS read of the tile
-// being consumed, serialising the prefetch.  Arrival is ordered by hand with
-// wait_vector_memory + workgroup_barrier.
-__device__ __forceinline__ void direct_load_16(const void* source, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"(source), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
+__device__ __forceinline__ float uniform(float value) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, value)));
 }
 
 struct KeyStream {
@@ -118,47 +88,96 @@ struct KeyStream {
     int page_size;
 };
 
-// Issue the direct-to-LDS loads of one 64-token tile.  Tokens past
-// `last_token` are clamped to it (their rows are zeroed afterwards), so no
-// byte outside the visible part of the sequence is ever read.
-__device__ __forceinline__ void issue_tile(unsigned char* stage_base, const KeyStream& keys, int key0, int last_token,
-                                           int wave, int lane) {
+// Where one 64-token tile comes from and goes to.  Tokens past the last visible
+// one are clamped to it (their rows are zeroed after arrival), so no byte
+// outside the visible part of the sequence is ever read.
+//
+// Wave w fills rows 16w .. 16w+15 (18 instructions of 64 slots = 16 rows of 72
+// slots), so every row / position split is a compile-time constant plus one
+// compare on the lane id.
+//
+// `contiguous`: the tile is one run of 576-wide rows (packed cache, and either
+// no paging or pages that hold whole tiles): a uniform 64-bit base plus a
+// 32-bit per-lane offset, about eight integer ops per load.  Such loads are
+// cheap enough to be issued one at a time between the MFMA groups of the tile
+// being consumed, which keeps the memory pipeline fed without ever stalling a
+// wave on a full request queue.
+struct TileSource {
+    const bf16_t* tile_base;   // contiguous form only
+    unsigned lds_base;         // LDS byte offset of this wave's 18 KB
+    int key0;
+    int row_limit;             // rows above it are clamped (>= 0: the tile holds a visible token)
+    bool contiguous;
+    bool enabled;
+};
+
+__device__ __forceinline__ TileSource locate_tile(unsigned char* stage_base, const KeyStream& keys, int key0,
+                                                  int last_token, int wave, bool enabled) {
+    TileSource source;
     const bool paged = keys.block_table != nullptr;
-    const bool page_holds_tile = paged && (keys.page_size % BN == 0);
-    long long tile_physical = key0;
-    if (page_holds_tile) {
-        const int page = keys.block_table[key0 / keys.page_size];
-        tile_physical = (long long)page * keys.page_size + key0 % keys.page_size;
+    const bool page_holds_tile = !paged || (keys.page_size % BN == 0);
+    const bool packed = keys.rope == keys.latent + RANK && keys.latent_stride == WIDTH && keys.rope_stride == WIDTH;
+    source.contiguous = packed && page_holds_tile;
+    source.enabled = enabled;
+    source.key0 = key0;
+    source.row_limit = last_token - key0;
+    source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(stage_base) + wave * (LOADS_PER_THREAD * 1024));
+    source.tile_base = keys.latent;
+    if (enabled && source.contiguous) {
+        long long tile_physical = key0;
+        if (paged) {
+            const int page = keys.block_table[key0 / keys.page_size];
+            tile_physical = (long long)page * keys.page_size + key0 % keys.page_size;
+        }
+        source.tile_base = keys.latent + tile_physical * WIDTH;
     }
-    // Slot of load i is (4*i + wave)*64 + lane; it advances by 256 = 3*72 + 40
-    // per load, which keeps row / position an add and a compare instead of a
-    // division (and keeps 18 precomputed addresses out of the register file).
-    int row = (wave * 64 + lane) / CHUNKS;
-    int position = (wave * 64 + lane) % CHUNKS;
-    unsigned destination_offset = lds_offset_of(stage_base) + wave * 1024;
+    return source;
+}
+
+// Load number i (0..17) of a contiguous tile; i is a constant after unrolling,
+// which leaves scalar arithmetic for the row part of the address and three
+// cheap vector ops (add, xor, shift-add) per candidate row for the lane part.
+__device__ __forceinline__ void issue_contiguous_load(const TileSource& source, int wave, int i, int lane) {
+    const int first_row = (64 * i) / CHUNKS;                 // row of lane 0 (within the wave's 16 rows)
+    const int boundary = CHUNKS * (first_row + 1) - 64 * i;  // first lane of the next row (may be >= 64)
+    // f depends on bits 1..3 of the row; 16*wave leaves them alone
+    const unsigned row_a = (unsigned)min(16 * wave + first_row, source.row_limit) * ROW_BYTES;        // scalar
+    unsigned offset = row_a + 16u * (unsigned)((lane + 64 * i - CHUNKS * first_row) ^ swizzle_of_row(first_row));
+    if (boundary < 64) {
+        const unsigned row_b = (unsigned)min(16 * wave + first_row + 1, source.row_limit) * ROW_BYTES;
+        const unsigned other =
+            row_b + 16u * (unsigned)((lane + 64 * i - CHUNKS * (first_row + 1)) ^ swizzle_of_row(first_row + 1));
+        offset = lane >= boundary ? other : offset;
+    }
+    direct_load_16_offset(source.tile_base, offset, source.lds_base + i * 1024);
+}
+
+// All 18 loads of a tile at once (first tile of a walk, and every tile of the
+// general form: per-lane page lookup and separate latent / rope tensors).
+__device__ __forceinline__ void issue_tile(const TileSource& source, const KeyStream& keys, int wave) {
+    if (!source.enabled) return;
+    if (source.contiguous) {
+#pragma unroll
+        for (int i = 0; i < LOADS_PER_THREAD; ++i) issue_contiguous_load(source, wave, i, fresh_lane_id());
+        return;
+    }
+    const int lane = fresh_lane_id();
+    const bool paged = keys.block_table != nullptr;
 #pragma unroll 1
     for (int i = 0; i < LOADS_PER_THREAD; ++i) {
-        const int chunk = position ^ swizzle_of_row(row);
-        const int token = min(key0 + row, last_token);
-        long long physical;
-        if (!paged) {
-            physical = token;
-        } else if (page_holds_tile) {
-            physical = tile_physical + (token - key0);
-        } else {
+        const int slot = 64 * i + lane;
+        const int local_row = slot / CHUNKS;
+        const int position = slot % CHUNKS;
+        const int chunk = position ^ swizzle_of_row(local_row);
+        const int token = source.key0 + min(16 * wave + local_row, source.row_limit);
+        long long physical = token;
+        if (paged) {
             const int page = keys.block_table[token / keys.page_size];
             physical = (long long)page * keys.page_size + token % keys.page_size;
         }
-        const bf16_t* source = chunk < RANK / 8 ? keys.latent + physical * keys.latent_stride + 8 * chunk
-                                                : keys.rope + physical * keys.rope_stride + 8 * (chunk - RANK / 8);
-        direct_load_16(source, destination_offset);
-        destination_offset += 4 * 1024;
-        row += 3;
-        position += 40;
-        if (position >= CHUNKS) {
-            position -= CHUNKS;
-            row += 1;
-        }
+        const bf16_t* address = chunk < RANK / 8 ? keys.latent + physical * keys.latent_stride + 8 * chunk
+                                                 : keys.rope + physical * keys.rope_stride + 8 * (chunk - RANK / 8);
+        direct_load_16(address, source.lds_base + i * 1024);
     }
 }
 
@@ -210,15 +229,14 @@ constexpr float FAST_LIMIT = 80.0f;
 template <bool SAFE>
 __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const bf16x8 (&qf)[KSTEPS],
                                              const unsigned char* stage, int key0, int limit, int wave_min_limit,
-                                             bool first, float c, int lane_id) {
+                                             bool first, float c, int lane_id, const TileSource& next_tile, int wave) {
     // The per-lane LDS offsets below are recomputed for every tile from an
     // lane id read afresh (volatile, so nothing derived from it is hoisted): kept
     // live across the loop they would be the registers that no longer fit and
     // get spilled, and a scratch reload inside the loop stalls on the tile
     // prefetch.
     (void)lane_id;
-    int lane;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    const int lane = fresh_lane_id();
     const int lq = lane % 32;
     const int g = lane / 32;
 
@@ -265,35 +283,44 @@ __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const 
         // and a compiler-issued MFMA would want 16 more of them for the scores.
         // The score chain is therefore issued by hand with its accumulator in
         // ordinary registers (score_mfma_*).
-        f32x16 s_acc;
+        f32x16 s_acc, s_odd;
         {
-            constexpr int GROUPS = KSTEPS / 4;
-            bf16x8 current[4], next[4];
+            constexpr int WIDTH_K = 4;   // K fragments per pipeline group
+            constexpr int GROUPS = KSTEPS / WIDTH_K;
+            bf16x8 current[WIDTH_K], next[WIDTH_K];
+            auto fragment = [&](int ks) {
+                return *reinterpret_cast<const bf16x8*>(k_lane[ks % 4] + mb * 32 * ROW_BYTES + (ks / 4) * 128);
+            };
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                current[j] = *reinterpret_cast<const bf16x8*>(k_lane[j] + mb * 32 * ROW_BYTES);
-            }
+            for (int j = 0; j < WIDTH_K; ++j) current[j] = fragment(j);
 #pragma unroll
             for (int group = 0; group < GROUPS; ++group) {
                 if (group + 1 < GROUPS) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        next[j] = *reinterpret_cast<const bf16x8*>(k_lane[j] + mb * 32 * ROW_BYTES + (group + 1) * 128);
-                    }
+                    for (int j = 0; j < WIDTH_K; ++j) next[j] = fragment(WIDTH_K * (group + 1) + j);
                 }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (group == 0 && j == 0) {
-                        score_mfma_first(s_acc, current[j], qf[0]);
+                for (int j = 0; j < WIDTH_K; ++j) {
+                    // two interleaved chains (even / odd k-steps): a dependent MFMA
+                    // would otherwise wait out the previous one's full latency
+                    const int ks = WIDTH_K * group + j;
+                    f32x16& chain = (ks % 2 == 0) ? s_acc : s_odd;
+                    if (ks < 2) {
+                        score_mfma_first(chain, current[j], qf[ks]);
                     } else {
-                        score_mfma(s_acc, current[j], qf[4 * group + j]);
+                        score_mfma(chain, current[j], qf[ks]);
                     }
                 }
+                // the next tile's loads ride along with the first half's MFMA groups
+                if (mb == 0 && next_tile.enabled && next_tile.contiguous) issue_contiguous_load(next_tile, wave, group, lane);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) current[j] = next[j];
+                for (int j = 0; j < WIDTH_K; ++j) current[j] = next[j];
             }
             score_mfma_drain(s_acc);
+            score_mfma_drain(s_odd);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_acc[i] += s_odd[i];
         }
 
         if (key0 + 32 * mb + 32 > wave_min_limit) {
@@ -343,8 +370,8 @@ __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const 
         __builtin_amdgcn_sched_barrier(0);
 
         {
-            // 32 MFMAs (2 key steps x 16 column blocks) in 16 groups of two column blocks
-            constexpr int WIDTH_G = 2;
+            // 32 MFMAs (2 key steps x 16 column blocks) in 8 groups of four column blocks
+            constexpr int WIDTH_G = 4;
             constexpr int GROUPS = 2 * DBLOCKS / WIDTH_G;
             s16x4 cur_lo[WIDTH_G], cur_hi[WIDTH_G], next_lo[WIDTH_G], next_hi[WIDTH_G];
             auto step_of = [&](int group, int j) {
@@ -372,6 +399,10 @@ __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const 
                     const int d = WIDTH_G * (group % (DBLOCKS / WIDTH_G)) + j;
                     const s16x8 both = __builtin_shufflevector(cur_lo[j], cur_hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
                     state.o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n], state.o[d], 0, 0, 0);
+                }
+                if (mb == 0 && next_tile.enabled && next_tile.contiguous) {
+                    issue_contiguous_load(next_tile, wave, KSTEPS / 4 + group, lane);
+                    if (group == GROUPS - 1) issue_contiguous_load(next_tile, wave, LOADS_PER_THREAD - 1, lane);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -509,47 +540,41 @@ __device__ __forceinline__ bool walk_tiles(RowState& state, const bf16x8 (&qf)[K
     // Drain the query loads here: a wait for them inside the loop would also
     // wait for the tile prefetch that is kept in flight there.
     wait_vector_memory<0>();
-    issue_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, last_token, wave, lane);
+    issue_tile(locate_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, last_token, wave, true), keys,
+               wave);
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         unsigned char* stage = lds + (tile & 1) * STAGE_BYTES;
-        if (tile + 1 < tile_end) {
-            issue_tile(lds + ((tile + 1) & 1) * STAGE_BYTES, keys, (tile + 1) * BN, last_token, wave, lane);
-            wait_vector_memory<LOADS_PER_THREAD>();
-        } else {
-            wait_vector_memory<0>();
-        }
+        wait_vector_memory<0>();   // this tile was requested while the previous one was consumed
         workgroup_barrier();
         const int key0 = tile * BN;
         if (key0 + BN > tokens) {
             zero_tail_rows(stage, tokens - key0, tid);
             workgroup_barrier();
         }
-        process_tile<SAFE>(state, risk, qf, stage, key0, limit, wave_min_limit, tile == tile_begin, c, lane);
+        // The other stage was last read for tile-1, which every wave has left.
+        const TileSource next_tile = locate_tile(lds + ((tile + 1) & 1) * STAGE_BYTES, keys, (tile + 1) * BN, last_token,
+                                                 wave, tile + 1 < tile_end);
+        if (!next_tile.contiguous) issue_tile(next_tile, keys, wave);
+        process_tile<SAFE>(state, risk, qf, stage, key0, limit, wave_min_limit, tile == tile_begin, c, lane, next_tile,
+                           wave);
         workgroup_barrier();
     }
     return risk;
 }
 
-// Fast walk first; the rare workgroup in which some row outran the fixed
-// reference repeats the walk with the rescaling variant.  Each variant loads
-// its own copy of the query fragments so that the register allocation of the
-// fast loop does not have to carry them across the slow one.
-__device__ __forceinline__ void walk_tiles_checked(RowState& state, const bf16_t* query_latent_row,
-                                                   const bf16_t* query_rope_row, bool valid, unsigned char* lds,
-                                                   const KeyStream& keys, int tile_begin, int tile_end, int tokens,
-                                                   int limit, float c, int tid) {
-    const int g = (tid % 64) / 32;
-    bool risk;
-    {
-        bf16x8 qf[KSTEPS];
-        load_query(qf, query_latent_row, query_rope_row, valid, g);
-        risk = walk_tiles<false>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
-    }
-    if (__syncthreads_or(risk)) {
-        bf16x8 qf[KSTEPS];
-        load_query(qf, query_latent_row, query_rope_row, valid, g);
-        walk_tiles<true>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
-    }
+// Loads the query fragments of this lane's row and walks the tiles with one
+// variant.  Returns whether any wave of the workgroup reported overflow risk
+// (workgroup-uniform; always false for SAFE).
+template <bool SAFE>
+__device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_latent_row,
+                                          const bf16_t* query_rope_row, bool valid, unsigned char* lds,
+                                          const KeyStream& keys, int tile_begin, int tile_end, int tokens, int limit,
+                                          float c, int tid) {
+    bf16x8 qf[KSTEPS];
+    load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
+    const bool risk = walk_tiles<SAFE>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
+    if (SAFE) return false;
+    return __syncthreads_or(risk) != 0;
 }
 
 __device__ __forceinline__ int tiles_of(int length) {
@@ -595,6 +620,14 @@ struct DecodeSlots {
     float* partial_stats;    // [slots][H][2]  (max in log2 units, sum)
 };
 
+// SAFE == false is the kernel that does the work.  A workgroup in which some
+// row outran the fixed softmax reference (see process_tile) raises its flag
+// word instead of trusting its results; the SAFE == true instantiation,
+// launched right after, repeats exactly the flagged workgroups with the
+// rescaling variant and returns at once everywhere else.  Two kernels rather
+// than two paths in one keep the register allocation of the hot loop free of
+// the slow path's pressure.
+template <bool SAFE>
 __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query,
     const bf16_t* __restrict__ paged_kv_cache, const int* __restrict__ block_table,
@@ -611,7 +644,13 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     const int g = lane / 32;
     const int workgroup = blockIdx.x;
     const int head0 = blockIdx.y * ROWS;
-    const float c = scale * LOG2E;
+    const float c = uniform(scale * LOG2E);
+
+    // one flag word per workgroup, behind the partial-result slots (or at the start of
+    // the workspace when sequences are not cut and no slot is used)
+    const size_t slots = whole_sequences ? 0 : (size_t)workgroups + batch_size;
+    int* flag = reinterpret_cast<int*>(workspace + slots * heads * (RANK + 2)) + blockIdx.y * gridDim.x + workgroup;
+    if (SAFE && *flag == 0) return;
 
     const int total = scan_tiles(prefix, scratch, cache_lengths, batch_size, tid);
     int range_begin, range_end, sequence;
@@ -631,9 +670,11 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         }
         sequence = low;
     }
-    if (range_begin >= range_end) return;
+    if (range_begin >= range_end) {
+        if (!SAFE && tid == 0) *flag = 0;
+        return;
+    }
 
-    const size_t slots = (size_t)workgroups + batch_size;
     float* partial_output = workspace;
     float* partial_stats = workspace + slots * heads * RANK;
 
@@ -643,6 +684,7 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     unsigned char* wave_lds = lds + wave * 32 * EPILOGUE_PITCH;
 
     RowState state;
+    bool any_risk = false;
     int position = range_begin;
     while (position < range_end) {
         const int sequence_begin = prefix[sequence];
@@ -664,8 +706,10 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.rope_stride = WIDTH;
         keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
         keys.page_size = page_size;
-        walk_tiles_checked(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
-                           segment_end - sequence_begin, tokens, tokens, c, tid);
+        if (walk_rows<SAFE>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
+                            segment_end - sequence_begin, tokens, tokens, c, tid)) {
+            any_risk = true;
+        }
 
         const float total_sum = half_wave_sum(state.row_sum);
         if (wave_active) {
@@ -695,6 +739,7 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         position = segment_end;
         ++sequence;
     }
+    if (!SAFE && tid == 0) *flag = any_risk ? 1 : 0;
 }
 
 // Merge the partial results of every sequence that was cut by a range boundary.
@@ -774,7 +819,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
     const int wave = tid / 64;
     const int lq = lane % 32;
     const int g = lane / 32;
-    const float c = scale * LOG2E;
+    const float c = uniform(scale * LOG2E);
 
     // heaviest (latest) row blocks first
     const int batch = blockIdx.x / row_blocks;
@@ -799,8 +844,10 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
     keys.rope_stride = ROPE;
     keys.block_table = nullptr;
     keys.page_size = 0;
-    walk_tiles_checked(state, query_latent + global_row * RANK, query_rope + global_row * ROPE, valid, lds, keys, 0,
-                       tiles_of(visible), visible, token + 1, c, tid);
+    // This entry point is kept for interface parity at the reference's shapes; it
+    // always takes the rescaling variant, which needs no overflow fallback.
+    walk_rows<true>(state, query_latent + global_row * RANK, query_rope + global_row * ROPE, valid, lds, keys, 0,
+                    tiles_of(visible), visible, token + 1, c, tid);
 
     if (!wave_active) return;
     const float total_sum = half_wave_sum(state.row_sum);
@@ -845,21 +892,29 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
     }
     static thread_local bool prepared = false;
     if (!prepared) {
-        allow_large_lds(mla_decode_split_kernel);
+        allow_large_lds(mla_decode_split_kernel<false>);
+        allow_large_lds(mla_decode_split_kernel<true>);
         prepared = true;
     }
-    // Slots workgroups + batch must fit the B*H*splits*(C+2) workspace: with
-    // splits == 1 every sequence is finished by one workgroup and no slot is used.
+    // Workspace B*H*splits*(C+2) floats holds workgroups + batch partial-result
+    // slots of H*(C+2) floats and, behind them, one flag word per workgroup (the
+    // flags fit one more slot).  With splits == 1 every sequence is finished by
+    // one workgroup, no slot is used and the flags sit at the start.
     const int whole_sequences = splits == 1 ? 1 : 0;
     int workgroups = batch_size;
     if (!whole_sequences) {
-        const long long by_workspace = (long long)batch_size * (splits - 1);
-        workgroups = (int)std::min<long long>(compute_units(), by_workspace);
+        const long long by_workspace = (long long)batch_size * (splits - 1) - 1;
+        workgroups = (int)std::max<long long>(1, std::min<long long>(compute_units(), by_workspace));
     }
     const int head_groups = (heads + ROWS - 1) / ROWS;
-    hipLaunchKernelGGL(mla_decode_split_kernel, dim3(workgroups, head_groups), dim3(THREADS), LDS_BYTES, stream,
-                       output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
-                       heads, page_size, pages_per_sequence, workgroups, whole_sequences, scale);
+    const dim3 grid(workgroups, head_groups);
+    hipLaunchKernelGGL(mla_decode_split_kernel<false>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
+                       paged_kv_cache, block_table, cache_lengths, workspace, batch_size, heads, page_size,
+                       pages_per_sequence, workgroups, whole_sequences, scale);
+    HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(mla_decode_split_kernel<true>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
+                       paged_kv_cache, block_table, cache_lengths, workspace, batch_size, heads, page_size,
+                       pages_per_sequence, workgroups, whole_sequences, scale);
     HIP_CHECK(hipGetLastError());
     if (!whole_sequences) {
         hipLaunchKernelGGL(mla_decode_combine_kernel, dim3(heads, batch_size), dim3(128), 0, stream, output,

@@ -10,6 +10,7 @@ is an error, there is no fallback implementation.
 from __future__ import annotations
 
 import ctypes
+import os
 from pathlib import Path
 
 import torch
@@ -21,7 +22,11 @@ _LIBRARIES: dict[str, ctypes.CDLL] = {}
 
 
 def library_path(name: str) -> Path:
-    return ROOT / "build" / f"libdscuda_{name}_bench.so"
+    """``build/`` under the repository root, or the directory named by the
+    environment variable DSCUDA_AMD_LIBRARY_DIR."""
+    directory = os.environ.get("DSCUDA_AMD_LIBRARY_DIR")
+    base = Path(directory) if directory else ROOT / "build"
+    return base / f"libdscuda_{name}_bench.so"
 
 
 def library(name: str) -> ctypes.CDLL:
