@@ -334,6 +334,333 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Two-phase ("ping-pong") variant for long sequences, 8 waves = 2 per SIMD.
+//
+// A SIMD's matrix pipeline idles while its waves run the softmax, and with one
+// barrier per tile both waves of a SIMD run it at the same time.  Here every
+// wave alternates between two phases that end in a workgroup barrier:
+//     X(j): request later tiles, softmax of S(j) -> P(j)          (VALU, exp)
+//     Y(j): O += V(j)^T P(j), then S(j+1) = K(j+1) Q^T            (MFMA, LDS reads)
+// Waves 4..7 run one extra barrier before their first phase, so they are in X
+// while waves 0..3 (the other wave of each SIMD) are in Y and the reverse: the
+// matrix pipeline always has a wave feeding it.  Y raises its wave priority.
+//
+// Y is one stream of MFMAs (PV then QK), each with one A fragment from LDS.
+// Fragments go through a ring of RING registers sets that runs RING MFMAs
+// ahead of their use; the first RING fragments (of V(j)) are read at the end of
+// X(j), before the barrier, so that Y starts with its operands in registers.
+//
+// K tiles sit in a ring of three slots, V tiles in a ring of four.  A wave
+// requests K(j+2) and V(j+2) during X(j) and waits for its own requests at the
+// end of Y(j); the barrier that ends Y(j) of the later group publishes them.
+// K(j+2) is first read in Y(j+1), V(j+2) at the end of X(j+2); the slots they
+// overwrite (K(j-1), V(j-2)) were last read in Y(j-2).
+struct PingPong {
+    static constexpr int K_SLOTS = 3;
+    static constexpr int V_SLOTS = 4;
+    static constexpr int RING = 8;
+};
+
+template <int DQK, int DV>
+__global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
+    bf16_t* __restrict__ output, float* __restrict__ logsumexp,
+    const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
+    int sequence_length, int query_heads, int key_value_heads, int query_blocks, float scale) {
+    using C = FwdConfig<DQK, DV, 8>;
+    constexpr int BN = C::BN;
+    constexpr int KSTEPS = DQK / 16;
+    constexpr int DBLOCKS = DV / 32;
+    constexpr int SPAN = (C::K_ROW % 256 == 0) ? 16 : 8;   // chunk positions the K swizzle permutes
+    constexpr int KLOW = SPAN / 2;                          // k-steps with distinct swizzled addresses
+    constexpr int V_RING = PingPong::K_SLOTS * C::K_BYTES;  // byte offset of the V slots
+    constexpr int RING = PingPong::RING;
+    constexpr int PV_MFMAS = 4 * DBLOCKS;
+    constexpr int QK_MFMAS = 2 * KSTEPS;
+    constexpr int REQUESTS = C::K_LOADS_PER_WAVE + C::V_LOADS_PER_WAVE;
+    static_assert(REQUESTS <= 6, "X has six places for tile requests");
+    static_assert(PV_MFMAS >= RING, "the fragments read ahead in X must all belong to V");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int group = wave / 4;
+    const int lane = tid % 64;
+    const int lq = lane % 32;
+    const int g = lane / 32;
+
+    int bh, qb_rank;
+    xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, qb_rank);
+    const int qb = query_blocks - 1 - qb_rank;
+    const int b = bh / query_heads;
+    const int h = bh % query_heads;
+    const int hk = h / (query_heads / key_value_heads);
+    const int S = sequence_length;
+
+    const int q0 = qb * C::BM;
+    const int wave_q0 = q0 + 32 * wave;
+    const int q_row = wave_q0 + lq;
+
+    const size_t q_stride = (size_t)query_heads * DQK;
+    const unsigned k_stride_bytes = (unsigned)key_value_heads * DQK * 2;
+    const unsigned v_stride_bytes = (unsigned)key_value_heads * DV * 2;
+    const bf16_t* q_base = query + ((size_t)b * S * query_heads + h) * DQK;
+    const unsigned char* k_base =
+        reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * key_value_heads + hk) * DQK);
+    const unsigned char* v_base =
+        reinterpret_cast<const unsigned char*>(value + ((size_t)b * S * key_value_heads + hk) * DV);
+
+    bf16x8 qf[KSTEPS];
+    {
+        const bool valid = q_row < S;
+        const bf16_t* row = q_base + (size_t)(valid ? q_row : 0) * q_stride + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 bits = {0, 0, 0, 0};
+            if (valid) {
+                bits = *reinterpret_cast<const u32x4*>(row + 16 * ks);
+            }
+            qf[ks] = __builtin_bit_cast(bf16x8, bits);
+        }
+    }
+
+    const int last_key = min(S, q0 + C::BM) - 1;
+    const int tiles = last_key / BN + 1;
+    const unsigned lds_base = lds_offset_of(lds);
+
+    // One 1 KB piece (index `part` of this wave's share) of the K and V tiles
+    // `tile`: parts 0..K_LOADS_PER_WAVE-1 belong to K, the rest to V.
+    auto request_part = [&](int tile, int k_slot, int v_slot, int part) {
+        const int key0 = tile * BN;
+        const int row_limit = S - 1 - key0;
+        if (part < C::K_LOADS_PER_WAVE) {
+            const unsigned char* k_tile = k_base + (size_t)key0 * k_stride_bytes;
+            const int load = wave * C::K_LOADS_PER_WAVE + part;
+            const int position = 64 * load + lane;
+            const int row = position / C::K_CHUNKS;
+            const int chunk = (position % C::K_CHUNKS) ^ C::k_swizzle(row);
+            const unsigned offset = (unsigned)min(row, row_limit) * k_stride_bytes + 16u * chunk;
+            direct_load_16_offset(k_tile, offset, lds_base + k_slot * C::K_BYTES + load * 1024);
+        } else {
+            const unsigned char* v_tile = v_base + (size_t)key0 * v_stride_bytes;
+            const int load = wave * C::V_LOADS_PER_WAVE + (part - C::K_LOADS_PER_WAVE);
+            const int position = 64 * load + lane;
+            const int row = position / C::V_CHUNKS;
+            const int chunk = (position % C::V_CHUNKS) ^ (C::v_flip(row) << 2);
+            const unsigned offset = (unsigned)min(row, row_limit) * v_stride_bytes + 16u * chunk;
+            direct_load_16_offset(v_tile, offset, lds_base + V_RING + v_slot * C::V_BYTES + load * 1024);
+        }
+    };
+
+    // Per-lane byte offsets of the fragment reads inside a slot.  K: chunk
+    // 2*ks + g of row lq sits at position (2*ks + g) ^ swizzle; the XOR only
+    // touches the low bits, so KLOW addresses plus immediates cover all k-steps.
+    unsigned k_read[KLOW];
+    {
+        const int t = g ^ C::k_swizzle(lq);
+#pragma unroll
+        for (int i = 0; i < KLOW; ++i) k_read[i] = lq * C::K_ROW + 16 * ((2 * i) ^ t);
+    }
+    unsigned v_read[DBLOCKS];
+    {
+        const int s16 = lane % 16;
+        const int v_row = 4 * g + s16 / 4;
+        const int in_group = 32 * ((lane / 16) % 2) + 8 * (s16 % 4);
+#pragma unroll
+        for (int d = 0; d < DBLOCKS; ++d) v_read[d] = v_row * C::V_ROW + 64 * (d ^ C::v_flip(v_row)) + in_group;
+    }
+    auto k_fragment = [&](const unsigned char* k_tile, int ks, int mb) -> bf16x8 {
+        return *reinterpret_cast<const bf16x8*>(k_tile + k_read[ks % KLOW] + (ks / KLOW) * (SPAN * 16) +
+                                                mb * 32 * C::K_ROW);
+    };
+    auto v_fragment = [&](const unsigned char* v_tile, int n, int d) -> bf16x8 {
+        const unsigned char* first = v_tile + v_read[d] + n * 16 * C::V_ROW;
+        const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)first);
+        const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(first + 8 * C::V_ROW));
+        return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    // fragment i of the Y stream: PV_MFMAS fragments of V (16-key step i / DBLOCKS,
+    // column block i % DBLOCKS), then QK_MFMAS fragments of K (k-step, key half)
+    auto stream_fragment = [&](const unsigned char* v_tile, const unsigned char* k_tile, int i) -> bf16x8 {
+        if (i < PV_MFMAS) {
+            return v_fragment(v_tile, i / DBLOCKS, i % DBLOCKS);
+        }
+        return k_fragment(k_tile, (i - PV_MFMAS) / 2, (i - PV_MFMAS) % 2);
+    };
+
+    f32x16 o_acc[DBLOCKS];
+#pragma unroll
+    for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[d][i] = 0.f;
+    }
+    f32x16 s_acc[2];
+    bf16x8 pf[4];
+    bf16x8 ring[RING];
+    float row_max = -INFINITY;
+    float row_sum = 0.f;
+    const float c = scale * LOG2E;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // ---- prologue: tiles 0 and 1, S(0); then the phase shift
+    wait_vector_memory<0>();   // the query loads
+#pragma unroll
+    for (int part = 0; part < REQUESTS; ++part) request_part(0, 0, 0, part);
+    if (tiles > 1) {
+#pragma unroll
+        for (int part = 0; part < REQUESTS; ++part) request_part(1, 1, 1, part);
+    }
+    wait_vector_memory<0>();
+    workgroup_barrier();
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_fragment(lds, ks, mb), qf[ks],
+                                                                ks == 0 ? zero : s_acc[mb], 0, 0, 0);
+        }
+    }
+    if (group == 1) {
+        workgroup_barrier();
+    }
+
+    int k_slot = 0;      // tile % 3
+    for (int tile = 0; tile < tiles; ++tile) {
+        const int k_slot1 = k_slot == 2 ? 0 : k_slot + 1;
+        const int k_slot2 = k_slot1 == 2 ? 0 : k_slot1 + 1;
+        const int v_slot = tile & 3;
+        const int v_slot2 = (tile + 2) & 3;
+        const int key0 = tile * BN;
+        // Past the last tile the requests repeat it: the slots they land in are dead.
+        const int request_tile = min(tile + 2, tiles - 1);
+        const unsigned char* k_tile = lds + k_slot1 * C::K_BYTES;           // K(tile + 1)
+        const unsigned char* v_tile = lds + V_RING + v_slot * C::V_BYTES;   // V(tile)
+
+        // ================= X: softmax with the requests for tile + 2 spread through it =================
+        // A wave whose rows all lie before this tile runs it like any other: the
+        // mask turns its scores into zeros, and the phases are barrier-locked, so
+        // skipping would not end the tile sooner.
+        auto request_next = [&](int part) {
+            if (part < REQUESTS) {
+                request_part(request_tile, k_slot2, v_slot2, part);
+            }
+        };
+        request_next(0);
+        if (key0 + BN - 1 > wave_q0) {  // tile reaches past this wave's first row
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int k = key0 + 32 * mb + 8 * (i / 4) + 4 * g + (i % 4);
+                    if (k > q_row) s_acc[mb][i] = -INFINITY;
+                }
+            }
+        }
+        float tile_max = s_acc[0][0];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tile_max = fmaxf(tile_max, s_acc[mb][i]);
+        }
+        tile_max = half_wave_max(tile_max);
+        // lazy reference point, as in the single-phase kernel
+        const float new_max = fmaxf(row_max, tile_max);
+        const bool grew = (new_max - row_max) * c > 8.0f;
+        if (__any(grew)) {
+            const float alpha = __builtin_amdgcn_exp2f((row_max - new_max) * c);
+            row_max = new_max;
+            row_sum *= alpha;
+#pragma unroll
+            for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o_acc[d][i] *= alpha;
+            }
+        }
+        request_next(1);
+        {
+            const float offset = row_max * c;
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+                u32x4 packed;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = 8 * (n % 2) + 2 * j;
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[n / 2][i], c, -offset));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[n / 2][i + 1], c, -offset));
+                    row_sum += p0 + p1;   // unrounded: the logsumexp tolerance leaves no room for bf16 sums
+                    packed[j] = pack_bf16(p0, p1);
+                }
+                pf[n] = __builtin_bit_cast(bf16x8, packed);
+                request_next(2 + n);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RING; ++i) ring[i] = stream_fragment(v_tile, k_tile, i);
+        workgroup_barrier();
+
+        // ================= Y: O += V^T P, next S =================
+        __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+        for (int i = 0; i < PV_MFMAS + QK_MFMAS; ++i) {
+            if (i < PV_MFMAS) {
+                o_acc[i % DBLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], pf[i / DBLOCKS],
+                                                                             o_acc[i % DBLOCKS], 0, 0, 0);
+            } else {
+                const int ks = (i - PV_MFMAS) / 2;
+                const int mb = (i - PV_MFMAS) % 2;
+                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], qf[ks],
+                                                                    ks == 0 ? zero : s_acc[mb], 0, 0, 0);
+            }
+            if (i + RING < PV_MFMAS + QK_MFMAS) {
+                ring[i % RING] = stream_fragment(v_tile, k_tile, i + RING);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_s_setprio(0);
+        wait_vector_memory<0>();   // this wave's requests of X(tile)
+        workgroup_barrier();
+        k_slot = k_slot1;
+    }
+    if (group == 0) {
+        workgroup_barrier();
+    }
+
+    // ---- epilogue: every wave is past its last tile read
+    const float total = half_wave_sum(row_sum);
+    const float inverse = 1.0f / total;
+    if (g == 0 && q_row < S) {
+        logsumexp[((size_t)b * query_heads + h) * S + q_row] = row_max * scale + __logf(total);
+    }
+    unsigned char* o_lds = lds + (32 * wave) * C::O_PITCH;
+#pragma unroll
+    for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            u32x2 packed;
+            packed.x = pack_bf16(o_acc[d][4 * i4 + 0] * inverse, o_acc[d][4 * i4 + 1] * inverse);
+            packed.y = pack_bf16(o_acc[d][4 * i4 + 2] * inverse, o_acc[d][4 * i4 + 3] * inverse);
+            const int dv = 32 * d + 8 * i4 + 4 * g;
+            *reinterpret_cast<u32x2*>(o_lds + lq * C::O_PITCH + 2 * dv) = packed;
+        }
+    }
+    __syncthreads();
+    constexpr int ROW_CHUNKS = DV / 8;
+    constexpr int ROWS_PER_PASS = 64 / ROW_CHUNKS;
+    const size_t o_stride = (size_t)query_heads * DV;
+    bf16_t* o_base = output + ((size_t)b * S * query_heads + h) * DV;
+#pragma unroll
+    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+        const int row = pass * ROWS_PER_PASS + lane / ROW_CHUNKS;
+        const int chunk = lane % ROW_CHUNKS;
+        const int q = wave_q0 + row;
+        if (q < S) {
+            const u32x4 bits = *reinterpret_cast<const u32x4*>(o_lds + row * C::O_PITCH + 16 * chunk);
+            *reinterpret_cast<u32x4*>(o_base + (size_t)q * o_stride + 8 * chunk) = bits;
+        }
+    }
+}
+
 template <int DQK, int DV, int NWAVES>
 void launch_forward(bf16_t* output, float* logsumexp, const bf16_t* query, const bf16_t* key, const bf16_t* value,
                     int batch_size, int sequence_length, int query_heads, int key_value_heads, float scale,
@@ -363,6 +690,33 @@ void launch_forward(bf16_t* output, float* logsumexp, const bf16_t* query, const
     HIP_CHECK(hipGetLastError());
 }
 
+template <int DQK, int DV>
+void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* query, const bf16_t* key,
+                             const bf16_t* value, int batch_size, int sequence_length, int query_heads,
+                             int key_value_heads, float scale, hipStream_t stream) {
+    using C = FwdConfig<DQK, DV, 8>;
+    constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES;
+    static_assert(LDS_BYTES >= C::O_BYTES && LDS_BYTES <= 160 * 1024, "the tile slots must hold the O staging and fit the LDS");
+    const int query_blocks = (sequence_length + C::BM - 1) / C::BM;
+    const long long grid = (long long)batch_size * query_heads * query_blocks;
+    if (grid > 0x7fffffffLL) {
+        throw std::invalid_argument("attention forward: batch*heads*query_blocks exceeds the grid limit");
+    }
+    if ((long long)key_value_heads * (DQK > DV ? DQK : DV) * 2 * C::BN > 0x7fffffffLL) {
+        throw std::invalid_argument("attention forward: key_value_heads * head size is too large");
+    }
+    auto kernel = attention_forward_pingpong_kernel<DQK, DV>;
+    static thread_local bool raised = false;
+    if (!raised) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::THREADS), LDS_BYTES, stream, output, logsumexp, query,
+                       key, value, sequence_length, query_heads, key_value_heads, query_blocks, scale);
+    HIP_CHECK(hipGetLastError());
+}
+
 }  // namespace
 
 void attention_forward_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, const bf16_t* key,
@@ -377,8 +731,8 @@ void attention_forward_dispatch(bf16_t* output, float* logsumexp, const bf16_t* 
     if (qk_head_size == DQK && v_head_size == DV) {                                                               \
         if constexpr (DV >= 128) {                                                                                \
             if (large) {                                                                                          \
-                launch_forward<DQK, DV, 8>(output, logsumexp, query, key, value, batch_size, sequence_length,     \
-                                           query_heads, key_value_heads, scale, stream);                          \
+                launch_forward_pingpong<DQK, DV>(output, logsumexp, query, key, value, batch_size,               \
+                                                 sequence_length, query_heads, key_value_heads, scale, stream);   \
                 return;                                                                                           \
             }                                                                                                     \
         }                                                                                                         \

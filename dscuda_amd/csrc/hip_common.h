@@ -144,12 +144,24 @@ __device__ __forceinline__ int fresh_lane_id() {
 // XCD-aware work-item order.  Workgroups are handed to the 8 XCDs round-robin
 // by linear id; every XCD has a private L2.  Items are grouped so that the
 // `inner` items that share operands (the query blocks of one head) run on one
-// XCD back to back, and `outer` groups (heads) are dealt across XCDs.
+// XCD, and `outer` groups (heads) are dealt across XCDs.  Inside an XCD the
+// heads are taken two at a time and their items interleaved in inner order:
+// with items sorted from heavy to light (a causal triangle) the compute units
+// that got the light items of one pair pick up the heavy items of the next, so
+// the units finish together, while only two heads' operands are live in the L2.
 // Returns (outer index, inner index) for a linear workgroup id; falls back to
-// the plain order when `outer` is not a multiple of 8.
+// one head at a time when `outer` is a multiple of 8 but not of 16, and to the
+// plain order otherwise.
 __device__ __forceinline__ void xcd_order(int linear, int outer, int inner, int& outer_index, int& inner_index) {
     constexpr int XCDS = 8;
-    if (outer % XCDS == 0) {
+    if (outer % (2 * XCDS) == 0) {
+        const int xcd = linear % XCDS;
+        const int slot = linear / XCDS;
+        const int pair = slot / (2 * inner);
+        const int rest = slot % (2 * inner);
+        outer_index = xcd + XCDS * (2 * pair + rest % 2);
+        inner_index = rest / 2;
+    } else if (outer % XCDS == 0) {
         const int xcd = linear % XCDS;
         const int slot = linear / XCDS;
         outer_index = xcd + XCDS * (slot / inner);

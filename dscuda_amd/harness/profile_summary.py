@@ -1,0 +1,64 @@
+"""Condenses ``rocprofv3 --output-format csv`` output into the few lines worth
+keeping: per-kernel call count and average duration from a ``--kernel-trace
+--stats`` run, per-kernel counter averages from a ``--pmc`` run.
+
+    python3 dscuda_amd/harness/profile_summary.py --command "<what was run>" DIR [DIR ...]
+
+Every ``*_kernel_stats.csv`` and ``*_counter_collection.csv`` below each DIR is
+read; output is plain text on stdout.
+"""
+
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+from pathlib import Path
+
+
+def short_name(name: str) -> str:
+    name = name.replace("void ", "").replace("dscuda::(anonymous namespace)::", "")
+    cut = name.find("(")
+    return name if cut < 0 else name[:cut]
+
+
+def kernel_stats(path: Path) -> list[str]:
+    lines = [f"{'kernel':78s} {'calls':>6s} {'avg us':>10s} {'min us':>10s} {'max us':>10s} {'%':>6s}"]
+    with open(path, newline="") as handle:
+        for row in csv.DictReader(handle):
+            lines.append(f"{short_name(row['Name'])[:78]:78s} {int(row['Calls']):6d} "
+                         f"{float(row['AverageNs']) / 1e3:10.1f} {float(row['MinNs']) / 1e3:10.1f} "
+                         f"{float(row['MaxNs']) / 1e3:10.1f} {float(row['Percentage']):6.2f}")
+    return lines
+
+
+def counter_averages(path: Path) -> list[str]:
+    table = collections.defaultdict(lambda: collections.defaultdict(list))
+    with open(path, newline="") as handle:
+        for row in csv.DictReader(handle):
+            table[short_name(row["Kernel_Name"])][row["Counter_Name"]].append(float(row["Counter_Value"]))
+    lines = []
+    for kernel, counters in table.items():
+        lines.append(kernel[:100])
+        for counter, values in counters.items():
+            lines.append(f"    {counter:32s} {sum(values) / len(values):18.1f}   (mean of {len(values)} dispatches)")
+    return lines
+
+
+def main():
+    parser = argparse.ArgumentParser(description=__doc__)
+    parser.add_argument("--command", required=True, help="the profiled command line, recorded in the summary")
+    parser.add_argument("directories", nargs="+")
+    args = parser.parse_args()
+    print(f"command: {args.command}")
+    for directory in args.directories:
+        for path in sorted(Path(directory).rglob("*_kernel_stats.csv")):
+            print(f"\n[kernel trace] {path.name}")
+            print("\n".join(kernel_stats(path)))
+        for path in sorted(Path(directory).rglob("*_counter_collection.csv")):
+            print(f"\n[counters] {path.name}")
+            print("\n".join(counter_averages(path)))
+
+
+if __name__ == "__main__":
+    main()
