@@ -127,7 +127,7 @@ def main():
                                "0.5*N(0,1) seed 1, RoPE theta=10000, scale 1/sqrt(192)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
-                     "kernel": "attention_forward_kernel<192,128,8>", "kernel_ms": kernel_ms,
+                     "kernel": "attention_forward_pingpong_kernel<192,128>", "kernel_ms": kernel_ms,
                      "flops_per_launch": flops},
         "cpu_baseline": baseline,
         "parity": parity,

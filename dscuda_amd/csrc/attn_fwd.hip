@@ -47,6 +47,7 @@
 #include <cmath>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 
 namespace dscuda {
 namespace {
@@ -335,11 +336,14 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Two-phase ("ping-pong") variant for long sequences, 8 waves = 2 per SIMD.
+// Persistent two-phase ("ping-pong") variant for long sequences.
 //
-// A SIMD's matrix pipeline idles while its waves run the softmax, and with one
-// barrier per tile both waves of a SIMD run it at the same time.  Here every
-// wave alternates between two phases that end in a workgroup barrier:
+// One workgroup of 8 waves (2 per SIMD) per compute unit walks a list of work
+// items, an item being one block of 256 queries of one (batch, head).
+//
+// Phases.  A SIMD's matrix pipeline idles while its waves run the softmax, and
+// with one barrier per tile both waves of a SIMD run it at the same time.  Here
+// every wave alternates between two phases that end in a workgroup barrier:
 //     X(j): request later tiles, softmax of S(j) -> P(j)          (VALU, exp)
 //     Y(j): O += V(j)^T P(j), then S(j+1) = K(j+1) Q^T            (MFMA, LDS reads)
 // Waves 4..7 run one extra barrier before their first phase, so they are in X
@@ -347,26 +351,61 @@ __global__ __launch_bounds__(64 * NWAVES) void attention_forward_kernel(
 // matrix pipeline always has a wave feeding it.  Y raises its wave priority.
 //
 // Y is one stream of MFMAs (PV then QK), each with one A fragment from LDS.
-// Fragments go through a ring of RING registers sets that runs RING MFMAs
-// ahead of their use; the first RING fragments (of V(j)) are read at the end of
-// X(j), before the barrier, so that Y starts with its operands in registers.
+// Fragments go through a ring of RING register sets that runs RING MFMAs ahead
+// of their use; the first RING fragments (of V(j)) are read at the end of X(j),
+// before the barrier, so that Y starts with its operands in registers.
 //
-// K tiles sit in a ring of three slots, V tiles in a ring of four.  A wave
-// requests K(j+2) and V(j+2) during X(j) and waits for its own requests at the
-// end of Y(j); the barrier that ends Y(j) of the later group publishes them.
-// K(j+2) is first read in Y(j+1), V(j+2) at the end of X(j+2); the slots they
-// overwrite (K(j-1), V(j-2)) were last read in Y(j-2).
+// Tiles.  K tiles sit in a ring of three slots, V tiles in a ring of four, and
+// the tiles of all items of a workgroup form one stream: a wave requests stream
+// tile t+2 during X of stream tile t, whether it belongs to this item or to the
+// next one, and waits for its own requests at the end of that tile's Y; the
+// barrier that ends Y of the later group publishes them.  K(t+2) is first read
+// in Y(t+1), V(t+2) at the end of X(t+2); the slots they overwrite (K(t-1),
+// V(t-2)) were last read in Y(t-2).  So a new item finds its first two tiles in
+// LDS; what stays exposed at an item switch is the load of the new queries.
+//
+// Work order.  Workgroup w belongs to cluster w % 8 (workgroups are dealt
+// round-robin to the 8 XCDs, each with its own L2) and the (batch, head) pairs
+// are dealt to the clusters the same way.  Inside a cluster the items are laid
+// out two heads at a time, blocks from the heaviest (last) to the lightest, and
+// cut into rounds of one item per workgroup; odd rounds are handed out in
+// reverse, so a workgroup's heavy and light blocks add up to the same total
+// while the cluster works on two heads at any time.
 struct PingPong {
     static constexpr int K_SLOTS = 3;
     static constexpr int V_SLOTS = 4;
     static constexpr int RING = 8;
+    static constexpr int CLUSTERS = 8;
 };
+
+struct ForwardItem {
+    int batch_head;
+    int query_block;
+};
+
+// item `round` of workgroup `member` (of `members`) of a cluster that owns
+// `cluster_heads` (batch, head) pairs; false past the end of the list
+__device__ __forceinline__ bool forward_item(int round, int member, int members, int cluster, int clusters,
+                                             int cluster_heads, int query_blocks, ForwardItem& item) {
+    const int position = (round & 1) ? members - 1 - member : member;
+    const int index = round * members + position;
+    if (index >= cluster_heads * query_blocks) {
+        return false;
+    }
+    const int interleave = (cluster_heads % 2 == 0) ? 2 : 1;
+    const int group = index / (interleave * query_blocks);
+    const int rest = index % (interleave * query_blocks);
+    item.batch_head = cluster + clusters * (interleave * group + rest % interleave);
+    item.query_block = query_blocks - 1 - rest / interleave;
+    return true;
+}
 
 template <int DQK, int DV>
 __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
     bf16_t* __restrict__ output, float* __restrict__ logsumexp,
     const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
-    int sequence_length, int query_heads, int key_value_heads, int query_blocks, float scale) {
+    int sequence_length, int query_heads, int key_value_heads, int query_blocks, int batch_heads, int clusters,
+    float scale) {
     using C = FwdConfig<DQK, DV, 8>;
     constexpr int BN = C::BN;
     constexpr int KSTEPS = DQK / 16;
@@ -389,53 +428,42 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
-
-    int bh, qb_rank;
-    xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, qb_rank);
-    const int qb = query_blocks - 1 - qb_rank;
-    const int b = bh / query_heads;
-    const int h = bh % query_heads;
-    const int hk = h / (query_heads / key_value_heads);
     const int S = sequence_length;
 
-    const int q0 = qb * C::BM;
-    const int wave_q0 = q0 + 32 * wave;
-    const int q_row = wave_q0 + lq;
+    const int cluster = blockIdx.x % clusters;
+    const int member = blockIdx.x / clusters;
+    const int members = gridDim.x / clusters;
+    const int cluster_heads = batch_heads / clusters;
 
     const size_t q_stride = (size_t)query_heads * DQK;
+    const size_t o_stride = (size_t)query_heads * DV;
     const unsigned k_stride_bytes = (unsigned)key_value_heads * DQK * 2;
     const unsigned v_stride_bytes = (unsigned)key_value_heads * DV * 2;
-    const bf16_t* q_base = query + ((size_t)b * S * query_heads + h) * DQK;
-    const unsigned char* k_base =
-        reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * key_value_heads + hk) * DQK);
-    const unsigned char* v_base =
-        reinterpret_cast<const unsigned char*>(value + ((size_t)b * S * key_value_heads + hk) * DV);
-
-    bf16x8 qf[KSTEPS];
-    {
-        const bool valid = q_row < S;
-        const bf16_t* row = q_base + (size_t)(valid ? q_row : 0) * q_stride + 8 * g;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            u32x4 bits = {0, 0, 0, 0};
-            if (valid) {
-                bits = *reinterpret_cast<const u32x4*>(row + 16 * ks);
-            }
-            qf[ks] = __builtin_bit_cast(bf16x8, bits);
-        }
-    }
-
-    const int last_key = min(S, q0 + C::BM) - 1;
-    const int tiles = last_key / BN + 1;
     const unsigned lds_base = lds_offset_of(lds);
 
-    // One 1 KB piece (index `part` of this wave's share) of the K and V tiles
-    // `tile`: parts 0..K_LOADS_PER_WAVE-1 belong to K, the rest to V.
-    auto request_part = [&](int tile, int k_slot, int v_slot, int part) {
-        const int key0 = tile * BN;
+    // operands of an item
+    auto key_base = [&](const ForwardItem& item) {
+        const int b = item.batch_head / query_heads;
+        const int hk = (item.batch_head % query_heads) / (query_heads / key_value_heads);
+        return reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * key_value_heads + hk) * DQK);
+    };
+    auto value_base = [&](const ForwardItem& item) {
+        const int b = item.batch_head / query_heads;
+        const int hk = (item.batch_head % query_heads) / (query_heads / key_value_heads);
+        return reinterpret_cast<const unsigned char*>(value + ((size_t)b * S * key_value_heads + hk) * DV);
+    };
+    auto tile_count = [&](const ForwardItem& item) { return (min(S, (item.query_block + 1) * C::BM) - 1) / BN + 1; };
+
+    // One 1 KB piece (index `part` of this wave's share) of the K and V tiles that
+    // start at key `key0` of the head at (k_head, v_head): parts below
+    // K_LOADS_PER_WAVE belong to K, the rest to V.  Rows past the end of the
+    // sequence are clamped to the last one: such keys are invisible to every
+    // stored query, the data only has to be finite.
+    auto request_part = [&](const unsigned char* k_head, const unsigned char* v_head, int key0, int k_slot,
+                            int v_slot, int part) {
         const int row_limit = S - 1 - key0;
         if (part < C::K_LOADS_PER_WAVE) {
-            const unsigned char* k_tile = k_base + (size_t)key0 * k_stride_bytes;
+            const unsigned char* k_tile = k_head + (size_t)key0 * k_stride_bytes;
             const int load = wave * C::K_LOADS_PER_WAVE + part;
             const int position = 64 * load + lane;
             const int row = position / C::K_CHUNKS;
@@ -443,7 +471,7 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
             const unsigned offset = (unsigned)min(row, row_limit) * k_stride_bytes + 16u * chunk;
             direct_load_16_offset(k_tile, offset, lds_base + k_slot * C::K_BYTES + load * 1024);
         } else {
-            const unsigned char* v_tile = v_base + (size_t)key0 * v_stride_bytes;
+            const unsigned char* v_tile = v_head + (size_t)key0 * v_stride_bytes;
             const int load = wave * C::V_LOADS_PER_WAVE + (part - C::K_LOADS_PER_WAVE);
             const int position = 64 * load + lane;
             const int row = position / C::V_CHUNKS;
@@ -489,96 +517,144 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
         return k_fragment(k_tile, (i - PV_MFMAS) / 2, (i - PV_MFMAS) % 2);
     };
 
+    bf16x8 qf[KSTEPS];
     f32x16 o_acc[DBLOCKS];
-#pragma unroll
-    for (int d = 0; d < DBLOCKS; ++d) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[d][i] = 0.f;
-    }
     f32x16 s_acc[2];
     bf16x8 pf[4];
     bf16x8 ring[RING];
-    float row_max = -INFINITY;
-    float row_sum = 0.f;
+    float row_max, row_sum;
     const float c = scale * LOG2E;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: tiles 0 and 1, S(0); then the phase shift
-    wait_vector_memory<0>();   // the query loads
+    // Q fragments of an item (B operand: column = query lq, k = 16*ks + 8*g + j)
+    auto load_queries = [&](const ForwardItem& item) {
+        const int row_index = item.query_block * C::BM + 32 * wave + lq;
+        const bool valid = row_index < S;
+        const int b = item.batch_head / query_heads;
+        const int h = item.batch_head % query_heads;
+        const bf16_t* row = query + ((size_t)b * S * query_heads + h) * DQK + (size_t)(valid ? row_index : 0) * q_stride + 8 * g;
 #pragma unroll
-    for (int part = 0; part < REQUESTS; ++part) request_part(0, 0, 0, part);
-    if (tiles > 1) {
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 bits = {0, 0, 0, 0};
+            if (valid) {
+                bits = *reinterpret_cast<const u32x4*>(row + 16 * ks);
+            }
+            qf[ks] = __builtin_bit_cast(bf16x8, bits);
+        }
+    };
+
+    ForwardItem item, next_item;
+    if (!forward_item(0, member, members, cluster, clusters, cluster_heads, query_blocks, item)) {
+        return;   // uniform over the workgroup
+    }
+    bool has_next = forward_item(1, member, members, cluster, clusters, cluster_heads, query_blocks, next_item);
+
+    // ---- prologue of the first item: its queries and its tiles 0 and 1
+    load_queries(item);
+    wait_vector_memory<0>();
+    {
+        const unsigned char* k_head = key_base(item);
+        const unsigned char* v_head = value_base(item);
 #pragma unroll
-        for (int part = 0; part < REQUESTS; ++part) request_part(1, 1, 1, part);
+        for (int part = 0; part < REQUESTS; ++part) request_part(k_head, v_head, 0, 0, 0, part);
+#pragma unroll
+        for (int part = 0; part < REQUESTS; ++part) request_part(k_head, v_head, BN, 1, 1, part);
     }
     wait_vector_memory<0>();
     workgroup_barrier();
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_fragment(lds, ks, mb), qf[ks],
-                                                                ks == 0 ? zero : s_acc[mb], 0, 0, 0);
-        }
-    }
-    if (group == 1) {
-        workgroup_barrier();
-    }
 
-    int k_slot = 0;      // tile % 3
-    for (int tile = 0; tile < tiles; ++tile) {
-        const int k_slot1 = k_slot == 2 ? 0 : k_slot + 1;
-        const int k_slot2 = k_slot1 == 2 ? 0 : k_slot1 + 1;
-        const int v_slot = tile & 3;
-        const int v_slot2 = (tile + 2) & 3;
-        const int key0 = tile * BN;
-        // Past the last tile the requests repeat it: the slots they land in are dead.
-        const int request_tile = min(tile + 2, tiles - 1);
-        const unsigned char* k_tile = lds + k_slot1 * C::K_BYTES;           // K(tile + 1)
-        const unsigned char* v_tile = lds + V_RING + v_slot * C::V_BYTES;   // V(tile)
+    int k_slot = 0;     // slot of K of the current stream tile (stream index % 3)
+    int v_slot = 0;     // slot of V of the current stream tile (stream index % 4)
+    int round = 0;
+    bool shifted = false;
+    while (true) {
+        const int tiles = tile_count(item);
+        const int wave_q0 = item.query_block * C::BM + 32 * wave;
+        const int q_row = wave_q0 + lq;
+        const unsigned char* k_head = key_base(item);
+        const unsigned char* v_head = value_base(item);
+        const unsigned char* next_k_head = has_next ? key_base(next_item) : k_head;
+        const unsigned char* next_v_head = has_next ? value_base(next_item) : v_head;
 
-        // ================= X: softmax with the requests for tile + 2 spread through it =================
-        // A wave whose rows all lie before this tile runs it like any other: the
-        // mask turns its scores into zeros, and the phases are barrier-locked, so
-        // skipping would not end the tile sooner.
-        auto request_next = [&](int part) {
-            if (part < REQUESTS) {
-                request_part(request_tile, k_slot2, v_slot2, part);
-            }
-        };
-        request_next(0);
-        if (key0 + BN - 1 > wave_q0) {  // tile reaches past this wave's first row
+        // S(0) of the item; its K tile was requested two tiles ago
+        {
+            const unsigned char* k_tile = lds + k_slot * C::K_BYTES;
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
+            for (int ks = 0; ks < KSTEPS; ++ks) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int k = key0 + 32 * mb + 8 * (i / 4) + 4 * g + (i % 4);
-                    if (k > q_row) s_acc[mb][i] = -INFINITY;
+                for (int mb = 0; mb < 2; ++mb) {
+                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_fragment(k_tile, ks, mb), qf[ks],
+                                                                        ks == 0 ? zero : s_acc[mb], 0, 0, 0);
                 }
             }
         }
-        float tile_max = s_acc[0][0];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int d = 0; d < DBLOCKS; ++d) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) tile_max = fmaxf(tile_max, s_acc[mb][i]);
+            for (int i = 0; i < 16; ++i) o_acc[d][i] = 0.f;
         }
-        tile_max = half_wave_max(tile_max);
-        // lazy reference point, as in the single-phase kernel
-        const float new_max = fmaxf(row_max, tile_max);
-        const bool grew = (new_max - row_max) * c > 8.0f;
-        if (__any(grew)) {
-            const float alpha = __builtin_amdgcn_exp2f((row_max - new_max) * c);
-            row_max = new_max;
-            row_sum *= alpha;
-#pragma unroll
-            for (int d = 0; d < DBLOCKS; ++d) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o_acc[d][i] *= alpha;
+        row_max = -INFINITY;
+        row_sum = 0.f;
+        if (!shifted) {
+            shifted = true;
+            if (group == 1) {
+                workgroup_barrier();
             }
         }
-        request_next(1);
-        {
+
+        // X(tile): softmax with the requests for stream tile + 2 spread through it.
+        // A wave whose rows all lie before this tile runs it like any other: the
+        // mask turns its scores into zeros, and the phases are barrier-locked, so
+        // skipping would not end the tile sooner.  (Branching around the
+        // arithmetic of such tiles was tried: the extra control flow made the
+        // register allocator spill some 200 registers.)
+        auto phase_x = [&](int tile) {
+            const int key0 = tile * BN;
+            const int k_slot2 = k_slot == 0 ? 2 : k_slot - 1;      // (slot + 2) % 3
+            const int v_slot2 = (v_slot + 2) & 3;
+            const bool from_next = tile + 2 >= tiles;
+            const unsigned char* request_k = from_next ? next_k_head : k_head;
+            const unsigned char* request_v = from_next ? next_v_head : v_head;
+            const int request_key0 = (from_next ? tile + 2 - tiles : tile + 2) * BN;
+            auto request_next = [&](int part) {
+                if (part < REQUESTS) {
+                    request_part(request_k, request_v, request_key0, k_slot2, v_slot2, part);
+                }
+            };
+            request_next(0);
+            if (key0 + BN - 1 > wave_q0) {  // tile reaches past this wave's first row
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int k = key0 + 32 * mb + 8 * (i / 4) + 4 * g + (i % 4);
+                        if (k > q_row) s_acc[mb][i] = -INFINITY;
+                    }
+                }
+            }
+            float tile_max = s_acc[0][0];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) tile_max = fmaxf(tile_max, s_acc[mb][i]);
+            }
+            tile_max = half_wave_max(tile_max);
+            // The reference point only moves when some row's maximum grew by
+            // more than 2^8 in the exponent; until then probabilities may
+            // exceed one, which fp32 sums and bf16 operands hold without loss.
+            const float new_max = fmaxf(row_max, tile_max);
+            const bool grew = (new_max - row_max) * c > 8.0f;
+            if (__any(grew)) {
+                const float alpha = __builtin_amdgcn_exp2f((row_max - new_max) * c);
+                row_max = new_max;
+                row_sum *= alpha;
+#pragma unroll
+                for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o_acc[d][i] *= alpha;
+                }
+            }
+            request_next(1);
             const float offset = row_max * c;
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
@@ -594,70 +670,90 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                 pf[n] = __builtin_bit_cast(bf16x8, packed);
                 request_next(2 + n);
             }
-        }
+        };
+        // Y(tile): O += V^T P, and with FULL the next S.  The first RING fragments
+        // are read before the barrier that separates X from Y.
+        auto phase_y = [&](auto full_tag) {
+            constexpr bool FULL = decltype(full_tag)::value;
+            constexpr int COUNT = FULL ? PV_MFMAS + QK_MFMAS : PV_MFMAS;
+            const int k_slot1 = k_slot == 2 ? 0 : k_slot + 1;
+            const unsigned char* k_tile = lds + k_slot1 * C::K_BYTES;           // K(tile + 1)
+            const unsigned char* v_tile = lds + V_RING + v_slot * C::V_BYTES;   // V(tile)
 #pragma unroll
-        for (int i = 0; i < RING; ++i) ring[i] = stream_fragment(v_tile, k_tile, i);
-        workgroup_barrier();
+            for (int i = 0; i < RING; ++i) ring[i] = stream_fragment(v_tile, k_tile, i);
+            workgroup_barrier();
+            __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+            for (int i = 0; i < COUNT; ++i) {
+                if (i < PV_MFMAS) {
+                    o_acc[i % DBLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], pf[i / DBLOCKS],
+                                                                                 o_acc[i % DBLOCKS], 0, 0, 0);
+                } else {
+                    const int ks = (i - PV_MFMAS) / 2;
+                    const int mb = (i - PV_MFMAS) % 2;
+                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], qf[ks],
+                                                                        ks == 0 ? zero : s_acc[mb], 0, 0, 0);
+                }
+                if (i + RING < COUNT) {
+                    ring[i % RING] = stream_fragment(v_tile, k_tile, i + RING);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            __builtin_amdgcn_s_setprio(0);
+            wait_vector_memory<0>();   // this wave's requests of X(tile)
+            workgroup_barrier();
+            k_slot = k_slot1;
+            v_slot = (v_slot + 1) & 3;
+        };
 
-        // ================= Y: O += V^T P, next S =================
-        __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-        for (int i = 0; i < PV_MFMAS + QK_MFMAS; ++i) {
-            if (i < PV_MFMAS) {
-                o_acc[i % DBLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], pf[i / DBLOCKS],
-                                                                             o_acc[i % DBLOCKS], 0, 0, 0);
-            } else {
-                const int ks = (i - PV_MFMAS) / 2;
-                const int mb = (i - PV_MFMAS) % 2;
-                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % RING], qf[ks],
-                                                                    ks == 0 ? zero : s_acc[mb], 0, 0, 0);
-            }
-            if (i + RING < PV_MFMAS + QK_MFMAS) {
-                ring[i % RING] = stream_fragment(v_tile, k_tile, i + RING);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+        for (int tile = 0; tile + 1 < tiles; ++tile) {
+            phase_x(tile);
+            phase_y(std::true_type{});
         }
-        __builtin_amdgcn_s_setprio(0);
-        wait_vector_memory<0>();   // this wave's requests of X(tile)
-        workgroup_barrier();
-        k_slot = k_slot1;
+        // Last tile: the query registers are free from here on, the next item's
+        // queries load while this tile finishes.
+        phase_x(tiles - 1);
+        const float total = half_wave_sum(row_sum);
+        const float lse_value = row_max * scale + __logf(total);
+        const int store_row = q_row;
+        const int store_batch_head = item.batch_head;
+        if (has_next) {
+            load_queries(next_item);
+        }
+        phase_y(std::false_type{});
+
+        // ---- epilogue: normalise and store straight from the accumulators.  A
+        // lane holds 4 consecutive d_v of one query per (d, i4): 8-byte stores.
+        {
+            const float inverse = 1.0f / total;
+            const int b = store_batch_head / query_heads;
+            const int h = store_batch_head % query_heads;
+            if (store_row < S) {
+                if (g == 0) {
+                    logsumexp[((size_t)b * query_heads + h) * S + store_row] = lse_value;
+                }
+                bf16_t* o_row = output + ((size_t)b * S * query_heads + h) * DV + (size_t)store_row * o_stride;
+#pragma unroll
+                for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        u32x2 packed;
+                        packed.x = pack_bf16(o_acc[d][4 * i4 + 0] * inverse, o_acc[d][4 * i4 + 1] * inverse);
+                        packed.y = pack_bf16(o_acc[d][4 * i4 + 2] * inverse, o_acc[d][4 * i4 + 3] * inverse);
+                        *reinterpret_cast<u32x2*>(o_row + 32 * d + 8 * i4 + 4 * g) = packed;
+                    }
+                }
+            }
+        }
+        if (!has_next) {
+            break;
+        }
+        item = next_item;
+        ++round;
+        has_next = forward_item(round + 1, member, members, cluster, clusters, cluster_heads, query_blocks, next_item);
     }
     if (group == 0) {
         workgroup_barrier();
-    }
-
-    // ---- epilogue: every wave is past its last tile read
-    const float total = half_wave_sum(row_sum);
-    const float inverse = 1.0f / total;
-    if (g == 0 && q_row < S) {
-        logsumexp[((size_t)b * query_heads + h) * S + q_row] = row_max * scale + __logf(total);
-    }
-    unsigned char* o_lds = lds + (32 * wave) * C::O_PITCH;
-#pragma unroll
-    for (int d = 0; d < DBLOCKS; ++d) {
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-            u32x2 packed;
-            packed.x = pack_bf16(o_acc[d][4 * i4 + 0] * inverse, o_acc[d][4 * i4 + 1] * inverse);
-            packed.y = pack_bf16(o_acc[d][4 * i4 + 2] * inverse, o_acc[d][4 * i4 + 3] * inverse);
-            const int dv = 32 * d + 8 * i4 + 4 * g;
-            *reinterpret_cast<u32x2*>(o_lds + lq * C::O_PITCH + 2 * dv) = packed;
-        }
-    }
-    __syncthreads();
-    constexpr int ROW_CHUNKS = DV / 8;
-    constexpr int ROWS_PER_PASS = 64 / ROW_CHUNKS;
-    const size_t o_stride = (size_t)query_heads * DV;
-    bf16_t* o_base = output + ((size_t)b * S * query_heads + h) * DV;
-#pragma unroll
-    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
-        const int row = pass * ROWS_PER_PASS + lane / ROW_CHUNKS;
-        const int chunk = lane % ROW_CHUNKS;
-        const int q = wave_q0 + row;
-        if (q < S) {
-            const u32x4 bits = *reinterpret_cast<const u32x4*>(o_lds + row * C::O_PITCH + 16 * chunk);
-            *reinterpret_cast<u32x4*>(o_base + (size_t)q * o_stride + 8 * chunk) = bits;
-        }
     }
 }
 
@@ -696,14 +792,28 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
                              int key_value_heads, float scale, hipStream_t stream) {
     using C = FwdConfig<DQK, DV, 8>;
     constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES;
-    static_assert(LDS_BYTES >= C::O_BYTES && LDS_BYTES <= 160 * 1024, "the tile slots must hold the O staging and fit the LDS");
+    static_assert(LDS_BYTES <= 160 * 1024, "the tile slots must fit the LDS");
     const int query_blocks = (sequence_length + C::BM - 1) / C::BM;
-    const long long grid = (long long)batch_size * query_heads * query_blocks;
-    if (grid > 0x7fffffffLL) {
-        throw std::invalid_argument("attention forward: batch*heads*query_blocks exceeds the grid limit");
+    const long long batch_heads = (long long)batch_size * query_heads;
+    if (batch_heads * query_blocks > 0x7fffffffLL) {
+        throw std::invalid_argument("attention forward: batch*heads*query_blocks exceeds the item limit");
     }
     if ((long long)key_value_heads * (DQK > DV ? DQK : DV) * 2 * C::BN > 0x7fffffffLL) {
         throw std::invalid_argument("attention forward: key_value_heads * head size is too large");
+    }
+    // one workgroup per compute unit (the LDS footprint admits no second one)
+    static thread_local int compute_units = 0;
+    if (compute_units == 0) {
+        int device = 0;
+        HIP_CHECK(hipGetDevice(&device));
+        HIP_CHECK(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
+    }
+    const int clusters = (batch_heads % PingPong::CLUSTERS == 0 && compute_units >= PingPong::CLUSTERS)
+                             ? PingPong::CLUSTERS : 1;
+    long long grid = compute_units / clusters * clusters;
+    const long long items_per_cluster = batch_heads / clusters * query_blocks;
+    if (grid / clusters > items_per_cluster) {
+        grid = items_per_cluster * clusters;
     }
     auto kernel = attention_forward_pingpong_kernel<DQK, DV>;
     static thread_local bool raised = false;
@@ -713,7 +823,8 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
         raised = true;
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::THREADS), LDS_BYTES, stream, output, logsumexp, query,
-                       key, value, sequence_length, query_heads, key_value_heads, query_blocks, scale);
+                       key, value, sequence_length, query_heads, key_value_heads, query_blocks, (int)batch_heads,
+                       clusters, scale);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -726,7 +837,8 @@ void attention_forward_dispatch(bf16_t* output, float* logsumexp, const bf16_t* 
     // Few, large workgroups (256 queries) when there is enough work to fill the
     // chip; 128-query workgroups otherwise so that short problems still spread.
     const long long rows = (long long)batch_size * query_heads * sequence_length;
-    const bool large = rows >= 256LL * 256 * 2;
+    // the persistent kernel streams two tiles ahead across items: every item needs two tiles
+    const bool large = rows >= 256LL * 256 * 2 && sequence_length >= 128;
 #define DSCUDA_FWD_CASE(DQK, DV)                                                                                  \
     if (qk_head_size == DQK && v_head_size == DV) {                                                               \
         if constexpr (DV >= 128) {                                                                                \

@@ -17,25 +17,33 @@ from pathlib import Path
 
 
 def short_name(name: str) -> str:
-    name = name.replace("void ", "").replace("dscuda::(anonymous namespace)::", "")
+    name = name.replace("void ", "").replace("(anonymous namespace)::", "").replace("dscuda::", "")
     cut = name.find("(")
     return name if cut < 0 else name[:cut]
 
 
-def kernel_stats(path: Path) -> list[str]:
+def wanted(name: str, patterns: list[str]) -> bool:
+    return not patterns or any(pattern in name for pattern in patterns)
+
+
+def kernel_stats(path: Path, patterns: list[str]) -> list[str]:
     lines = [f"{'kernel':78s} {'calls':>6s} {'avg us':>10s} {'min us':>10s} {'max us':>10s} {'%':>6s}"]
     with open(path, newline="") as handle:
         for row in csv.DictReader(handle):
+            if not wanted(row["Name"], patterns):
+                continue
             lines.append(f"{short_name(row['Name'])[:78]:78s} {int(row['Calls']):6d} "
                          f"{float(row['AverageNs']) / 1e3:10.1f} {float(row['MinNs']) / 1e3:10.1f} "
                          f"{float(row['MaxNs']) / 1e3:10.1f} {float(row['Percentage']):6.2f}")
     return lines
 
 
-def counter_averages(path: Path) -> list[str]:
+def counter_averages(path: Path, patterns: list[str]) -> list[str]:
     table = collections.defaultdict(lambda: collections.defaultdict(list))
     with open(path, newline="") as handle:
         for row in csv.DictReader(handle):
+            if not wanted(row["Kernel_Name"], patterns):
+                continue
             table[short_name(row["Kernel_Name"])][row["Counter_Name"]].append(float(row["Counter_Value"]))
     lines = []
     for kernel, counters in table.items():
@@ -48,16 +56,19 @@ def counter_averages(path: Path) -> list[str]:
 def main():
     parser = argparse.ArgumentParser(description=__doc__)
     parser.add_argument("--command", required=True, help="the profiled command line, recorded in the summary")
+    parser.add_argument("--only", action="append", default=[],
+                        help="keep kernels whose name contains this text (repeatable; default: dscuda and copy kernels)")
     parser.add_argument("directories", nargs="+")
     args = parser.parse_args()
+    patterns = args.only or ["dscuda", "copyBuffer"]
     print(f"command: {args.command}")
     for directory in args.directories:
         for path in sorted(Path(directory).rglob("*_kernel_stats.csv")):
             print(f"\n[kernel trace] {path.name}")
-            print("\n".join(kernel_stats(path)))
+            print("\n".join(kernel_stats(path, patterns)))
         for path in sorted(Path(directory).rglob("*_counter_collection.csv")):
             print(f"\n[counters] {path.name}")
-            print("\n".join(counter_averages(path)))
+            print("\n".join(counter_averages(path, patterns)))
 
 
 if __name__ == "__main__":
