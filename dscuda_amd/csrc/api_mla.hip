@@ -95,7 +95,10 @@ void mla_prefill_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __
 
 std::size_t mla_prefill_backward_workspace_elements(int batch_size, int sequence_length, int heads,
                                                     int /*qk_head_size*/, int /*v_head_size*/) {
-    return static_cast<std::size_t>(batch_size) * heads * sequence_length;
+    if (batch_size <= 0 || sequence_length <= 0 || heads <= 0) {
+        return 0;
+    }
+    return attention_backward_workspace_elements(batch_size, sequence_length, heads);
 }
 
 void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,

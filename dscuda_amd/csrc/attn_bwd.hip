@@ -6,127 +6,223 @@
 // kernel for this form (its absorbed backward, kernels/attention/mla/sm89.cu:
 // 295-411, is one scalar workgroup per gradient row).
 //
-// Three launches, every gradient row has exactly one writer (no atomics):
+// Three launches; every gradient row has exactly one writer (no atomics):
 //
-//   delta      delta[b,h,s] = sum_c dO * O                        (fp32 workspace)
-//   dK/dV      a workgroup owns 128 keys (4 waves x 32) of one head, keeps them
-//              in registers, and walks the query tiles from the diagonal to the
-//              end of the sequence:   S = Q K^T, dP = dO V^T   (q x keys)
-//                                     dV += P^T dO,  dK += dS^T Q
-//   dQ         a workgroup owns 128 queries (4 waves x 32), keeps Q and dO in
-//              registers, and walks the key tiles up to the diagonal, producing
-//              scores transposed as the forward does:
-//                                     S^T = K Q^T, dP^T = V dO^T  (keys x q)
-//                                     dQ^T += K^T dS^T
+//   statistics   per query row: LSE * log2(e) and delta = sum_c dO * O, stored per
+//                64-query tile (padding rows carry LSE = +inf, so they weigh nothing)
+//   dK/dV        a workgroup owns 128 keys (4 waves x 32, K and V rows in registers)
+//                and walks the 64-query tiles from the diagonal to the end:
+//                    S = Q K^T, dP = dO V^T          (queries x keys)
+//                    dV += P^T dO,  dK += dS^T Q
+//                and leaves dS (bf16, before the scale factor) in the workspace,
+//                one 16 KB block per (key block, query tile)
+//   dQ           the separate accumulation pass: a plain product dQ = scale * dS K
+//                over the stored dS blocks, nothing is recomputed
 //
-// In both kernels the probabilities leave the MFMA in its C layout and go back
-// in as an operand whose contraction index is the C layout's row index, so P
-// and dS never cross lanes.  The other operand of those products is needed
-// with the tile's row index (query or key) contiguous per lane; the tile is
-// therefore stored in LDS twice, row-major and transposed (a 4x4 register
-// transpose per thread on the way in, rows regrouped so that the eight indices
-// a lane needs are one 16-byte read), exactly the V^T arrangement of the
-// forward kernel.  Row-major copies use a pitch of 2*D + 16 bytes, transposed
-// copies 128-byte rows with the 16-byte chunk index XORed with (row>>1)&7;
-// both make the 16-row column reads conflict free.
+// Operand feeds.  Q and dO tiles arrive by global_load_lds and are stored once,
+// row-major.  Both orientations are read from that one copy: 16-byte row reads
+// give the operand of S / dP (contraction over the head dimension), and
+// ds_read_b64_tr_b16 gives the operand of dV / dK (contraction over queries).
+// The 16-byte chunk c of row r sits at chunk c ^ f(r); f is chosen per row
+// length so that the 16-row column reads and the 4-row x 64-byte transposing
+// reads are both free of bank conflicts.  P and dS leave the MFMA in its C
+// layout and go back in as operands without crossing lanes.
+//
+// dS blocks are written exactly as the registers hold them (16 bytes per lane,
+// 1 KB per wave instruction, lanes permuted by a constant XOR so that the dQ
+// pass reads them back transposed without bank conflicts).
 #include "attn_kernels.h"
 #include "hip_common.h"
 
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 
 namespace dscuda {
 namespace {
 
 constexpr int BWD_THREADS = 256;
-constexpr int BWD_TILE = 64;   // rows of the streamed operand per tile
+constexpr int QTILE = 64;                            // queries per streamed tile
+constexpr int KBLOCK = 128;                          // keys per workgroup of the dK/dV kernel
+constexpr int DS_BLOCK_BYTES = KBLOCK * QTILE * 2;   // one (key block, query tile) of dS, bf16
+constexpr int DS_BLOCK_FLOATS = DS_BLOCK_BYTES / 4;
+constexpr int STAT_FLOATS = 2 * QTILE;               // per query tile: LSE*log2e [64], delta [64]
 
-// ---- shared tile plumbing ----------------------------------------------------
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4* transposing_read_pointer;
 
-// A [64 rows][D] bf16 tile held twice in LDS.
-template <int D>
-struct DualTile {
-    static constexpr int PITCH = 2 * D + 16;               // row-major copy
-    static constexpr int NATURAL_BYTES = BWD_TILE * PITCH;
-    static constexpr int T_PITCH = 2 * BWD_TILE;            // transposed copy, 128-byte rows
-    static constexpr int TRANSPOSED_BYTES = D * T_PITCH;
-    static constexpr int BYTES = NATURAL_BYTES + TRANSPOSED_BYTES;
-    static constexpr int UNITS = (BWD_TILE / 4) * (D / 4);  // 4 rows x 4 columns per unit
-    static constexpr int PER_THREAD = UNITS / BWD_THREADS;
-    static_assert(UNITS % BWD_THREADS == 0, "tile must divide evenly over the workgroup");
+// Position of dS block (key block kb, query tile qt), qt >= 2*kb, key block major.
+__host__ __device__ inline long long ds_block_index(int kb, int qt, int query_tiles) {
+    return (long long)kb * query_tiles - (long long)kb * (kb - 1) + (qt - 2 * kb);
+}
+
+__host__ __device__ inline long long ds_block_count(int key_blocks, int query_tiles) {
+    return (long long)key_blocks * query_tiles - (long long)key_blocks * (key_blocks - 1);
+}
+
+// Chunk permutation of a row-major LDS tile whose rows are ROW_BYTES long.
+// Row bytes = 0 (mod 256): the four bits of the row, pairs exchanged.
+// Row bytes = 128 (mod 256): the three bits of row>>1, bits 0 and 2 exchanged.
+template <int ROW_BYTES>
+__device__ __forceinline__ constexpr int tile_swizzle(int row) {
+    if constexpr (ROW_BYTES % 256 == 0) {
+        return ((row & 3) << 2) | ((row >> 2) & 3);
+    } else {
+        const int u = row >> 1;
+        return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
+    }
+}
+
+// global_load_lds with 4 bytes per lane (256 consecutive LDS bytes per wave instruction)
+__device__ __forceinline__ void direct_load_4_offset(const void* uniform_base, unsigned byte_offset, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(uniform_base), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
+// This wave's share of the global_load_lds requests of a [64][ROW_BYTES] tile.
+// LDS slot 64*load + lane (16 bytes each) holds chunk (slot % CHUNKS) ^ f(row) of
+// row slot / CHUNKS.  PERIOD loads cover PERIOD_ROWS whole rows; from one period
+// to the next only the low bits of f change, so load L = PERIOD*m + r reads at
+//     tile + m * PERIOD_ROWS * row_stride  +  (base[r] ^ 16 * (m % XOR_STEPS))
+// with one per-lane value per r.  A wave's LOADS consecutive loads start at a
+// multiple of PERIOD * XOR_STEPS, so r and the XOR term are compile-time.  At a
+// ragged end rows past `row_limit` repeat that row (slow path).
+template <int ROW_BYTES>
+struct TileRequests {
+    static constexpr int CHUNKS = ROW_BYTES / 16;
+    static constexpr int LOADS = QTILE * ROW_BYTES / 1024 / (BWD_THREADS / 64);
+    static constexpr int PERIOD = CHUNKS == 24 ? 3 : 1;
+    static constexpr int PERIOD_ROWS = 64 * PERIOD / CHUNKS;
+    static constexpr int XOR_STEPS = CHUNKS == 16 ? 4 : 2;
+    static_assert(CHUNKS == 8 || CHUNKS == 16 || CHUNKS == 24, "rows of 128, 256 or 384 bytes");
+    static_assert(QTILE * ROW_BYTES % (1024 * (BWD_THREADS / 64)) == 0, "tile must divide evenly over the waves");
+    static_assert(LOADS % (PERIOD * XOR_STEPS) == 0, "a wave's loads must start at a whole swizzle period");
+    unsigned base[PERIOD];
+
+    __device__ __forceinline__ static unsigned offset_of(int load, int lane, unsigned row_stride, int row_limit) {
+        const int slot = 64 * load + lane;
+        const int row = slot / CHUNKS;
+        const int chunk = (slot % CHUNKS) ^ tile_swizzle<ROW_BYTES>(row);
+        return (unsigned)min(row, row_limit) * row_stride + 16u * chunk;
+    }
+    __device__ __forceinline__ void init(unsigned row_stride, int lane) {
+#pragma unroll
+        for (int r = 0; r < PERIOD; ++r) base[r] = offset_of(r, lane, row_stride, QTILE);
+    }
+    // `tile` = address of the tile's first row (uniform)
+    __device__ __forceinline__ void request(const unsigned char* tile, unsigned row_stride, int row_limit,
+                                            unsigned lds_target, int wave) const {
+        if (row_limit >= QTILE - 1) {
+            const unsigned char* rows = tile + (size_t)(wave * LOADS / PERIOD * PERIOD_ROWS) * row_stride;
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                direct_load_16_offset(rows + (size_t)(i / PERIOD * PERIOD_ROWS) * row_stride,
+                                      base[i % PERIOD] ^ (16u * ((i / PERIOD) % XOR_STEPS)),
+                                      lds_target + (wave * LOADS + i) * 1024);
+            }
+        } else {
+            const int lane = fresh_lane_id();
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                direct_load_16_offset(tile, offset_of(wave * LOADS + i, lane, row_stride, row_limit),
+                                      lds_target + (wave * LOADS + i) * 1024);
+            }
+        }
+    }
 };
 
-// Loads the 4x4 units of a tile (rows row0.., `rows` valid) owned by this thread.
-template <int D>
-__device__ __forceinline__ void load_units(u32x2 (&stage)[DualTile<D>::PER_THREAD][4], const bf16_t* base,
-                                           size_t row_stride, int row0, int rows, int tid) {
-#pragma unroll
-    for (int i = 0; i < DualTile<D>::PER_THREAD; ++i) {
-        const int unit = tid + BWD_THREADS * i;
-        const int c4 = unit % (D / 4);
-        const int rg = unit / (D / 4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = row0 + 4 * rg + j;
-            u32x2 bits = {0, 0};
-            if (row < rows) {
-                bits = *reinterpret_cast<const u32x2*>(base + (size_t)row * row_stride + 4 * c4);
-            }
-            stage[i][j] = bits;
-        }
-    }
-}
+// Per-lane byte offsets of the fragment reads of a row-major swizzled tile.
+// The swizzle only touches the low SPAN chunk positions of a row, so a handful
+// of per-lane values plus compile-time immediates reach every fragment; a user
+// adds the (run-time) tile base to the per-lane values once per tile.
+//
+//   natural[i]        row lane%32, chunk (2i + g) ^ f(row): the operand whose
+//                     contraction index is the tile column (k-step ks = NAT*m + i
+//                     lies NAT*32*m bytes further, 32 rows down 32*ROW_BYTES)
+//   transposed[h][i]  for ds_read_b64_tr_b16: row 4g + s/4 + 8h (s = lane%16),
+//                     chunk (4i + 2*((lane/16)%2) + (s%4)/2) ^ f(row), byte 8*(s%2):
+//                     the operand whose contraction index is the tile row; MFMA
+//                     row/column lane%32 = tile column 32*block + lane%32, k = rows
+//                     {4g..4g+3, 8+4g..8+4g+3} of a 16-row step -- the order a
+//                     C-layout register block carries (block = TR*m + i lies
+//                     TR*64*m bytes further)
+template <int ROW_BYTES>
+struct TileReads {
+    static constexpr int SPAN = (ROW_BYTES % 256 == 0) ? 16 : 8;
+    static constexpr int NAT = SPAN / 2;
+    static constexpr int TR = SPAN / 4;
+    unsigned natural[NAT];
+    unsigned transposed[2][TR];
 
-// Writes the units row-major (if NATURAL) and transposed (if TRANSPOSED).
-template <int D, bool NATURAL, bool TRANSPOSED>
-__device__ __forceinline__ void store_units(const u32x2 (&stage)[DualTile<D>::PER_THREAD][4], unsigned char* natural,
-                                            unsigned char* transposed, int tid) {
-    using T = DualTile<D>;
+    __device__ __forceinline__ void init(int lane) {
+        const int lq = lane % 32;
+        const int g = lane / 32;
 #pragma unroll
-    for (int i = 0; i < T::PER_THREAD; ++i) {
-        const int unit = tid + BWD_THREADS * i;
-        const int c4 = unit % (D / 4);
-        const int rg = unit / (D / 4);
-        if (NATURAL) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<u32x2*>(natural + (4 * rg + j) * T::PITCH + 8 * c4) = stage[i][j];
-            }
+        for (int i = 0; i < NAT; ++i) {
+            natural[i] = lq * ROW_BYTES + 16 * ((2 * i + g) ^ tile_swizzle<ROW_BYTES>(lq));
         }
-        if (TRANSPOSED) {
-            // rows 4*rg .. 4*rg+3 = 16*n + 8*a + 4*g' + (0..3)  ->  position 16*n + 8*g' + 4*a
-            const int n = rg / 4;
-            const int a = (rg % 4) / 2;
-            const int gp = rg % 2;
-            const int chunk = 2 * n + gp;
-            const u32x2 r0 = stage[i][0], r1 = stage[i][1], r2 = stage[i][2], r3 = stage[i][3];
-            u32x2 t[4];
-            t[0] = u32x2{(r0.x & 0xffffu) | (r1.x << 16), (r2.x & 0xffffu) | (r3.x << 16)};
-            t[1] = u32x2{(r0.x >> 16) | (r1.x & 0xffff0000u), (r2.x >> 16) | (r3.x & 0xffff0000u)};
-            t[2] = u32x2{(r0.y & 0xffffu) | (r1.y << 16), (r2.y & 0xffffu) | (r3.y << 16)};
-            t[3] = u32x2{(r0.y >> 16) | (r1.y & 0xffff0000u), (r2.y >> 16) | (r3.y & 0xffff0000u)};
+        const int s = lane % 16;
+        const int low = 2 * ((lane / 16) % 2) + (s % 4) / 2;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int column = 4 * c4 + e;
-                const int swz = chunk ^ ((column >> 1) & 7);
-                *reinterpret_cast<u32x2*>(transposed + column * T::T_PITCH + 16 * swz + 8 * a) = t[e];
+        for (int h = 0; h < 2; ++h) {
+            const int row = 4 * g + s / 4 + 8 * h;
+#pragma unroll
+            for (int i = 0; i < TR; ++i) {
+                transposed[h][i] = row * ROW_BYTES + 16 * ((4 * i + low) ^ tile_swizzle<ROW_BYTES>(row)) + 8 * (s % 2);
             }
         }
     }
+};
+
+// `at` = TileReads::natural plus the tile's LDS offset; rows ROW0 + lane%32, k-step KS
+template <int ROW_BYTES, int ROW0, int KS>
+__device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* lds, const unsigned (&at)[TileReads<ROW_BYTES>::NAT]) {
+    constexpr int NAT = TileReads<ROW_BYTES>::NAT;
+    return *reinterpret_cast<const bf16x8*>(lds + at[KS % NAT] + (ROW0 * ROW_BYTES + (KS / NAT) * (NAT * 32)));
 }
 
-// Operand fragment from the row-major copy: row `row`, elements 16*ks + 8*g ..
-template <int D>
-__device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* natural, int row, int ks, int g) {
-    return *reinterpret_cast<const bf16x8*>(natural + row * DualTile<D>::PITCH + 32 * ks + 16 * g);
+// `at` = TileReads::transposed plus the tile's LDS offset; 16 rows from ROW0, column block BLOCK
+template <int ROW_BYTES, int ROW0, int BLOCK>
+__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* lds,
+                                                      const unsigned (&at)[2][TileReads<ROW_BYTES>::TR]) {
+    constexpr int TR = TileReads<ROW_BYTES>::TR;
+    constexpr int CONSTANT = ROW0 * ROW_BYTES + (BLOCK / TR) * (TR * 64);
+    const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (transposing_read_pointer)(lds + at[0][BLOCK % TR] + CONSTANT));
+    const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (transposing_read_pointer)(lds + at[1][BLOCK % TR] + CONSTANT));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
-// Operand fragment from the transposed copy: column `column`, the eight tile
-// rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}.
-template <int D>
-__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* transposed, int column, int n, int g) {
-    const int swz = (2 * n + g) ^ ((column >> 1) & 7);
-    return *reinterpret_cast<const bf16x8*>(transposed + column * DualTile<D>::T_PITCH + 16 * swz);
+// f(integral_constant<int, BEGIN>) ... f(integral_constant<int, END - 1>)
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+// Order of the score MFMAs of one half: S and dP steps alternate while dP lasts.
+__host__ __device__ constexpr bool score_slot_is_s(int k, int v_steps) { return k >= 2 * v_steps || k % 2 == 0; }
+__host__ __device__ constexpr int score_slot_step(int k, int v_steps) { return k >= 2 * v_steps ? k - v_steps : k / 2; }
+
+// at = reads + offset
+template <int N>
+__device__ __forceinline__ void rebase(unsigned (&at)[N], const unsigned (&reads)[N], unsigned offset) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) at[i] = reads[i] + offset;
+}
+template <int N>
+__device__ __forceinline__ void rebase(unsigned (&at)[2][N], const unsigned (&reads)[2][N], unsigned offset) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) at[h][i] = reads[h][i] + offset;
+    }
 }
 
 // Registers of an operand that stays with the wave: row `row` of a [.][D] matrix.
@@ -144,86 +240,97 @@ __device__ __forceinline__ void load_row_fragments(bf16x8 (&fragments)[D / 16], 
     }
 }
 
+// Element of an MFMA result that lives in the accumulation registers, copied where
+// it is needed (the compiler would otherwise copy all sixteen at the first use and
+// hold them).  Two further MFMAs must have been issued since the one that produced it.
+template <int I>
+__device__ __forceinline__ float accumulator_element(const f32x16& accumulator) {
+    float value;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(value) : "a"(accumulator[I]));
+    return value;
+}
+
 __device__ __forceinline__ void clear(f32x16& value) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) value[i] = 0.f;
 }
 
-// ---- delta -------------------------------------------------------------------
+// ---- statistics ---------------------------------------------------------------
 
-// One 16-lane group per (b, s, h) row: delta = sum_c dO * O, written as [B,H,S].
+// One 16-lane group per (b, s, h) row of the sequence padded to whole query tiles.
 template <int DV>
-__global__ __launch_bounds__(256) void attention_delta_kernel(float* __restrict__ delta,
-                                                              const bf16_t* __restrict__ output_gradient,
-                                                              const bf16_t* __restrict__ output, int batch_size,
-                                                              int sequence_length, int heads) {
-    const long long rows = (long long)batch_size * sequence_length * heads;
+__global__ __launch_bounds__(256) void attention_backward_statistics_kernel(
+    float* __restrict__ statistics, const bf16_t* __restrict__ output_gradient, const bf16_t* __restrict__ output,
+    const float* __restrict__ logsumexp, int batch_size, int sequence_length, int heads, int query_tiles) {
+    const long long padded = (long long)query_tiles * QTILE;
+    const long long rows = (long long)batch_size * padded * heads;
     const long long row = (long long)blockIdx.x * 16 + threadIdx.x / 16;
     const int part = threadIdx.x % 16;
+    if (row >= rows) {
+        return;
+    }
+    const long long h = row % heads;
+    const long long s = (row / heads) % padded;
+    const long long b = row / (heads * padded);
     float sum = 0.f;
-    if (row < rows) {
+    float lse2 = INFINITY;
+    if (s < sequence_length) {
+        const long long source = ((b * sequence_length + s) * heads + h) * DV;
 #pragma unroll
         for (int c = part * 8; c < DV; c += 128) {
-            const u32x4 a = *reinterpret_cast<const u32x4*>(output_gradient + row * DV + c);
-            const u32x4 b = *reinterpret_cast<const u32x4*>(output + row * DV + c);
+            const u32x4 x = *reinterpret_cast<const u32x4*>(output_gradient + source + c);
+            const u32x4 y = *reinterpret_cast<const u32x4*>(output + source + c);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                sum += bf16_bits_to_float(a[j] & 0xffffu) * bf16_bits_to_float(b[j] & 0xffffu);
-                sum += bf16_bits_to_float(a[j] >> 16) * bf16_bits_to_float(b[j] >> 16);
+                sum += bf16_bits_to_float(x[j] & 0xffffu) * bf16_bits_to_float(y[j] & 0xffffu);
+                sum += bf16_bits_to_float(x[j] >> 16) * bf16_bits_to_float(y[j] >> 16);
             }
         }
+        lse2 = logsumexp[(b * heads + h) * sequence_length + s] * LOG2E;
     }
 #pragma unroll
     for (int offset = 1; offset < 16; offset <<= 1) sum += __shfl_xor(sum, offset);
-    if (row < rows && part == 0) {
-        const long long h = row % heads;
-        const long long s = (row / heads) % sequence_length;
-        const long long b = row / ((long long)heads * sequence_length);
-        delta[(b * heads + h) * sequence_length + s] = sum;
+    if (part == 0) {
+        float* target = statistics + ((b * heads + h) * query_tiles + s / QTILE) * STAT_FLOATS + s % QTILE;
+        target[0] = lse2;
+        target[QTILE] = sum;
     }
 }
 
-// ---- dK / dV -----------------------------------------------------------------
+// ---- dK / dV (and dS) -----------------------------------------------------------
 
 template <int DQK, int DV>
-struct KeyGradConfig {
-    using QT = DualTile<DQK>;
-    using OT = DualTile<DV>;
-    static constexpr int KEYS = 128;  // per workgroup
-    static constexpr int Q_NATURAL = 0;
-    static constexpr int Q_TRANSPOSED = Q_NATURAL + QT::NATURAL_BYTES;
-    static constexpr int DO_NATURAL = Q_TRANSPOSED + QT::TRANSPOSED_BYTES;
-    static constexpr int DO_TRANSPOSED = DO_NATURAL + OT::NATURAL_BYTES;
-    static constexpr int STATS = DO_TRANSPOSED + OT::TRANSPOSED_BYTES;   // lse*log2e [64], delta [64]
-    static constexpr int LDS_BYTES = STATS + 2 * BWD_TILE * 4;
+struct KeyValueGradConfig {
+    static constexpr int Q_ROW = 2 * DQK;
+    static constexpr int O_ROW = 2 * DV;
+    static constexpr int Q_BYTES = QTILE * Q_ROW;
+    static constexpr int O_BYTES = QTILE * O_ROW;
+    static constexpr int STAT_BYTES = STAT_FLOATS * 4;
+    static constexpr int STAGE_BYTES = Q_BYTES + O_BYTES + STAT_BYTES;
+    static constexpr int STAGES = 3;
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     static constexpr int DK_PITCH = 2 * DQK;   // epilogue staging
     static constexpr int DV_PITCH = 2 * DV;
     static_assert(4 * 32 * (DK_PITCH + DV_PITCH) <= LDS_BYTES, "epilogue staging must fit");
+    static_assert(LDS_BYTES <= 160 * 1024, "stages must fit the LDS");
 };
 
 template <int DQK, int DV>
-__global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
-    bf16_t* __restrict__ key_gradient, bf16_t* __restrict__ value_gradient,
-    const bf16_t* __restrict__ output_gradient, const float* __restrict__ logsumexp, const float* __restrict__ delta,
+__global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kernel(
+    bf16_t* __restrict__ key_gradient, bf16_t* __restrict__ value_gradient, unsigned char* __restrict__ ds_blocks,
+    const float* __restrict__ statistics, const bf16_t* __restrict__ output_gradient,
     const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
-    int sequence_length, int heads, int key_blocks, float scale) {
-    using C = KeyGradConfig<DQK, DV>;
-    using QT = DualTile<DQK>;
-    using OT = DualTile<DV>;
+    int sequence_length, int heads, int key_blocks, int query_tiles, float scale) {
+    using C = KeyValueGradConfig<DQK, DV>;
     constexpr int QK_STEPS = DQK / 16;
     constexpr int V_STEPS = DV / 16;
     constexpr int DK_BLOCKS = DQK / 32;
     constexpr int DV_BLOCKS = DV / 32;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* q_natural = lds + C::Q_NATURAL;
-    unsigned char* q_transposed = lds + C::Q_TRANSPOSED;
-    unsigned char* do_natural = lds + C::DO_NATURAL;
-    unsigned char* do_transposed = lds + C::DO_TRANSPOSED;
-    float* stats = reinterpret_cast<float*>(lds + C::STATS);
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
@@ -233,18 +340,22 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
     xcd_order(blockIdx.x, gridDim.x / key_blocks, key_blocks, bh, kb);
     const int b = bh / heads;
     const int h = bh % heads;
-    const int k0 = kb * C::KEYS;
+    const int k0 = kb * KBLOCK;
     const int wave_k0 = k0 + 32 * wave;
     const int key_row = wave_k0 + lq;
 
     const size_t qk_stride = (size_t)heads * DQK;
     const size_t v_stride = (size_t)heads * DV;
-    const bf16_t* q_base = query + ((size_t)b * S * heads + h) * DQK;
+    const unsigned q_stride_bytes = (unsigned)heads * DQK * 2;
+    const unsigned o_stride_bytes = (unsigned)heads * DV * 2;
+    const unsigned char* q_base = reinterpret_cast<const unsigned char*>(query + ((size_t)b * S * heads + h) * DQK);
+    const unsigned char* do_base =
+        reinterpret_cast<const unsigned char*>(output_gradient + ((size_t)b * S * heads + h) * DV);
     const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
     const bf16_t* v_base = value + ((size_t)b * S * heads + h) * DV;
-    const bf16_t* do_base = output_gradient + ((size_t)b * S * heads + h) * DV;
-    const float* lse_base = logsumexp + ((size_t)b * heads + h) * S;
-    const float* delta_base = delta + ((size_t)b * heads + h) * S;
+    const float* stat_base = statistics + (size_t)bh * query_tiles * STAT_FLOATS;
+    unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+    const unsigned lds_base = lds_offset_of(lds);
 
     // K and V rows of this wave, as B operands (column = key lq)
     bf16x8 kf[QK_STEPS], vf[V_STEPS];
@@ -258,99 +369,305 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
     for (int d = 0; d < DV_BLOCKS; ++d) clear(dv_acc[d]);
 
     const float c = scale * LOG2E;
-    const int first_tile = k0 / BWD_TILE;
-    const int last_tile = (S - 1) / BWD_TILE;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int first_tile = 2 * kb;
+    const int tiles = query_tiles - first_tile;   // >= 1
 
-    u32x2 q_stage[QT::PER_THREAD][4], do_stage[OT::PER_THREAD][4];
-    float stat_stage = 0.f;
-    auto load_tile = [&](int tile) {
-        const int row0 = tile * BWD_TILE;
-        load_units<DQK>(q_stage, q_base, qk_stride, row0, S, tid);
-        load_units<DV>(do_stage, do_base, v_stride, row0, S, tid);
-        if (tid < 2 * BWD_TILE) {
-            const int row = row0 + tid % BWD_TILE;
-            stat_stage = 0.f;
-            if (row < S) stat_stage = tid < BWD_TILE ? lse_base[row] * LOG2E : delta_base[row];
+    TileRequests<C::Q_ROW> q_requests;
+    TileRequests<C::O_ROW> o_requests;
+    q_requests.init(q_stride_bytes, lane);
+    o_requests.init(o_stride_bytes, lane);
+    auto request_tile = [&](int index, int stage) {
+        const int tile = first_tile + index;
+        const int row0 = tile * QTILE;
+        const int row_limit = S - 1 - row0;
+        const unsigned target = lds_base + stage * C::STAGE_BYTES;
+        q_requests.request(q_base + (size_t)row0 * q_stride_bytes, q_stride_bytes, row_limit, target, wave);
+        o_requests.request(do_base + (size_t)row0 * o_stride_bytes, o_stride_bytes, row_limit, target + C::Q_BYTES, wave);
+        if (wave < 2) {
+            direct_load_4_offset(stat_base + (size_t)tile * STAT_FLOATS + 64 * wave, 4u * lane,
+                                 target + C::Q_BYTES + C::O_BYTES + 256 * wave);
         }
     };
-    auto store_tile = [&]() {
-        store_units<DQK, true, true>(q_stage, q_natural, q_transposed, tid);
-        store_units<DV, true, true>(do_stage, do_natural, do_transposed, tid);
-        if (tid < 2 * BWD_TILE) stats[tid] = stat_stage;
+
+    // per-lane read offsets inside a stage, and their per-stage instances
+    TileReads<C::Q_ROW> q_reads;
+    TileReads<C::O_ROW> o_reads;
+    q_reads.init(lane);
+    o_reads.init(lane);
+    struct ScoreReads {
+        unsigned q[TileReads<C::Q_ROW>::NAT];
+        unsigned o[TileReads<C::O_ROW>::NAT];
+    };
+    struct GradientReads {
+        unsigned q[2][TileReads<C::Q_ROW>::TR];
+        unsigned o[2][TileReads<C::O_ROW>::TR];
+    };
+    auto score_reads = [&](ScoreReads& at, int stage) {
+        rebase(at.q, q_reads.natural, stage * C::STAGE_BYTES);
+        rebase(at.o, o_reads.natural, stage * C::STAGE_BYTES + C::Q_BYTES);
+    };
+    auto gradient_reads = [&](GradientReads& at, int stage) {
+        rebase(at.q, q_reads.transposed, stage * C::STAGE_BYTES);
+        rebase(at.o, o_reads.transposed, stage * C::STAGE_BYTES + C::Q_BYTES);
+    };
+    auto stats_of = [&](int stage) -> unsigned { return stage * C::STAGE_BYTES + C::Q_BYTES + C::O_BYTES + 16 * g; };
+
+    // Half tiles.  The unit of the software pipeline is half a tile (32 queries):
+    //     S, dP (SCORE_MFMAS) -> P, dS (VALU) -> dV, dK (GRAD_MFMAS).
+    // Half j keeps its scores in set j%2 of (s_acc, dp_acc) and its operands in
+    // set j%2 of (pf, dsf).  One "half step" issues, as a single stream of MFMA
+    // slots, the gradient products of half j and the score products of half j + 2,
+    // with the probabilities of half j + 1 cut into small pieces that follow the
+    // MFMAs one by one: the three jobs touch disjoint registers, and a wave then
+    // keeps the matrix pipeline fed from its own instruction stream (a 32x32x16
+    // MFMA occupies it for 32 clocks, enough for seven other instructions).
+    // Every MFMA takes one fragment from LDS; the fragments run through a ring of
+    // RING register sets, read RING slots ahead -- across half steps and across
+    // the barrier between tiles (the tile read ahead has landed one tile earlier).
+    // All slot, set and register indices are compile-time constants.
+    constexpr int RING = 8;
+    constexpr int PER_STEP = DV_BLOCKS + DK_BLOCKS;        // gradient MFMAs per 16 queries
+    constexpr int GRAD_MFMAS = 2 * PER_STEP;
+    constexpr int SCORE_MFMAS = QK_STEPS + V_STEPS;
+    constexpr int PIECES = 20;                             // of the probabilities of one half
+    constexpr int PIECE_DELAY = 2;                         // slots before the first piece: the scores it reads
+                                                           // were finished by the last MFMA of the previous half step
+    static_assert(GRAD_MFMAS >= RING, "the fragments read ahead must all belong to the gradient products");
+    static_assert(QK_STEPS >= V_STEPS, "score slots alternate S and dP while dP lasts");
+
+    f32x16 s_acc[2], dp_acc[2];
+    u32x4 pf[2][2], dsf[2][2];   // [set][16-query step]: packed bf16 operands
+    bf16x8 ring[RING];
+    f32x4 lse4[2], delta4[2];    // two sets: a group of four queries is loaded while the previous one is used
+    float p[4], ds[4];
+
+    // fragment of gradient slot K (K < GRAD_MFMAS) of query half QB
+    auto gradient_fragment = [&](const GradientReads& at, auto qb_tag, auto k_tag) -> bf16x8 {
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int K = decltype(k_tag)::value;
+        constexpr int N = K / PER_STEP;
+        constexpr int R = K % PER_STEP;
+        if constexpr (R < DV_BLOCKS) {
+            return transposed_fragment<C::O_ROW, 32 * QB + 16 * N, R>(lds, at.o);
+        } else {
+            return transposed_fragment<C::Q_ROW, 32 * QB + 16 * N, R - DV_BLOCKS>(lds, at.q);
+        }
+    };
+    // score slot K: S and dP steps alternate while dP lasts (two independent chains)
+    auto score_fragment = [&](const ScoreReads& at, auto qb_tag, auto k_tag) -> bf16x8 {
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int K = decltype(k_tag)::value;
+        if constexpr (score_slot_is_s(K, V_STEPS)) {
+            return natural_fragment<C::Q_ROW, 32 * QB, score_slot_step(K, V_STEPS)>(lds, at.q);
+        } else {
+            return natural_fragment<C::O_ROW, 32 * QB, score_slot_step(K, V_STEPS)>(lds, at.o);
+        }
+    };
+    auto score_mfma = [&](auto qb_tag, auto k_tag, bf16x8 fragment) {
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int K = decltype(k_tag)::value;
+        constexpr int STEP = score_slot_step(K, V_STEPS);
+        if constexpr (score_slot_is_s(K, V_STEPS)) {
+            s_acc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[STEP], STEP == 0 ? zero : s_acc[QB], 0, 0, 0);
+        } else {
+            dp_acc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, vf[STEP], STEP == 0 ? zero : dp_acc[QB], 0, 0, 0);
+        }
+    };
+    auto gradient_mfma = [&](auto qb_tag, auto k_tag, bf16x8 fragment) {
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int K = decltype(k_tag)::value;
+        constexpr int N = K / PER_STEP;
+        constexpr int R = K % PER_STEP;
+        if constexpr (R < DV_BLOCKS) {
+            dv_acc[R] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[QB][N]), fragment,
+                                                                dv_acc[R], 0, 0, 0);
+        } else {
+            dk_acc[R - DV_BLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, dsf[QB][N]),
+                                                                            fragment, dk_acc[R - DV_BLOCKS], 0, 0, 0);
+        }
     };
 
-    load_tile(first_tile);
-    for (int tile = first_tile; tile <= last_tile; ++tile) {
-        __syncthreads();   // every wave is done with the previous tile
-        store_tile();
-        __syncthreads();
-        if (tile < last_tile) load_tile(tile + 1);
-        const int q0 = tile * BWD_TILE;
-        // Tiles whose queries all precede this wave's keys (at most one per wave)
-        // are not skipped: they contribute exact zeros through the mask, and a
-        // branch around the accumulator updates makes the compiler shuttle all
-        // 160 accumulators through scratch.
-
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-            // S and dP for 32 queries x this wave's 32 keys
-            f32x16 s_acc, dp_acc;
-            clear(s_acc);
-            clear(dp_acc);
-#pragma unroll
-            for (int ks = 0; ks < QK_STEPS; ++ks) {
-                const bf16x8 a = natural_fragment<DQK>(q_natural, 32 * qb + lq, ks, g);
-                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[ks], s_acc, 0, 0, 0);
-            }
-#pragma unroll
-            for (int ks = 0; ks < V_STEPS; ++ks) {
-                const bf16x8 a = natural_fragment<DV>(do_natural, 32 * qb + lq, ks, g);
-                dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vf[ks], dp_acc, 0, 0, 0);
-            }
-            // lane holds key lq and queries 32*qb + 8*(i/4) + 4*g + i%4
-            const bool diagonal = q0 + 32 * qb < wave_k0 + 31;
-            bf16x8 pf[2], dsf[2];
-#pragma unroll
-            for (int n = 0; n < 2; ++n) {
-                u32x4 p_packed, ds_packed;
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int i4 = 2 * n + half;
-                    const int q_local = 32 * qb + 8 * i4 + 4 * g;
-                    const f32x4 lse4 = *reinterpret_cast<const f32x4*>(stats + q_local);
-                    const f32x4 delta4 = *reinterpret_cast<const f32x4*>(stats + BWD_TILE + q_local);
-                    float p[4], ds[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int i = 4 * i4 + e;
-                        float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[e]));
-                        if (diagonal && q0 + q_local + e < key_row) probability = 0.f;
-                        p[e] = probability;
-                        ds[e] = probability * (dp_acc[i] - delta4[e]) * scale;
-                    }
-                    p_packed[2 * half] = pack_bf16(p[0], p[1]);
-                    p_packed[2 * half + 1] = pack_bf16(p[2], p[3]);
-                    ds_packed[2 * half] = pack_bf16(ds[0], ds[1]);
-                    ds_packed[2 * half + 1] = pack_bf16(ds[2], ds[3]);
-                }
-                pf[n] = __builtin_bit_cast(bf16x8, p_packed);
-                dsf[n] = __builtin_bit_cast(bf16x8, ds_packed);
-            }
-            // dV += P^T dO, dK += dS^T Q (contraction over the 32 queries)
-#pragma unroll
-            for (int n = 0; n < 2; ++n) {
-#pragma unroll
-                for (int d = 0; d < DV_BLOCKS; ++d) {
-                    const bf16x8 bo = transposed_fragment<DV>(do_transposed, 32 * d + lq, 2 * qb + n, g);
-                    dv_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[n], bo, dv_acc[d], 0, 0, 0);
-                }
-#pragma unroll
-                for (int d = 0; d < DK_BLOCKS; ++d) {
-                    const bf16x8 bq = transposed_fragment<DQK>(q_transposed, 32 * d + lq, 2 * qb + n, g);
-                    dk_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[n], bq, dk_acc[d], 0, 0, 0);
-                }
-            }
+    // statistics of queries 32*QB + 8*I4 + 4*g + (0..3) (stats_at carries the 16*g)
+    auto load_statistics = [&](unsigned stats_at, auto qb_tag, auto i4_tag) {
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int I4 = decltype(i4_tag)::value;
+        lse4[I4 % 2] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
+        delta4[I4 % 2] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (QTILE + 32 * QB + 8 * I4));
+    };
+    // Piece V (0..19) of the probabilities of half QB: lane holds key lq and queries
+    // 32*QB + 8*I4 + 4*g + E, I4 = V/5; pieces 5*I4 + E do element E (and the first of
+    // them requests the statistics of the next four queries), piece 5*I4 + 4 packs
+    // the four.  `threshold` = key_row - 4*g - q0: a query with local index below it
+    // lies before this lane's key.
+    auto probability_piece = [&](auto masked_tag, auto qb_tag, auto v_tag, unsigned stats_at, int threshold) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr int QB = decltype(qb_tag)::value;
+        constexpr int V = decltype(v_tag)::value;
+        constexpr int I4 = V / 5;
+        constexpr int E = V % 5;
+        if constexpr (E == 0 && I4 + 1 < 4) {
+            load_statistics(stats_at, qb_tag, std::integral_constant<int, (I4 + 1) % 4>{});
         }
+        if constexpr (E < 4) {
+            constexpr int I = 4 * I4 + E;
+            p[E] = __builtin_amdgcn_exp2f(fmaf(accumulator_element<I>(s_acc[QB]), c, -lse4[I4 % 2][E]));
+            if (MASKED && 32 * QB + 8 * I4 + E < threshold) {
+                p[E] = 0.f;
+            }
+            ds[E] = p[E] * (accumulator_element<I>(dp_acc[QB]) - delta4[I4 % 2][E]);
+        } else {
+            constexpr int N = I4 / 2;
+            constexpr int HALF = I4 % 2;
+            pf[QB][N][2 * HALF] = pack_bf16(p[0], p[1]);
+            pf[QB][N][2 * HALF + 1] = pack_bf16(p[2], p[3]);
+            dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
+            dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
+        }
+    };
+
+    // dS of half QB of tile `index` to its block: 16 bytes per lane, slot
+    // (lane ^ (4g + 8n)) of the 1 KB piece (wave, QB, n)
+    auto store_ds = [&](int index, auto qb_tag) {
+        constexpr int QB = decltype(qb_tag)::value;
+        unsigned char* block = ds_head + (size_t)ds_block_index(kb, first_tile + index, query_tiles) * DS_BLOCK_BYTES;
+        *reinterpret_cast<u32x4*>(block + ((wave * 2 + QB) * 2 + 0) * 1024 + 16 * (lane ^ (4 * g))) = dsf[QB][0];
+        *reinterpret_cast<u32x4*>(block + ((wave * 2 + QB) * 2 + 1) * 1024 + 16 * (lane ^ (4 * g + 8))) = dsf[QB][1];
+    };
+    auto threshold_of = [&](int index) { return key_row - 4 * g - (first_tile + index) * QTILE; };
+
+    // One half step.  Gradient products of half QB of the tile in stage
+    // `grad_stage` (operands set QB); with SCORES the score products of half QB of
+    // the tile in `score_stage` (into set QB); with PROBS the probabilities of half
+    // 1 - QB of the tile in `prob_stage` (scores set 1 - QB, into operand set
+    // 1 - QB).  With AHEAD the first RING fragments of the following half step
+    // (gradient fragments of half 1 - QB of the tile in next_stage) are read at
+    // the end.  Read addresses are formed where they are first needed.
+    auto half_step = [&](auto masked_tag, auto scores_tag, auto probs_tag, auto ahead_tag, auto qb_tag, auto phase_tag,
+                         int grad_stage, int score_stage, int prob_stage, int prob_threshold, int next_stage) {
+        constexpr int PHASE = decltype(phase_tag)::value;   // ring set of slot 0: slots consumed before, mod RING
+        constexpr bool SCORES = decltype(scores_tag)::value;
+        constexpr bool PROBS = decltype(probs_tag)::value;
+        constexpr bool AHEAD = decltype(ahead_tag)::value;
+        constexpr int QB = decltype(qb_tag)::value;
+        using Other = std::integral_constant<int, 1 - QB>;
+        constexpr int COUNT = GRAD_MFMAS + (SCORES ? SCORE_MFMAS : 0);
+        constexpr int SPAN = COUNT - PIECE_DELAY;   // slots that carry pieces
+        static_assert(4 * SPAN >= PIECES, "at most four pieces per slot");
+        GradientReads grad_at, next_at;
+        ScoreReads score_at;
+        gradient_reads(grad_at, grad_stage);
+        const unsigned prob_stats = stats_of(prob_stage);
+        if constexpr (PROBS) {
+            load_statistics(prob_stats, Other{}, std::integral_constant<int, 0>{});
+        }
+        static_for<0, COUNT>([&](auto slot) {
+            constexpr int I = decltype(slot)::value;
+            if constexpr (I < GRAD_MFMAS) {
+                gradient_mfma(qb_tag, slot, ring[(I + PHASE) % RING]);
+            } else {
+                score_mfma(qb_tag, std::integral_constant<int, I - GRAD_MFMAS>{}, ring[(I + PHASE) % RING]);
+            }
+            constexpr int A = I + RING;
+            if constexpr (SCORES && A == GRAD_MFMAS) {
+                score_reads(score_at, score_stage);
+            }
+            if constexpr (AHEAD && A == COUNT) {
+                gradient_reads(next_at, next_stage);
+            }
+            if constexpr (A < GRAD_MFMAS) {
+                ring[(I + PHASE) % RING] = gradient_fragment(grad_at, qb_tag, std::integral_constant<int, A>{});
+            } else if constexpr (A < COUNT) {
+                ring[(I + PHASE) % RING] = score_fragment(score_at, qb_tag, std::integral_constant<int, A - GRAD_MFMAS>{});
+            } else if constexpr (AHEAD) {
+                ring[(I + PHASE) % RING] = gradient_fragment(next_at, Other{}, std::integral_constant<int, A - COUNT>{});
+            }
+            if constexpr (PROBS && I >= PIECE_DELAY) {
+                // piece v goes to slot PIECE_DELAY + v * SPAN / PIECES: spread evenly
+                constexpr int J = I - PIECE_DELAY;
+                constexpr int FIRST = (J * PIECES + SPAN - 1) / SPAN;
+                constexpr int LAST = ((J + 1) * PIECES + SPAN - 1) / SPAN;
+                static_for<FIRST, LAST>([&](auto v_tag) {
+                    probability_piece(masked_tag, Other{}, v_tag, prob_stats, prob_threshold);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    // ---- prologue: tiles 0 and 1 requested; S, dP of tile 0 and P, dS of its first
+    // half formed; the ring primed with the first gradient fragments of tile 0
+    wait_vector_memory<0>();   // the K / V row loads: no wait for them may remain inside the loop
+    request_tile(0, 0);
+    if (tiles > 1) {
+        request_tile(1, 1);
+    }
+    wait_vector_memory<0>();
+    workgroup_barrier();
+    {
+        ScoreReads at;
+        score_reads(at, 0);
+        static_for<0, 2>([&](auto qb_tag) {
+            static_for<0, SCORE_MFMAS>([&](auto k_tag) { score_mfma(qb_tag, k_tag, score_fragment(at, qb_tag, k_tag)); });
+        });
+        // the scores must have left the matrix pipeline before their elements are copied out
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned stats_at = stats_of(0);
+        load_statistics(stats_at, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+        static_for<0, PIECES>([&](auto v_tag) {
+            probability_piece(std::true_type{}, std::integral_constant<int, 0>{}, v_tag, stats_at, threshold_of(0));
+        });
+        GradientReads first;
+        gradient_reads(first, 0);
+        static_for<0, RING>([&](auto k_tag) {
+            ring[decltype(k_tag)::value] = gradient_fragment(first, std::integral_constant<int, 0>{}, k_tag);
+        });
+    }
+
+    // Tile `index`: both halves are accumulated while the scores of tile index + 1
+    // and the probabilities of the halves in between are formed.  MASKED applies
+    // the causal mask to those probabilities, LAST leaves out everything that
+    // belongs to tile index + 1.
+    auto body = [&](auto masked_tag, auto last_tag, int index) {
+        constexpr bool LAST = decltype(last_tag)::value;
+        using NotLast = std::integral_constant<bool, !LAST>;
+        const int stage = index % 3;
+        const int next_stage = stage == 2 ? 0 : stage + 1;
+        wait_vector_memory<0>();   // this wave's share of tile index + 1 has landed
+        workgroup_barrier();       // ... and everybody's; every wave has left tile index - 1
+        if (index + 2 < tiles) {
+            request_tile(index + 2, (index + 2) % 3);
+        }
+        store_ds(index, std::integral_constant<int, 0>{});
+        if (index > 0) {
+            store_ds(index - 1, std::integral_constant<int, 1>{});
+        }
+        // a whole tile's slots are a multiple of RING; half a LAST tile's need not be
+        static_assert((GRAD_MFMAS + SCORE_MFMAS) % RING == 0, "the ring must close over a half step");
+        using SecondPhase = std::integral_constant<int, LAST ? GRAD_MFMAS % RING : 0>;
+        half_step(masked_tag, NotLast{}, std::true_type{}, std::true_type{}, std::integral_constant<int, 0>{},
+                  std::integral_constant<int, 0>{}, stage, next_stage, stage, threshold_of(index), stage);
+        half_step(masked_tag, NotLast{}, NotLast{}, NotLast{}, std::integral_constant<int, 1>{}, SecondPhase{}, stage,
+                  next_stage, next_stage, threshold_of(index + 1), next_stage);
+    };
+
+    // the causal mask can only bite in the first two tiles of a key block
+    {
+        int index = 0;
+        for (; index < 2 && index + 1 < tiles; ++index) {
+            body(std::true_type{}, std::false_type{}, index);
+        }
+        for (; index + 1 < tiles; ++index) {
+            body(std::false_type{}, std::false_type{}, index);
+        }
+        if (index < 2) {
+            body(std::true_type{}, std::true_type{}, index);
+        } else {
+            body(std::false_type{}, std::true_type{}, index);
+        }
+        store_ds(index, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
@@ -362,7 +679,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int row = 8 * (i / 4) + 4 * g + i % 4;
-            const __bf16 rounded = (__bf16)dk_acc[d][i];
+            const __bf16 rounded = (__bf16)(dk_acc[d][i] * scale);
             *reinterpret_cast<__bf16*>(dk_lds + row * C::DK_PITCH + 2 * (32 * d + lq)) = rounded;
         }
     }
@@ -378,17 +695,17 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
     __syncthreads();
     bf16_t* dk_base = key_gradient + ((size_t)b * S * heads + h) * DQK;
     bf16_t* dv_base = value_gradient + ((size_t)b * S * heads + h) * DV;
-    for (int index = lane; index < 32 * (DQK / 8); index += 64) {
-        const int row = index / (DQK / 8);
-        const int chunk = index % (DQK / 8);
+    for (int position = lane; position < 32 * (DQK / 8); position += 64) {
+        const int row = position / (DQK / 8);
+        const int chunk = position % (DQK / 8);
         if (wave_k0 + row < S) {
             const u32x4 bits = *reinterpret_cast<const u32x4*>(dk_lds + row * C::DK_PITCH + 16 * chunk);
             *reinterpret_cast<u32x4*>(dk_base + (size_t)(wave_k0 + row) * qk_stride + 8 * chunk) = bits;
         }
     }
-    for (int index = lane; index < 32 * (DV / 8); index += 64) {
-        const int row = index / (DV / 8);
-        const int chunk = index % (DV / 8);
+    for (int position = lane; position < 32 * (DV / 8); position += 64) {
+        const int row = position / (DV / 8);
+        const int chunk = position % (DV / 8);
         if (wave_k0 + row < S) {
             const u32x4 bits = *reinterpret_cast<const u32x4*>(dv_lds + row * C::DV_PITCH + 16 * chunk);
             *reinterpret_cast<u32x4*>(dv_base + (size_t)(wave_k0 + row) * v_stride + 8 * chunk) = bits;
@@ -396,194 +713,181 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_gradient_kernel(
     }
 }
 
-// ---- dQ ----------------------------------------------------------------------
+// ---- dQ -------------------------------------------------------------------------
 
-template <int DQK, int DV>
+template <int DQK>
 struct QueryGradConfig {
-    using KT = DualTile<DQK>;
-    static constexpr int QUERIES = 128;  // per workgroup
-    static constexpr int V_PITCH = 2 * DV + 16;
-    static constexpr int V_BYTES = BWD_TILE * V_PITCH;
-    static constexpr int V_CHUNKS = BWD_TILE * (DV / 8);
-    static constexpr int V_PER_THREAD = V_CHUNKS / BWD_THREADS;
-    static constexpr int K_NATURAL = 0;
-    static constexpr int K_TRANSPOSED = K_NATURAL + KT::NATURAL_BYTES;
-    static constexpr int V_NATURAL = K_TRANSPOSED + KT::TRANSPOSED_BYTES;
-    static constexpr int STAGE_BYTES = V_NATURAL + V_BYTES;
-    static constexpr int DQ_PITCH = 2 * DQK + 16;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-    static_assert(QUERIES * DQ_PITCH <= LDS_BYTES, "epilogue staging must fit");
-    static_assert(V_CHUNKS % BWD_THREADS == 0, "V tile must divide evenly over the workgroup");
+    static constexpr int QUERIES = 2 * QTILE;            // per workgroup: two query tiles
+    static constexpr int STEP_KEYS = 64;                 // keys per step: half a dS block
+    static constexpr int K_ROW = 2 * DQK;
+    static constexpr int K_BYTES = STEP_KEYS * K_ROW;
+    static constexpr int DS_HALF = DS_BLOCK_BYTES / 2;   // 64 keys x 64 queries
+    static constexpr int STAGE_BYTES = K_BYTES + 2 * DS_HALF;
+    static constexpr int STAGES = 3;
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int D_BLOCKS = DQK / 64;            // 32-column blocks per wave
+    static_assert(LDS_BYTES <= 160 * 1024, "stages must fit the LDS");
 };
 
-template <int DQK, int DV>
+// dQ^T (d x queries) = sum over keys of K^T (d x keys) dS^T (keys x queries).
+// Wave w owns query tile w%2 of the workgroup's two and the 32-column blocks 2*d + w/2.
+template <int DQK>
 __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
-    bf16_t* __restrict__ query_gradient, const bf16_t* __restrict__ output_gradient,
-    const float* __restrict__ logsumexp, const float* __restrict__ delta, const bf16_t* __restrict__ query,
-    const bf16_t* __restrict__ key, const bf16_t* __restrict__ value, int sequence_length, int heads,
-    int query_blocks, float scale) {
-    using C = QueryGradConfig<DQK, DV>;
-    using KT = DualTile<DQK>;
-    constexpr int QK_STEPS = DQK / 16;
-    constexpr int V_STEPS = DV / 16;
-    constexpr int DQ_BLOCKS = DQK / 32;
+    bf16_t* __restrict__ query_gradient, const unsigned char* __restrict__ ds_blocks, const bf16_t* __restrict__ key,
+    int sequence_length, int heads, int query_blocks, int key_blocks, int query_tiles, float scale) {
+    using C = QueryGradConfig<DQK>;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
     const int S = sequence_length;
 
-    int bh, qb_rank;
-    xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, qb_rank);
-    const int qb = query_blocks - 1 - qb_rank;  // heaviest (last) query blocks first
+    int bh, rank;
+    xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, rank);
+    const int jb = query_blocks - 1 - rank;   // heaviest (last) query blocks first
     const int b = bh / heads;
     const int h = bh % heads;
-    const int q0 = qb * C::QUERIES;
-    const int wave_q0 = q0 + 32 * wave;
-    const int q_row = wave_q0 + lq;
-    const bool valid = q_row < S;
+    const int tile_of_wave = wave % 2;
+    const int column_half = wave / 2;
 
-    const size_t qk_stride = (size_t)heads * DQK;
-    const size_t v_stride = (size_t)heads * DV;
-    const bf16_t* q_base = query + ((size_t)b * S * heads + h) * DQK;
-    const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
-    const bf16_t* v_base = value + ((size_t)b * S * heads + h) * DV;
-    const bf16_t* do_base = output_gradient + ((size_t)b * S * heads + h) * DV;
+    const unsigned k_stride_bytes = (unsigned)heads * DQK * 2;
+    const unsigned char* k_base = reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * heads + h) * DQK);
+    const unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+    const unsigned lds_base = lds_offset_of(lds);
 
-    // Q and dO rows of this wave as B operands (column = query lq)
-    bf16x8 qf[QK_STEPS], dof[V_STEPS];
-    load_row_fragments<DQK>(qf, q_base, qk_stride, q_row, valid, g);
-    load_row_fragments<DV>(dof, do_base, v_stride, q_row, valid, g);
-    const float lse2 = valid ? logsumexp[((size_t)b * heads + h) * S + q_row] * LOG2E : 0.f;
-    const float row_delta = valid ? delta[((size_t)b * heads + h) * S + q_row] : 0.f;
+    // query tiles of this workgroup (the second may not exist at a ragged end: it
+    // then repeats the first, and its rows are not stored)
+    int tile_index[2];
+    tile_index[0] = 2 * jb;
+    tile_index[1] = min(2 * jb + 1, query_tiles - 1);
 
-    f32x16 dq_acc[DQ_BLOCKS];
+    const int steps = 2 * (jb + 1);   // 64-key steps up to the end of key block jb
+    TileRequests<C::K_ROW> k_requests;
+    k_requests.init(k_stride_bytes, lane);
+    auto request_step = [&](int step, int stage) {
+        const int kb = step / 2;
+        const int half = step % 2;
+        const int row0 = kb * KBLOCK + half * C::STEP_KEYS;
+        const unsigned target = lds_base + stage * C::STAGE_BYTES;
+        // rows past the end of the sequence repeat the last one: their dS is zero
+        k_requests.request(k_base + (size_t)min(row0, S - 1) * k_stride_bytes, k_stride_bytes, max(S - 1 - row0, 0),
+                           target, wave);
 #pragma unroll
-    for (int d = 0; d < DQ_BLOCKS; ++d) clear(dq_acc[d]);
-
-    const float c = scale * LOG2E;
-    const int last_key = min(S, q0 + C::QUERIES) - 1;
-    const int tiles = last_key / BWD_TILE + 1;
-
-    u32x2 k_stage[KT::PER_THREAD][4];
-    u32x4 v_stage[C::V_PER_THREAD];
-    auto load_tile = [&](int tile) {
-        const int row0 = tile * BWD_TILE;
-        load_units<DQK>(k_stage, k_base, qk_stride, row0, S, tid);
-#pragma unroll
-        for (int i = 0; i < C::V_PER_THREAD; ++i) {
-            const int id = tid + BWD_THREADS * i;
-            const int row = row0 + id / (DV / 8);
-            u32x4 bits = {0, 0, 0, 0};
-            if (row < S) bits = *reinterpret_cast<const u32x4*>(v_base + (size_t)row * v_stride + 8 * (id % (DV / 8)));
-            v_stage[i] = bits;
-        }
-    };
-    auto store_tile = [&](int stage) {
-        unsigned char* base = lds + stage * C::STAGE_BYTES;
-        store_units<DQK, true, true>(k_stage, base + C::K_NATURAL, base + C::K_TRANSPOSED, tid);
-#pragma unroll
-        for (int i = 0; i < C::V_PER_THREAD; ++i) {
-            const int id = tid + BWD_THREADS * i;
-            *reinterpret_cast<u32x4*>(base + C::V_NATURAL + (id / (DV / 8)) * C::V_PITCH + 16 * (id % (DV / 8))) = v_stage[i];
+        for (int i = 0; i < 4; ++i) {
+            const int load = 4 * wave + i;   // 16 pieces of 1 KB: two query tiles x 8
+            const int t = load / 8;
+            const int part = load % 8;
+            const unsigned char* block =
+                ds_head + (size_t)ds_block_index(kb, tile_index[t], query_tiles) * DS_BLOCK_BYTES + half * C::DS_HALF;
+            direct_load_16_offset(block, (unsigned)(part * 1024 + lane * 16),
+                                  target + C::K_BYTES + t * C::DS_HALF + part * 1024);
         }
     };
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (int tile = 0; tile < tiles; ++tile) {
-        const int stage = tile & 1;
-        const bool more = tile + 1 < tiles;
-        if (more) load_tile(tile + 1);
-        const int key0 = tile * BWD_TILE;
-        if (key0 <= wave_q0 + 31) {
-            const unsigned char* base = lds + stage * C::STAGE_BYTES;
-            const unsigned char* k_natural = base + C::K_NATURAL;
-            const unsigned char* k_transposed = base + C::K_TRANSPOSED;
-            const unsigned char* v_natural = base + C::V_NATURAL;
+    f32x16 dq_acc[C::D_BLOCKS][2];
+#pragma unroll
+    for (int d = 0; d < C::D_BLOCKS; ++d) {
+        clear(dq_acc[d][0]);
+        clear(dq_acc[d][1]);
+    }
 
-            f32x16 s_acc[2], dp_acc[2];
+    // K^T operand (ds_read_b64_tr_b16 on the row-major K rows).  A wave's column
+    // blocks are 2*d + column_half, so the swizzle-dependent part of the address
+    // (block % TR) is fixed per wave up to d, and the rest is an immediate.
+    constexpr int TR = TileReads<C::K_ROW>::TR;
+    constexpr int SEL = TR / 2;
+    unsigned k_reads[2][SEL];
+    {
+        TileReads<C::K_ROW> reads;
+        reads.init(lane);
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
-                clear(s_acc[mb]);
-                clear(dp_acc[mb]);
+        for (int h2 = 0; h2 < 2; ++h2) {
+#pragma unroll
+            for (int j = 0; j < SEL; ++j) {
+                k_reads[h2][j] = column_half ? reads.transposed[h2][2 * j + 1] : reads.transposed[h2][2 * j];
+            }
+        }
+    }
+    // dS^T operand: column = query 32*qb + lane%32 of the tile, k = keys {4g.., 8+4g..}
+    // of a 16-key step; the bytes sit where the dK/dV kernel's lanes put them.  Lane s
+    // of a 16-lane group fetches the 8 bytes that hold queries 4*(s%4).. of key s/4
+    // (+8 for the second read): slot ((key%32 + 32*g') ^ (4*g' + 8*n)) of the 1 KB piece
+    // (key/32, qb, n), n = (lane/16)%2, g' = s%2, second half of the slot if (s%4)/2.
+    unsigned ds_reads[2];
+    {
+        const int s = lane % 16;
+        const int n = (lane / 16) % 2;
+        const int gp = s % 2;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            const int slot = s / 4 + 4 * (g ^ gp) + 8 * (h2 ^ n) + 32 * gp;
+            ds_reads[h2] = C::K_BYTES + tile_of_wave * C::DS_HALF + n * 1024 + 16 * slot + 8 * ((s % 4) / 2);
+        }
+    }
+
+    request_step(0, 0);
+    request_step(1, 1);   // steps >= 2 always
+    for (int step = 0; step < steps; ++step) {
+        wait_vector_memory<0>();
+        workgroup_barrier();
+        if (step + 2 < steps) {
+            request_step(step + 2, (step + 2) % 3);
+        }
+        const unsigned stage_offset = (step % 3) * C::STAGE_BYTES;
+        unsigned k_at[2][SEL], ds_at[2];
+        rebase(k_at, k_reads, stage_offset);
+        rebase(ds_at, ds_reads, stage_offset);
+#pragma unroll
+        for (int kk = 0; kk < C::STEP_KEYS / 16; ++kk) {
+            bf16x8 ds[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const int constant = (kk / 2) * 4096 + qb * 2048 + (kk % 2) * 256;
+                const s16x4 low =
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(lds + ds_at[0] + constant));
+                const s16x4 high =
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(lds + ds_at[1] + constant));
+                ds[qb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
             }
 #pragma unroll
-            for (int ks = 0; ks < QK_STEPS; ++ks) {
-#pragma unroll
-                for (int mb = 0; mb < 2; ++mb) {
-                    const bf16x8 a = natural_fragment<DQK>(k_natural, 32 * mb + lq, ks, g);
-                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s_acc[mb], 0, 0, 0);
-                }
+            for (int d = 0; d < C::D_BLOCKS; ++d) {
+                const int constant = 16 * kk * C::K_ROW + (d / SEL) * (TR * 64);
+                const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (transposing_read_pointer)(lds + k_at[0][d % SEL] + constant));
+                const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (transposing_read_pointer)(lds + k_at[1][d % SEL] + constant));
+                const bf16x8 kt =
+                    __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
+                dq_acc[d][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, ds[0], dq_acc[d][0], 0, 0, 0);
+                dq_acc[d][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, ds[1], dq_acc[d][1], 0, 0, 0);
             }
+        }
+    }
+
+    // ---- epilogue: lane holds query lq and columns 32*block + 8*(i/4) + 4*g + i%4
+    if (2 * jb + tile_of_wave < query_tiles) {
+        bf16_t* dq_base = query_gradient + ((size_t)b * S * heads + h) * DQK;
+        const size_t q_stride = (size_t)heads * DQK;
 #pragma unroll
-            for (int ks = 0; ks < V_STEPS; ++ks) {
+        for (int qb = 0; qb < 2; ++qb) {
+            const int q_row = (2 * jb + tile_of_wave) * QTILE + 32 * qb + lq;
+            if (q_row < S) {
 #pragma unroll
-                for (int mb = 0; mb < 2; ++mb) {
-                    const bf16x8 a = *reinterpret_cast<const bf16x8*>(v_natural + (32 * mb + lq) * C::V_PITCH + 32 * ks + 16 * g);
-                    dp_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dof[ks], dp_acc[mb], 0, 0, 0);
-                }
-            }
-            // lane holds query lq and keys key0 + 32*mb + 8*(i/4) + 4*g + i%4
-            const bool diagonal = key0 + BWD_TILE - 1 > wave_q0;
-            bf16x8 dsf[4];
+                for (int d = 0; d < C::D_BLOCKS; ++d) {
+                    const int column0 = 32 * (2 * d + column_half);
 #pragma unroll
-            for (int n = 0; n < 4; ++n) {
-                u32x4 packed;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = 8 * (n % 2) + 2 * j;
-                    float ds[2];
-#pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[n / 2][i + e], c, -lse2));
-                        const int k = key0 + 32 * (n / 2) + 8 * ((i + e) / 4) + 4 * g + (i + e) % 4;
-                        if (diagonal && k > q_row) probability = 0.f;
-                        ds[e] = probability * (dp_acc[n / 2][i + e] - row_delta) * scale;
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        u32x2 packed;
+                        packed.x = pack_bf16(dq_acc[d][qb][4 * i4 + 0] * scale, dq_acc[d][qb][4 * i4 + 1] * scale);
+                        packed.y = pack_bf16(dq_acc[d][qb][4 * i4 + 2] * scale, dq_acc[d][qb][4 * i4 + 3] * scale);
+                        *reinterpret_cast<u32x2*>(dq_base + (size_t)q_row * q_stride + column0 + 8 * i4 + 4 * g) = packed;
                     }
-                    packed[j] = pack_bf16(ds[0], ds[1]);
-                }
-                dsf[n] = __builtin_bit_cast(bf16x8, packed);
-            }
-            // dQ^T += K^T dS^T (contraction over the 64 keys)
-#pragma unroll
-            for (int n = 0; n < 4; ++n) {
-#pragma unroll
-                for (int d = 0; d < DQ_BLOCKS; ++d) {
-                    const bf16x8 a = transposed_fragment<DQK>(k_transposed, 32 * d + lq, n, g);
-                    dq_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsf[n], dq_acc[d], 0, 0, 0);
                 }
             }
-        }
-        if (more) store_tile(stage ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue: lane holds query lq and columns 32*d + 8*(i/4) + 4*g + i%4
-    unsigned char* dq_lds = lds + (32 * wave) * C::DQ_PITCH;
-#pragma unroll
-    for (int d = 0; d < DQ_BLOCKS; ++d) {
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-            u32x2 packed;
-            packed.x = pack_bf16(dq_acc[d][4 * i4 + 0], dq_acc[d][4 * i4 + 1]);
-            packed.y = pack_bf16(dq_acc[d][4 * i4 + 2], dq_acc[d][4 * i4 + 3]);
-            *reinterpret_cast<u32x2*>(dq_lds + lq * C::DQ_PITCH + 2 * (32 * d + 8 * i4 + 4 * g)) = packed;
-        }
-    }
-    __syncthreads();
-    bf16_t* dq_base = query_gradient + ((size_t)b * S * heads + h) * DQK;
-    for (int index = lane; index < 32 * (DQK / 8); index += 64) {
-        const int row = index / (DQK / 8);
-        const int chunk = index % (DQK / 8);
-        if (wave_q0 + row < S) {
-            const u32x4 bits = *reinterpret_cast<const u32x4*>(dq_lds + row * C::DQ_PITCH + 16 * chunk);
-            *reinterpret_cast<u32x4*>(dq_base + (size_t)(wave_q0 + row) * qk_stride + 8 * chunk) = bits;
         }
     }
 }
@@ -596,50 +900,81 @@ void raise_lds_limit(Kernel kernel, int bytes) {
     }
 }
 
+struct BackwardShape {
+    int key_blocks;
+    int query_tiles;
+    int query_blocks;
+    long long statistics_floats;   // per launch
+    long long ds_floats;
+};
+
+BackwardShape backward_shape(int batch_size, int sequence_length, int heads) {
+    BackwardShape shape;
+    shape.key_blocks = (sequence_length + KBLOCK - 1) / KBLOCK;
+    shape.query_tiles = (sequence_length + QTILE - 1) / QTILE;
+    shape.query_blocks = shape.key_blocks;   // 128 queries per workgroup of the dQ pass
+    const long long groups = (long long)batch_size * heads;
+    shape.statistics_floats = groups * shape.query_tiles * STAT_FLOATS;
+    shape.ds_floats = groups * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_FLOATS;
+    return shape;
+}
+
 template <int DQK, int DV>
 void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value_gradient,
                      const bf16_t* output_gradient, const bf16_t* output, const float* logsumexp,
-                     const bf16_t* query, const bf16_t* key, const bf16_t* value, float* delta, int batch_size,
+                     const bf16_t* query, const bf16_t* key, const bf16_t* value, float* workspace, int batch_size,
                      int sequence_length, int heads, float scale, hipStream_t stream) {
-    using KC = KeyGradConfig<DQK, DV>;
-    using QC = QueryGradConfig<DQK, DV>;
-    const long long rows = (long long)batch_size * sequence_length * heads;
+    using KC = KeyValueGradConfig<DQK, DV>;
+    using QC = QueryGradConfig<DQK>;
+    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads);
     const long long groups = (long long)batch_size * heads;
-    const int key_blocks = (sequence_length + KC::KEYS - 1) / KC::KEYS;
-    const int query_blocks = (sequence_length + QC::QUERIES - 1) / QC::QUERIES;
-    if ((rows + 15) / 16 > 0x7fffffffLL || groups * key_blocks > 0x7fffffffLL) {
+    const long long padded_rows = groups * shape.query_tiles * QTILE;
+    if ((padded_rows + 15) / 16 > 0x7fffffffLL || groups * shape.key_blocks > 0x7fffffffLL) {
         throw std::invalid_argument("attention backward: problem exceeds the grid limit");
     }
+    // per-lane byte offsets inside a tile are 32-bit
+    if ((long long)heads * (DQK > DV ? DQK : DV) * 2 * QTILE > 0x7fffffffLL) {
+        throw std::invalid_argument("attention backward: heads * head size is too large");
+    }
+    float* statistics = workspace;
+    unsigned char* ds_blocks = reinterpret_cast<unsigned char*>(workspace + shape.statistics_floats);
     static thread_local bool prepared = false;
     if (!prepared) {
-        raise_lds_limit(attention_key_gradient_kernel<DQK, DV>, KC::LDS_BYTES);
-        raise_lds_limit(attention_query_gradient_kernel<DQK, DV>, QC::LDS_BYTES);
+        raise_lds_limit(attention_key_value_gradient_kernel<DQK, DV>, KC::LDS_BYTES);
+        raise_lds_limit(attention_query_gradient_kernel<DQK>, QC::LDS_BYTES);
         prepared = true;
     }
-    hipLaunchKernelGGL((attention_delta_kernel<DV>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream, delta,
-                       output_gradient, output, batch_size, sequence_length, heads);
+    hipLaunchKernelGGL((attention_backward_statistics_kernel<DV>), dim3((unsigned)((padded_rows + 15) / 16)), dim3(256),
+                       0, stream, statistics, output_gradient, output, logsumexp, batch_size, sequence_length, heads,
+                       shape.query_tiles);
     HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL((attention_key_gradient_kernel<DQK, DV>), dim3((unsigned)(groups * key_blocks)),
-                       dim3(BWD_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, output_gradient,
-                       logsumexp, delta, query, key, value, sequence_length, heads, key_blocks, scale);
+    hipLaunchKernelGGL((attention_key_value_gradient_kernel<DQK, DV>), dim3((unsigned)(groups * shape.key_blocks)),
+                       dim3(BWD_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
+                       output_gradient, query, key, value, sequence_length, heads, shape.key_blocks,
+                       shape.query_tiles, scale);
     HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL((attention_query_gradient_kernel<DQK, DV>), dim3((unsigned)(groups * query_blocks)),
-                       dim3(BWD_THREADS), QC::LDS_BYTES, stream, query_gradient, output_gradient, logsumexp, delta,
-                       query, key, value, sequence_length, heads, query_blocks, scale);
+    hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>), dim3((unsigned)(groups * shape.query_blocks)),
+                       dim3(BWD_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
+                       heads, shape.query_blocks, shape.key_blocks, shape.query_tiles, scale);
     HIP_CHECK(hipGetLastError());
 }
 
 }  // namespace
 
+std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads) {
+    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads);
+    return static_cast<std::size_t>(shape.statistics_floats + shape.ds_floats);
+}
+
 void attention_backward_dispatch(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value_gradient,
                                  const bf16_t* output_gradient, const bf16_t* output, const float* logsumexp,
-                                 const bf16_t* query, const bf16_t* key, const bf16_t* value, float* delta,
+                                 const bf16_t* query, const bf16_t* key, const bf16_t* value, float* workspace,
                                  int batch_size, int sequence_length, int heads, int qk_head_size, int v_head_size,
                                  float scale, hipStream_t stream) {
 #define DSCUDA_BWD_CASE(DQK, DV)                                                                                   \
     if (qk_head_size == DQK && v_head_size == DV) {                                                                \
         launch_backward<DQK, DV>(query_gradient, key_gradient, value_gradient, output_gradient, output, logsumexp, \
-                                 query, key, value, delta, batch_size, sequence_length, heads, scale, stream);      \
+                                 query, key, value, workspace, batch_size, sequence_length, heads, scale, stream);  \
         return;                                                                                                    \
     }
     DSCUDA_BWD_CASE(192, 128)

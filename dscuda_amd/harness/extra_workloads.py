@@ -22,13 +22,13 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3)
     # MLA backward, same shape, dO ~ N(0,1) seed 2
     dout = configs.mla_prefill_dout(batch, seq, heads, dv, seed=2).to(device)
     grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
-    workspace = torch.empty(batch * heads * seq, device=device, dtype=torch.float32)
+    workspace = ops.mla_prefill_backward_workspace(batch, seq, heads, dqk, dv, device)
     ms, _ = event_time_ms(lambda: ops.mla_prefill_backward(dout, out, lse, q, k, v, scale, workspace, grads),
                           steps, warmup)
     flops = configs.backward_flops(batch, heads, seq, dqk, dv)
     results["mla_backward_S4096_H128"] = {
         "ms": ms, "tflops": flops / ms / 1e9, "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS,
-        "flops": flops, "kernels": "attention_delta + attention_key_gradient + attention_query_gradient"}
+        "flops": flops, "kernels": "attention_backward_statistics + attention_key_value_gradient + attention_query_gradient"}
     del dout, grads, workspace
 
     # absorbed decode, B=64 H=128, lengths ~ U[1024,8192] seed 3, 64-token pages

@@ -89,6 +89,13 @@ def mla_prefill_forward(query, key, value, scale, out=None, lse=None):
     return out, lse
 
 
+def mla_prefill_backward_workspace(batch, seq, heads, dqk, dv, device="cuda"):
+    """fp32 workspace of the per-head backward: row statistics plus the bf16 dS blocks
+    that the dK/dV kernel hands to the dQ pass (about S^2 bytes per head)."""
+    elements = mla_library().prefill_workspace(batch, seq, heads, dqk, dv)
+    return torch.empty(elements, device=device, dtype=torch.float32)
+
+
 def mla_prefill_backward(dout, out, lse, query, key, value, scale, workspace=None, grads=None):
     """-> (dQ, dK [B,S,H,d_qk], dV [B,S,H,d_v]) bf16, overwritten."""
     _require_cuda(dout, out, lse, query, key, value)
@@ -96,7 +103,7 @@ def mla_prefill_backward(dout, out, lse, query, key, value, scale, workspace=Non
     dv = value.shape[-1]
     lib = mla_library()
     if workspace is None:
-        workspace = torch.empty(lib.prefill_workspace(b, s, h, dqk, dv), device=query.device, dtype=torch.float32)
+        workspace = mla_prefill_backward_workspace(b, s, h, dqk, dv, query.device)
     if grads is None:
         grads = (torch.empty_like(query), torch.empty_like(key), torch.empty_like(value))
     checked(lib.lib, "mla", lib.prefill_backward(

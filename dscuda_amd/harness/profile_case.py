@@ -55,7 +55,7 @@ def main():
         else:
             dout = randn((1, s, h, 128), 1.0)
             grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
-            workspace = torch.empty(h * s, device=device)
+            workspace = ops.mla_prefill_backward_workspace(1, s, h, 192, 128, device)
             call = lambda: ops.mla_prefill_backward(dout, out, lse, q, k, v, scale, workspace, grads)
     elif args.workload == "decode":
         lengths, _ = configs.decode_lengths()

@@ -47,7 +47,11 @@ def test_workspace_elements_match_the_reference_formula():
     assert size(64, 128, 8, 512) == 64 * 128 * 8 * 514
     assert size(4096, 128, 64, 512) == 4096 * 128 * 64 * 514  # needs size_t
     prefill = bind(lib, "dscuda_mla_prefill_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
-    assert prefill(1, 4096, 128, 192, 128) == 4096 * 128
+    # per (batch, head): 128 floats of row statistics per 64-query tile, plus one 16 KB bf16 dS
+    # block (4096 floats) per (128-key block, 64-query tile) pair on or below the diagonal
+    assert prefill(1, 4096, 128, 192, 128) == 128 * (64 * 128 + (32 * 64 - 32 * 31) * 4096)
+    assert prefill(2, 65, 3, 192, 128) == 2 * 3 * (2 * 128 + 2 * 4096)   # ragged: 1 key block, 2 query tiles
+    assert prefill(0, 65, 3, 192, 128) == 0
 
 
 def _status_and_message(lib, prefix, status):
