@@ -10,8 +10,8 @@
 //
 //   statistics   per query row: LSE * log2(e) and delta = sum_c dO * O, stored per
 //                64-query tile (padding rows carry LSE = +inf, so they weigh nothing)
-//   dK/dV        a workgroup owns 128 keys (4 waves x 32, K and V rows in registers)
-//                and walks the 64-query tiles from the diagonal to the end:
+//   dK/dV        a workgroup owns 128 keys and walks the 64-query tiles from the
+//                diagonal to the end:
 //                    S = Q K^T, dP = dO V^T          (queries x keys)
 //                    dV += P^T dO,  dK += dS^T Q
 //                and leaves dS (bf16, before the scale factor) in the workspace,
@@ -82,24 +82,28 @@ __device__ __forceinline__ void direct_load_4_offset(const void* uniform_base, u
                  : "memory", "m0");
 }
 
-// This wave's share of the global_load_lds requests of a [64][ROW_BYTES] tile.
-// LDS slot 64*load + lane (16 bytes each) holds chunk (slot % CHUNKS) ^ f(row) of
-// row slot / CHUNKS.  PERIOD loads cover PERIOD_ROWS whole rows; from one period
-// to the next only the low bits of f change, so load L = PERIOD*m + r reads at
-//     tile + m * PERIOD_ROWS * row_stride  +  (base[r] ^ 16 * (m % XOR_STEPS))
-// with one per-lane value per r.  A wave's LOADS consecutive loads start at a
-// multiple of PERIOD * XOR_STEPS, so r and the XOR term are compile-time.  At a
-// ragged end rows past `row_limit` repeat that row (slow path).
-template <int ROW_BYTES>
+// One wave's share of the global_load_lds requests of a [64][ROW_BYTES] tile that
+// WAVES waves fetch together.  LDS slot 64*load + lane (16 bytes each) holds chunk
+// (slot % CHUNKS) ^ f(row) of row slot / CHUNKS.  PERIOD loads cover PERIOD_ROWS
+// whole rows; from one period to the next only the low bits of f change, so load
+// L = PERIOD*m + r reads at
+//     tile + m * PERIOD_ROWS * row_stride  +  (offset of load r) ^ 16 * (m % XOR_STEPS)
+// The periods of a wave's LOADS consecutive loads are m = wave * LOADS/PERIOD + j;
+// LOADS/PERIOD and XOR_STEPS are powers of two, so the two parts of m touch
+// different bits of the XOR term: the wave's part is folded into base[r] once and
+// j's part is a compile-time constant.  At a ragged end rows past `row_limit`
+// repeat that row (slow path).
+template <int ROW_BYTES, int WAVES>
 struct TileRequests {
     static constexpr int CHUNKS = ROW_BYTES / 16;
-    static constexpr int LOADS = QTILE * ROW_BYTES / 1024 / (BWD_THREADS / 64);
+    static constexpr int LOADS = QTILE * ROW_BYTES / 1024 / WAVES;
     static constexpr int PERIOD = CHUNKS == 24 ? 3 : 1;
     static constexpr int PERIOD_ROWS = 64 * PERIOD / CHUNKS;
     static constexpr int XOR_STEPS = CHUNKS == 16 ? 4 : 2;
+    static constexpr int PERIODS = LOADS / PERIOD;   // per wave
     static_assert(CHUNKS == 8 || CHUNKS == 16 || CHUNKS == 24, "rows of 128, 256 or 384 bytes");
-    static_assert(QTILE * ROW_BYTES % (1024 * (BWD_THREADS / 64)) == 0, "tile must divide evenly over the waves");
-    static_assert(LOADS % (PERIOD * XOR_STEPS) == 0, "a wave's loads must start at a whole swizzle period");
+    static_assert(QTILE * ROW_BYTES % (1024 * WAVES) == 0 && LOADS % PERIOD == 0, "tile must divide evenly over the waves");
+    static_assert(PERIODS == 1 || PERIODS == 2 || PERIODS == 4, "periods per wave must be a power of two");
     unsigned base[PERIOD];
 
     __device__ __forceinline__ static unsigned offset_of(int load, int lane, unsigned row_stride, int row_limit) {
@@ -108,15 +112,17 @@ struct TileRequests {
         const int chunk = (slot % CHUNKS) ^ tile_swizzle<ROW_BYTES>(row);
         return (unsigned)min(row, row_limit) * row_stride + 16u * chunk;
     }
-    __device__ __forceinline__ void init(unsigned row_stride, int lane) {
+    __device__ __forceinline__ void init(unsigned row_stride, int wave, int lane) {
 #pragma unroll
-        for (int r = 0; r < PERIOD; ++r) base[r] = offset_of(r, lane, row_stride, QTILE);
+        for (int r = 0; r < PERIOD; ++r) {
+            base[r] = offset_of(r, lane, row_stride, QTILE) ^ (16u * ((wave * PERIODS) % XOR_STEPS));
+        }
     }
     // `tile` = address of the tile's first row (uniform)
     __device__ __forceinline__ void request(const unsigned char* tile, unsigned row_stride, int row_limit,
                                             unsigned lds_target, int wave) const {
         if (row_limit >= QTILE - 1) {
-            const unsigned char* rows = tile + (size_t)(wave * LOADS / PERIOD * PERIOD_ROWS) * row_stride;
+            const unsigned char* rows = tile + (size_t)(wave * PERIODS * PERIOD_ROWS) * row_stride;
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 direct_load_16_offset(rows + (size_t)(i / PERIOD * PERIOD_ROWS) * row_stride,
@@ -210,18 +216,24 @@ __device__ __forceinline__ void static_for(F&& f) {
 __host__ __device__ constexpr bool score_slot_is_s(int k, int v_steps) { return k >= 2 * v_steps || k % 2 == 0; }
 __host__ __device__ constexpr int score_slot_step(int k, int v_steps) { return k >= 2 * v_steps ? k - v_steps : k / 2; }
 
-// at = reads + offset
+// at = reads + offset, as values the optimiser cannot take apart again: the
+// fragment reads then keep the form (per-lane register) + (immediate) instead of
+// one address computation per read.
+__device__ __forceinline__ unsigned opaque(unsigned value) {
+    asm volatile("" : "+v"(value));
+    return value;
+}
 template <int N>
 __device__ __forceinline__ void rebase(unsigned (&at)[N], const unsigned (&reads)[N], unsigned offset) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) at[i] = reads[i] + offset;
+    for (int i = 0; i < N; ++i) at[i] = opaque(reads[i] + offset);
 }
 template <int N>
 __device__ __forceinline__ void rebase(unsigned (&at)[2][N], const unsigned (&reads)[2][N], unsigned offset) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
-        for (int i = 0; i < N; ++i) at[h][i] = reads[h][i] + offset;
+        for (int i = 0; i < N; ++i) at[h][i] = opaque(reads[h][i] + offset);
     }
 }
 
@@ -298,6 +310,28 @@ __global__ __launch_bounds__(256) void attention_backward_statistics_kernel(
 }
 
 // ---- dK / dV (and dS) -----------------------------------------------------------
+//
+// Eight waves, two per SIMD.  Waves g and g + 4 (g = 0..3, the same SIMD) share the
+// 32 keys of group g and split the work of a tile by product:
+//
+//   value wave (g)      S = Q K^T (K rows in registers)  ->  P = exp2(S c - LSE)
+//                       ->  dV += P^T dO;  P goes to the key wave through LDS
+//   key wave (g + 4)    dP = dO V^T (V rows in registers)  ->  dS = P (dP - delta)
+//                       ->  dK += dS^T Q;  dS goes to the workspace
+//
+// A wave cannot overlap its own MFMAs with its own vector arithmetic, but the two
+// waves of a SIMD can: the key wave runs one tile behind and in the opposite order
+// (arithmetic first), so while one wave forms probabilities the other feeds the
+// matrix pipeline.  One workgroup barrier per tile keeps the pair, the tile stages
+// and the P hand-over in step:
+//
+//   iteration i    value wave: S(i) | P(i) -> LDS | dV(i)
+//                  key wave:   dS(i-1) from P(i-1), dP(i-1) | dK(i-1) | dP(i)
+//
+// Tile i lives in stage i % 3 and is requested one iteration ahead; P(i) lives in
+// hand-over buffer i % 2 of its key group.
+
+constexpr int KV_THREADS = 512;
 
 template <int DQK, int DV>
 struct KeyValueGradConfig {
@@ -308,15 +342,17 @@ struct KeyValueGradConfig {
     static constexpr int STAT_BYTES = STAT_FLOATS * 4;
     static constexpr int STAGE_BYTES = Q_BYTES + O_BYTES + STAT_BYTES;
     static constexpr int STAGES = 3;
-    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int P_BYTES = QTILE * 32 * 2;                  // P of one tile and key group, bf16
+    static constexpr int HANDOVER_AT = STAGES * STAGE_BYTES;
+    static constexpr int LDS_BYTES = HANDOVER_AT + 4 * 2 * P_BYTES;  // 4 key groups x 2 buffers
     static constexpr int DK_PITCH = 2 * DQK;   // epilogue staging
     static constexpr int DV_PITCH = 2 * DV;
-    static_assert(4 * 32 * (DK_PITCH + DV_PITCH) <= LDS_BYTES, "epilogue staging must fit");
+    static_assert(4 * 32 * (DK_PITCH + DV_PITCH) <= HANDOVER_AT, "epilogue staging must fit");
     static_assert(LDS_BYTES <= 160 * 1024, "stages must fit the LDS");
 };
 
 template <int DQK, int DV>
-__global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kernel(
+__global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kernel(
     bf16_t* __restrict__ key_gradient, bf16_t* __restrict__ value_gradient, unsigned char* __restrict__ ds_blocks,
     const float* __restrict__ statistics, const bf16_t* __restrict__ output_gradient,
     const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
@@ -326,11 +362,14 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kern
     constexpr int V_STEPS = DV / 16;
     constexpr int DK_BLOCKS = DQK / 32;
     constexpr int DV_BLOCKS = DV / 32;
+    constexpr int WAVES = KV_THREADS / 64;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const bool key_wave = wave >= 4;
+    const int group = wave % 4;
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
@@ -341,8 +380,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kern
     const int b = bh / heads;
     const int h = bh % heads;
     const int k0 = kb * KBLOCK;
-    const int wave_k0 = k0 + 32 * wave;
-    const int key_row = wave_k0 + lq;
+    const int group_k0 = k0 + 32 * group;
+    const int key_row = group_k0 + lq;
 
     const size_t qk_stride = (size_t)heads * DQK;
     const size_t v_stride = (size_t)heads * DV;
@@ -351,37 +390,21 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kern
     const unsigned char* q_base = reinterpret_cast<const unsigned char*>(query + ((size_t)b * S * heads + h) * DQK);
     const unsigned char* do_base =
         reinterpret_cast<const unsigned char*>(output_gradient + ((size_t)b * S * heads + h) * DV);
-    const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
-    const bf16_t* v_base = value + ((size_t)b * S * heads + h) * DV;
     const float* stat_base = statistics + (size_t)bh * query_tiles * STAT_FLOATS;
-    unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
     const unsigned lds_base = lds_offset_of(lds);
 
-    // K and V rows of this wave, as B operands (column = key lq)
-    bf16x8 kf[QK_STEPS], vf[V_STEPS];
-    load_row_fragments<DQK>(kf, k_base, qk_stride, key_row, key_row < S, g);
-    load_row_fragments<DV>(vf, v_base, v_stride, key_row, key_row < S, g);
-
-    f32x16 dk_acc[DK_BLOCKS], dv_acc[DV_BLOCKS];
-#pragma unroll
-    for (int d = 0; d < DK_BLOCKS; ++d) clear(dk_acc[d]);
-#pragma unroll
-    for (int d = 0; d < DV_BLOCKS; ++d) clear(dv_acc[d]);
-
-    const float c = scale * LOG2E;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int first_tile = 2 * kb;
     const int tiles = query_tiles - first_tile;   // >= 1
 
-    TileRequests<C::Q_ROW> q_requests;
-    TileRequests<C::O_ROW> o_requests;
-    q_requests.init(q_stride_bytes, lane);
-    o_requests.init(o_stride_bytes, lane);
-    auto request_tile = [&](int index, int stage) {
+    TileRequests<C::Q_ROW, WAVES> q_requests;
+    TileRequests<C::O_ROW, WAVES> o_requests;
+    q_requests.init(q_stride_bytes, wave, lane);
+    o_requests.init(o_stride_bytes, wave, lane);
+    auto request_tile = [&](int index) {
         const int tile = first_tile + index;
         const int row0 = tile * QTILE;
         const int row_limit = S - 1 - row0;
-        const unsigned target = lds_base + stage * C::STAGE_BYTES;
+        const unsigned target = lds_base + (index % 3) * C::STAGE_BYTES;
         q_requests.request(q_base + (size_t)row0 * q_stride_bytes, q_stride_bytes, row_limit, target, wave);
         o_requests.request(do_base + (size_t)row0 * o_stride_bytes, o_stride_bytes, row_limit, target + C::Q_BYTES, wave);
         if (wave < 2) {
@@ -390,325 +413,217 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_key_value_gradient_kern
         }
     };
 
-    // per-lane read offsets inside a stage, and their per-stage instances
+    // per-lane read offsets inside a stage
     TileReads<C::Q_ROW> q_reads;
     TileReads<C::O_ROW> o_reads;
     q_reads.init(lane);
     o_reads.init(lane);
-    struct ScoreReads {
-        unsigned q[TileReads<C::Q_ROW>::NAT];
-        unsigned o[TileReads<C::O_ROW>::NAT];
-    };
-    struct GradientReads {
-        unsigned q[2][TileReads<C::Q_ROW>::TR];
-        unsigned o[2][TileReads<C::O_ROW>::TR];
-    };
-    auto score_reads = [&](ScoreReads& at, int stage) {
-        rebase(at.q, q_reads.natural, stage * C::STAGE_BYTES);
-        rebase(at.o, o_reads.natural, stage * C::STAGE_BYTES + C::Q_BYTES);
-    };
-    auto gradient_reads = [&](GradientReads& at, int stage) {
-        rebase(at.q, q_reads.transposed, stage * C::STAGE_BYTES);
-        rebase(at.o, o_reads.transposed, stage * C::STAGE_BYTES + C::Q_BYTES);
-    };
-    auto stats_of = [&](int stage) -> unsigned { return stage * C::STAGE_BYTES + C::Q_BYTES + C::O_BYTES + 16 * g; };
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // hand-over buffers of this key group: P as the value wave's registers hold it,
+    // piece (query half, 16-query step) of 1 KB, 16 bytes per lane
+    const unsigned handover = C::HANDOVER_AT + group * 2 * C::P_BYTES + 16 * lane;
 
-    // Half tiles.  The unit of the software pipeline is half a tile (32 queries):
-    //     S, dP (SCORE_MFMAS) -> P, dS (VALU) -> dV, dK (GRAD_MFMAS).
-    // Half j keeps its scores in set j%2 of (s_acc, dp_acc) and its operands in
-    // set j%2 of (pf, dsf).  One "half step" issues, as a single stream of MFMA
-    // slots, the gradient products of half j and the score products of half j + 2,
-    // with the probabilities of half j + 1 cut into small pieces that follow the
-    // MFMAs one by one: the three jobs touch disjoint registers, and a wave then
-    // keeps the matrix pipeline fed from its own instruction stream (a 32x32x16
-    // MFMA occupies it for 32 clocks, enough for seven other instructions).
-    // Every MFMA takes one fragment from LDS; the fragments run through a ring of
-    // RING register sets, read RING slots ahead -- across half steps and across
-    // the barrier between tiles (the tile read ahead has landed one tile earlier).
-    // All slot, set and register indices are compile-time constants.
-    constexpr int RING = 8;
-    constexpr int PER_STEP = DV_BLOCKS + DK_BLOCKS;        // gradient MFMAs per 16 queries
-    constexpr int GRAD_MFMAS = 2 * PER_STEP;
-    constexpr int SCORE_MFMAS = QK_STEPS + V_STEPS;
-    constexpr int PIECES = 20;                             // of the probabilities of one half
-    constexpr int PIECE_DELAY = 2;                         // slots before the first piece: the scores it reads
-                                                           // were finished by the last MFMA of the previous half step
-    static_assert(GRAD_MFMAS >= RING, "the fragments read ahead must all belong to the gradient products");
-    static_assert(QK_STEPS >= V_STEPS, "score slots alternate S and dP while dP lasts");
+    request_tile(0);
 
-    f32x16 s_acc[2], dp_acc[2];
-    u32x4 pf[2][2], dsf[2][2];   // [set][16-query step]: packed bf16 operands
-    bf16x8 ring[RING];
-    f32x4 lse4[2], delta4[2];    // two sets: a group of four queries is loaded while the previous one is used
-    float p[4], ds[4];
+    if (!key_wave) {
+        // ================= value wave: S, P, dV =================
+        const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
+        bf16x8 kf[QK_STEPS];   // B operand: column = key lq
+        load_row_fragments<DQK>(kf, k_base, qk_stride, key_row, key_row < S, g);
+        f32x16 dv_acc[DV_BLOCKS];
+#pragma unroll
+        for (int d = 0; d < DV_BLOCKS; ++d) clear(dv_acc[d]);
+        const float c = scale * LOG2E;
 
-    // fragment of gradient slot K (K < GRAD_MFMAS) of query half QB
-    auto gradient_fragment = [&](const GradientReads& at, auto qb_tag, auto k_tag) -> bf16x8 {
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int K = decltype(k_tag)::value;
-        constexpr int N = K / PER_STEP;
-        constexpr int R = K % PER_STEP;
-        if constexpr (R < DV_BLOCKS) {
-            return transposed_fragment<C::O_ROW, 32 * QB + 16 * N, R>(lds, at.o);
-        } else {
-            return transposed_fragment<C::Q_ROW, 32 * QB + 16 * N, R - DV_BLOCKS>(lds, at.q);
-        }
-    };
-    // score slot K: S and dP steps alternate while dP lasts (two independent chains)
-    auto score_fragment = [&](const ScoreReads& at, auto qb_tag, auto k_tag) -> bf16x8 {
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int K = decltype(k_tag)::value;
-        if constexpr (score_slot_is_s(K, V_STEPS)) {
-            return natural_fragment<C::Q_ROW, 32 * QB, score_slot_step(K, V_STEPS)>(lds, at.q);
-        } else {
-            return natural_fragment<C::O_ROW, 32 * QB, score_slot_step(K, V_STEPS)>(lds, at.o);
-        }
-    };
-    auto score_mfma = [&](auto qb_tag, auto k_tag, bf16x8 fragment) {
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int K = decltype(k_tag)::value;
-        constexpr int STEP = score_slot_step(K, V_STEPS);
-        if constexpr (score_slot_is_s(K, V_STEPS)) {
-            s_acc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[STEP], STEP == 0 ? zero : s_acc[QB], 0, 0, 0);
-        } else {
-            dp_acc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, vf[STEP], STEP == 0 ? zero : dp_acc[QB], 0, 0, 0);
-        }
-    };
-    auto gradient_mfma = [&](auto qb_tag, auto k_tag, bf16x8 fragment) {
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int K = decltype(k_tag)::value;
-        constexpr int N = K / PER_STEP;
-        constexpr int R = K % PER_STEP;
-        if constexpr (R < DV_BLOCKS) {
-            dv_acc[R] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[QB][N]), fragment,
-                                                                dv_acc[R], 0, 0, 0);
-        } else {
-            dk_acc[R - DV_BLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, dsf[QB][N]),
-                                                                            fragment, dk_acc[R - DV_BLOCKS], 0, 0, 0);
-        }
-    };
-
-    // statistics of queries 32*QB + 8*I4 + 4*g + (0..3) (stats_at carries the 16*g)
-    auto load_statistics = [&](unsigned stats_at, auto qb_tag, auto i4_tag) {
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int I4 = decltype(i4_tag)::value;
-        lse4[I4 % 2] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
-        delta4[I4 % 2] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (QTILE + 32 * QB + 8 * I4));
-    };
-    // Piece V (0..19) of the probabilities of half QB: lane holds key lq and queries
-    // 32*QB + 8*I4 + 4*g + E, I4 = V/5; pieces 5*I4 + E do element E (and the first of
-    // them requests the statistics of the next four queries), piece 5*I4 + 4 packs
-    // the four.  `threshold` = key_row - 4*g - q0: a query with local index below it
-    // lies before this lane's key.
-    auto probability_piece = [&](auto masked_tag, auto qb_tag, auto v_tag, unsigned stats_at, int threshold) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        constexpr int QB = decltype(qb_tag)::value;
-        constexpr int V = decltype(v_tag)::value;
-        constexpr int I4 = V / 5;
-        constexpr int E = V % 5;
-        if constexpr (E == 0 && I4 + 1 < 4) {
-            load_statistics(stats_at, qb_tag, std::integral_constant<int, (I4 + 1) % 4>{});
-        }
-        if constexpr (E < 4) {
-            constexpr int I = 4 * I4 + E;
-            p[E] = __builtin_amdgcn_exp2f(fmaf(accumulator_element<I>(s_acc[QB]), c, -lse4[I4 % 2][E]));
-            if (MASKED && 32 * QB + 8 * I4 + E < threshold) {
-                p[E] = 0.f;
+        for (int index = 0; index <= tiles; ++index) {
+            wait_vector_memory<0>();   // this wave's share of tile `index` has landed
+            workgroup_barrier();       // ... and everybody's; every wave has left tile index - 2
+            if (index + 1 < tiles) {
+                request_tile(index + 1);
             }
-            ds[E] = p[E] * (accumulator_element<I>(dp_acc[QB]) - delta4[I4 % 2][E]);
-        } else {
-            constexpr int N = I4 / 2;
-            constexpr int HALF = I4 % 2;
-            pf[QB][N][2 * HALF] = pack_bf16(p[0], p[1]);
-            pf[QB][N][2 * HALF + 1] = pack_bf16(p[2], p[3]);
-            dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
-            dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
-        }
-    };
+            if (index < tiles) {
+                const unsigned stage = (index % 3) * C::STAGE_BYTES;
+                unsigned q_at[TileReads<C::Q_ROW>::NAT], o_at[2][TileReads<C::O_ROW>::TR];
+                rebase(q_at, q_reads.natural, stage);
+                rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
+                const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g);
 
-    // dS of half QB of tile `index` to its block: 16 bytes per lane, slot
-    // (lane ^ (4g + 8n)) of the 1 KB piece (wave, QB, n)
-    auto store_ds = [&](int index, auto qb_tag) {
-        constexpr int QB = decltype(qb_tag)::value;
-        unsigned char* block = ds_head + (size_t)ds_block_index(kb, first_tile + index, query_tiles) * DS_BLOCK_BYTES;
-        *reinterpret_cast<u32x4*>(block + ((wave * 2 + QB) * 2 + 0) * 1024 + 16 * (lane ^ (4 * g))) = dsf[QB][0];
-        *reinterpret_cast<u32x4*>(block + ((wave * 2 + QB) * 2 + 1) * 1024 + 16 * (lane ^ (4 * g + 8))) = dsf[QB][1];
-    };
-    auto threshold_of = [&](int index) { return key_row - 4 * g - (first_tile + index) * QTILE; };
+                // S of both query halves: two independent accumulation chains
+                f32x16 s_acc[2];
+                static_for<0, QK_STEPS>([&](auto ks_tag) {
+                    constexpr int KS = decltype(ks_tag)::value;
+                    s_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::Q_ROW, 0, KS>(lds, q_at), kf[KS],
+                                                                       KS == 0 ? zero : s_acc[0], 0, 0, 0);
+                    s_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::Q_ROW, 32, KS>(lds, q_at), kf[KS],
+                                                                       KS == 0 ? zero : s_acc[1], 0, 0, 0);
+                });
 
-    // One half step.  Gradient products of half QB of the tile in stage
-    // `grad_stage` (operands set QB); with SCORES the score products of half QB of
-    // the tile in `score_stage` (into set QB); with PROBS the probabilities of half
-    // 1 - QB of the tile in `prob_stage` (scores set 1 - QB, into operand set
-    // 1 - QB).  With AHEAD the first RING fragments of the following half step
-    // (gradient fragments of half 1 - QB of the tile in next_stage) are read at
-    // the end.  Read addresses are formed where they are first needed.
-    auto half_step = [&](auto masked_tag, auto scores_tag, auto probs_tag, auto ahead_tag, auto qb_tag, auto phase_tag,
-                         int grad_stage, int score_stage, int prob_stage, int prob_threshold, int next_stage) {
-        constexpr int PHASE = decltype(phase_tag)::value;   // ring set of slot 0: slots consumed before, mod RING
-        constexpr bool SCORES = decltype(scores_tag)::value;
-        constexpr bool PROBS = decltype(probs_tag)::value;
-        constexpr bool AHEAD = decltype(ahead_tag)::value;
-        constexpr int QB = decltype(qb_tag)::value;
-        using Other = std::integral_constant<int, 1 - QB>;
-        constexpr int COUNT = GRAD_MFMAS + (SCORES ? SCORE_MFMAS : 0);
-        constexpr int SPAN = COUNT - PIECE_DELAY;   // slots that carry pieces
-        static_assert(4 * SPAN >= PIECES, "at most four pieces per slot");
-        GradientReads grad_at, next_at;
-        ScoreReads score_at;
-        gradient_reads(grad_at, grad_stage);
-        const unsigned prob_stats = stats_of(prob_stage);
-        if constexpr (PROBS) {
-            load_statistics(prob_stats, Other{}, std::integral_constant<int, 0>{});
-        }
-        static_for<0, COUNT>([&](auto slot) {
-            constexpr int I = decltype(slot)::value;
-            if constexpr (I < GRAD_MFMAS) {
-                gradient_mfma(qb_tag, slot, ring[(I + PHASE) % RING]);
-            } else {
-                score_mfma(qb_tag, std::integral_constant<int, I - GRAD_MFMAS>{}, ring[(I + PHASE) % RING]);
-            }
-            constexpr int A = I + RING;
-            if constexpr (SCORES && A == GRAD_MFMAS) {
-                score_reads(score_at, score_stage);
-            }
-            if constexpr (AHEAD && A == COUNT) {
-                gradient_reads(next_at, next_stage);
-            }
-            if constexpr (A < GRAD_MFMAS) {
-                ring[(I + PHASE) % RING] = gradient_fragment(grad_at, qb_tag, std::integral_constant<int, A>{});
-            } else if constexpr (A < COUNT) {
-                ring[(I + PHASE) % RING] = score_fragment(score_at, qb_tag, std::integral_constant<int, A - GRAD_MFMAS>{});
-            } else if constexpr (AHEAD) {
-                ring[(I + PHASE) % RING] = gradient_fragment(next_at, Other{}, std::integral_constant<int, A - COUNT>{});
-            }
-            if constexpr (PROBS && I >= PIECE_DELAY) {
-                // piece v goes to slot PIECE_DELAY + v * SPAN / PIECES: spread evenly
-                constexpr int J = I - PIECE_DELAY;
-                constexpr int FIRST = (J * PIECES + SPAN - 1) / SPAN;
-                constexpr int LAST = ((J + 1) * PIECES + SPAN - 1) / SPAN;
-                static_for<FIRST, LAST>([&](auto v_tag) {
-                    probability_piece(masked_tag, Other{}, v_tag, prob_stats, prob_threshold);
+                // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
+                // local index below `threshold` lies before this lane's key (only the
+                // first two tiles of a key block can meet the diagonal).
+                u32x4 pf[2][2];
+                const bool masked = index < 2;
+                const int threshold = key_row - 4 * g - (first_tile + index) * QTILE;
+                static_for<0, 2>([&](auto qb_tag) {
+                    constexpr int QB = decltype(qb_tag)::value;
+                    static_for<0, 4>([&](auto i4_tag) {
+                        constexpr int I4 = decltype(i4_tag)::value;
+                        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
+                        float p[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            p[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[QB][4 * I4 + e], c, -lse4[e]));
+                        }
+                        if (masked) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                if (32 * QB + 8 * I4 + e < threshold) p[e] = 0.f;
+                            }
+                        }
+                        pf[QB][I4 / 2][2 * (I4 % 2)] = pack_bf16(p[0], p[1]);
+                        pf[QB][I4 / 2][2 * (I4 % 2) + 1] = pack_bf16(p[2], p[3]);
+                    });
+                });
+                // hand P to the key wave
+                {
+                    unsigned char* buffer = lds + opaque(handover + (index % 2) * C::P_BYTES);
+                    static_for<0, 4>([&](auto piece_tag) {
+                        constexpr int PIECE = decltype(piece_tag)::value;
+                        *reinterpret_cast<u32x4*>(buffer + PIECE * 1024) = pf[PIECE / 2][PIECE % 2];
+                    });
+                }
+                // dV += P^T dO (contraction over the tile's 64 queries)
+                static_for<0, 4>([&](auto step_tag) {
+                    constexpr int STEP = decltype(step_tag)::value;   // 16-query step
+                    static_for<0, DV_BLOCKS>([&](auto d_tag) {
+                        constexpr int D = decltype(d_tag)::value;
+                        dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
+                            transposed_fragment<C::O_ROW, 16 * STEP, D>(lds, o_at), dv_acc[D], 0, 0, 0);
+                    });
                 });
             }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-    };
+        }
 
-    // ---- prologue: tiles 0 and 1 requested; S, dP of tile 0 and P, dS of its first
-    // half formed; the ring primed with the first gradient fragments of tile 0
-    wait_vector_memory<0>();   // the K / V row loads: no wait for them may remain inside the loop
-    request_tile(0, 0);
-    if (tiles > 1) {
-        request_tile(1, 1);
-    }
-    wait_vector_memory<0>();
-    workgroup_barrier();
-    {
-        ScoreReads at;
-        score_reads(at, 0);
-        static_for<0, 2>([&](auto qb_tag) {
-            static_for<0, SCORE_MFMAS>([&](auto k_tag) { score_mfma(qb_tag, k_tag, score_fragment(at, qb_tag, k_tag)); });
-        });
-        // the scores must have left the matrix pipeline before their elements are copied out
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
-        __builtin_amdgcn_sched_barrier(0);
-        const unsigned stats_at = stats_of(0);
-        load_statistics(stats_at, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-        static_for<0, PIECES>([&](auto v_tag) {
-            probability_piece(std::true_type{}, std::integral_constant<int, 0>{}, v_tag, stats_at, threshold_of(0));
-        });
-        GradientReads first;
-        gradient_reads(first, 0);
-        static_for<0, RING>([&](auto k_tag) {
-            ring[decltype(k_tag)::value] = gradient_fragment(first, std::integral_constant<int, 0>{}, k_tag);
-        });
-    }
+        // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
+        __syncthreads();
+        unsigned char* dv_lds = lds + group * 32 * (C::DK_PITCH + C::DV_PITCH) + 32 * C::DK_PITCH;
+#pragma unroll
+        for (int d = 0; d < DV_BLOCKS; ++d) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = 8 * (i / 4) + 4 * g + i % 4;
+                *reinterpret_cast<__bf16*>(dv_lds + row * C::DV_PITCH + 2 * (32 * d + lq)) = (__bf16)dv_acc[d][i];
+            }
+        }
+        __syncthreads();
+        bf16_t* dv_base = value_gradient + ((size_t)b * S * heads + h) * DV;
+        for (int position = lane; position < 32 * (DV / 8); position += 64) {
+            const int row = position / (DV / 8);
+            const int chunk = position % (DV / 8);
+            if (group_k0 + row < S) {
+                const u32x4 bits = *reinterpret_cast<const u32x4*>(dv_lds + row * C::DV_PITCH + 16 * chunk);
+                *reinterpret_cast<u32x4*>(dv_base + (size_t)(group_k0 + row) * v_stride + 8 * chunk) = bits;
+            }
+        }
+    } else {
+        // ================= key wave: dP, dS, dK =================
+        const bf16_t* v_base = value + ((size_t)b * S * heads + h) * DV;
+        bf16x8 vf[V_STEPS];   // B operand: column = key lq
+        load_row_fragments<DV>(vf, v_base, v_stride, key_row, key_row < S, g);
+        f32x16 dk_acc[DK_BLOCKS];
+#pragma unroll
+        for (int d = 0; d < DK_BLOCKS; ++d) clear(dk_acc[d]);
+        unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+        f32x16 dp_acc[2];
+        clear(dp_acc[0]);
+        clear(dp_acc[1]);
 
-    // Tile `index`: both halves are accumulated while the scores of tile index + 1
-    // and the probabilities of the halves in between are formed.  MASKED applies
-    // the causal mask to those probabilities, LAST leaves out everything that
-    // belongs to tile index + 1.
-    auto body = [&](auto masked_tag, auto last_tag, int index) {
-        constexpr bool LAST = decltype(last_tag)::value;
-        using NotLast = std::integral_constant<bool, !LAST>;
-        const int stage = index % 3;
-        const int next_stage = stage == 2 ? 0 : stage + 1;
-        wait_vector_memory<0>();   // this wave's share of tile index + 1 has landed
-        workgroup_barrier();       // ... and everybody's; every wave has left tile index - 1
-        if (index + 2 < tiles) {
-            request_tile(index + 2, (index + 2) % 3);
+        for (int index = 0; index <= tiles; ++index) {
+            wait_vector_memory<0>();
+            workgroup_barrier();
+            if (index + 1 < tiles) {
+                request_tile(index + 1);
+            }
+            if (index > 0) {
+                // tile index - 1: dS = P (dP - delta), dK += dS^T Q
+                const int previous = index - 1;
+                const unsigned stage = (previous % 3) * C::STAGE_BYTES;
+                unsigned q_at[2][TileReads<C::Q_ROW>::TR];
+                rebase(q_at, q_reads.transposed, stage);
+                const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g + 4 * QTILE);
+                const unsigned char* buffer = lds + opaque(handover + (previous % 2) * C::P_BYTES);
+                unsigned char* block =
+                    ds_head + (size_t)ds_block_index(kb, first_tile + previous, query_tiles) * DS_BLOCK_BYTES;
+                u32x4 dsf[2][2];
+                static_for<0, 4>([&](auto piece_tag) {
+                    constexpr int PIECE = decltype(piece_tag)::value;   // (query half, 16-query step)
+                    constexpr int QB = PIECE / 2;
+                    constexpr int N = PIECE % 2;
+                    const u32x4 packed = *reinterpret_cast<const u32x4*>(buffer + PIECE * 1024);
+                    static_for<0, 2>([&](auto half_tag) {
+                        constexpr int HALF = decltype(half_tag)::value;
+                        constexpr int I4 = 2 * N + HALF;
+                        const f32x4 delta4 = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
+                        float ds[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t pair = packed[2 * HALF + e / 2];
+                            const float p = (e % 2) ? __uint_as_float(pair & 0xffff0000u) : __uint_as_float(pair << 16);
+                            ds[e] = p * (dp_acc[QB][4 * I4 + e] - delta4[e]);
+                        }
+                        dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
+                        dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
+                    });
+                    // 16 bytes per lane, slot (lane ^ (4g + 8n)) of the 1 KB piece (group, qb, n)
+                    *reinterpret_cast<u32x4*>(block + ((group * 2 + QB) * 2 + N) * 1024 + 16 * (lane ^ (4 * g + 8 * N))) =
+                        dsf[QB][N];
+                });
+                static_for<0, 4>([&](auto step_tag) {
+                    constexpr int STEP = decltype(step_tag)::value;
+                    static_for<0, DK_BLOCKS>([&](auto d_tag) {
+                        constexpr int D = decltype(d_tag)::value;
+                        dk_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8, dsf[STEP / 2][STEP % 2]),
+                            transposed_fragment<C::Q_ROW, 16 * STEP, D>(lds, q_at), dk_acc[D], 0, 0, 0);
+                    });
+                });
+            }
+            if (index < tiles) {
+                // dP of tile `index`, consumed in the next iteration
+                const unsigned stage = (index % 3) * C::STAGE_BYTES;
+                unsigned o_at[TileReads<C::O_ROW>::NAT];
+                rebase(o_at, o_reads.natural, stage + C::Q_BYTES);
+                static_for<0, V_STEPS>([&](auto ks_tag) {
+                    constexpr int KS = decltype(ks_tag)::value;
+                    dp_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::O_ROW, 0, KS>(lds, o_at), vf[KS],
+                                                                        KS == 0 ? zero : dp_acc[0], 0, 0, 0);
+                    dp_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::O_ROW, 32, KS>(lds, o_at), vf[KS],
+                                                                        KS == 0 ? zero : dp_acc[1], 0, 0, 0);
+                });
+            }
         }
-        store_ds(index, std::integral_constant<int, 0>{});
-        if (index > 0) {
-            store_ds(index - 1, std::integral_constant<int, 1>{});
-        }
-        // a whole tile's slots are a multiple of RING; half a LAST tile's need not be
-        static_assert((GRAD_MFMAS + SCORE_MFMAS) % RING == 0, "the ring must close over a half step");
-        using SecondPhase = std::integral_constant<int, LAST ? GRAD_MFMAS % RING : 0>;
-        half_step(masked_tag, NotLast{}, std::true_type{}, std::true_type{}, std::integral_constant<int, 0>{},
-                  std::integral_constant<int, 0>{}, stage, next_stage, stage, threshold_of(index), stage);
-        half_step(masked_tag, NotLast{}, NotLast{}, NotLast{}, std::integral_constant<int, 1>{}, SecondPhase{}, stage,
-                  next_stage, next_stage, threshold_of(index + 1), next_stage);
-    };
 
-    // the causal mask can only bite in the first two tiles of a key block
-    {
-        int index = 0;
-        for (; index < 2 && index + 1 < tiles; ++index) {
-            body(std::true_type{}, std::false_type{}, index);
-        }
-        for (; index + 1 < tiles; ++index) {
-            body(std::false_type{}, std::false_type{}, index);
-        }
-        if (index < 2) {
-            body(std::true_type{}, std::true_type{}, index);
-        } else {
-            body(std::false_type{}, std::true_type{}, index);
-        }
-        store_ds(index, std::integral_constant<int, 1>{});
-    }
-
-    // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
-    __syncthreads();
-    unsigned char* dk_lds = lds + wave * 32 * (C::DK_PITCH + C::DV_PITCH);
-    unsigned char* dv_lds = dk_lds + 32 * C::DK_PITCH;
+        // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
+        __syncthreads();
+        unsigned char* dk_lds = lds + group * 32 * (C::DK_PITCH + C::DV_PITCH);
 #pragma unroll
-    for (int d = 0; d < DK_BLOCKS; ++d) {
+        for (int d = 0; d < DK_BLOCKS; ++d) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = 8 * (i / 4) + 4 * g + i % 4;
-            const __bf16 rounded = (__bf16)(dk_acc[d][i] * scale);
-            *reinterpret_cast<__bf16*>(dk_lds + row * C::DK_PITCH + 2 * (32 * d + lq)) = rounded;
+            for (int i = 0; i < 16; ++i) {
+                const int row = 8 * (i / 4) + 4 * g + i % 4;
+                *reinterpret_cast<__bf16*>(dk_lds + row * C::DK_PITCH + 2 * (32 * d + lq)) = (__bf16)(dk_acc[d][i] * scale);
+            }
         }
-    }
-#pragma unroll
-    for (int d = 0; d < DV_BLOCKS; ++d) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = 8 * (i / 4) + 4 * g + i % 4;
-            const __bf16 rounded = (__bf16)dv_acc[d][i];
-            *reinterpret_cast<__bf16*>(dv_lds + row * C::DV_PITCH + 2 * (32 * d + lq)) = rounded;
-        }
-    }
-    __syncthreads();
-    bf16_t* dk_base = key_gradient + ((size_t)b * S * heads + h) * DQK;
-    bf16_t* dv_base = value_gradient + ((size_t)b * S * heads + h) * DV;
-    for (int position = lane; position < 32 * (DQK / 8); position += 64) {
-        const int row = position / (DQK / 8);
-        const int chunk = position % (DQK / 8);
-        if (wave_k0 + row < S) {
-            const u32x4 bits = *reinterpret_cast<const u32x4*>(dk_lds + row * C::DK_PITCH + 16 * chunk);
-            *reinterpret_cast<u32x4*>(dk_base + (size_t)(wave_k0 + row) * qk_stride + 8 * chunk) = bits;
-        }
-    }
-    for (int position = lane; position < 32 * (DV / 8); position += 64) {
-        const int row = position / (DV / 8);
-        const int chunk = position % (DV / 8);
-        if (wave_k0 + row < S) {
-            const u32x4 bits = *reinterpret_cast<const u32x4*>(dv_lds + row * C::DV_PITCH + 16 * chunk);
-            *reinterpret_cast<u32x4*>(dv_base + (size_t)(wave_k0 + row) * v_stride + 8 * chunk) = bits;
+        __syncthreads();
+        bf16_t* dk_base = key_gradient + ((size_t)b * S * heads + h) * DQK;
+        for (int position = lane; position < 32 * (DQK / 8); position += 64) {
+            const int row = position / (DQK / 8);
+            const int chunk = position % (DQK / 8);
+            if (group_k0 + row < S) {
+                const u32x4 bits = *reinterpret_cast<const u32x4*>(dk_lds + row * C::DK_PITCH + 16 * chunk);
+                *reinterpret_cast<u32x4*>(dk_base + (size_t)(group_k0 + row) * qk_stride + 8 * chunk) = bits;
+            }
         }
     }
 }
@@ -766,8 +681,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
     tile_index[1] = min(2 * jb + 1, query_tiles - 1);
 
     const int steps = 2 * (jb + 1);   // 64-key steps up to the end of key block jb
-    TileRequests<C::K_ROW> k_requests;
-    k_requests.init(k_stride_bytes, lane);
+    TileRequests<C::K_ROW, BWD_THREADS / 64> k_requests;
+    k_requests.init(k_stride_bytes, wave, lane);
     auto request_step = [&](int step, int stage) {
         const int kb = step / 2;
         const int half = step % 2;
@@ -949,7 +864,7 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
                        shape.query_tiles);
     HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL((attention_key_value_gradient_kernel<DQK, DV>), dim3((unsigned)(groups * shape.key_blocks)),
-                       dim3(BWD_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
+                       dim3(KV_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
                        output_gradient, query, key, value, sequence_length, heads, shape.key_blocks,
                        shape.query_tiles, scale);
     HIP_CHECK(hipGetLastError());
