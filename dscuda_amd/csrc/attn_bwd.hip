@@ -363,6 +363,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     constexpr int DK_BLOCKS = DQK / 32;
     constexpr int DV_BLOCKS = DV / 32;
     constexpr int WAVES = KV_THREADS / 64;
+    constexpr int RING = 4;   // fragments read ahead of the MFMA that takes them
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -434,28 +435,48 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
 #pragma unroll
         for (int d = 0; d < DV_BLOCKS; ++d) clear(dv_acc[d]);
         const float c = scale * LOG2E;
+        constexpr int S_MFMAS = 2 * QK_STEPS;
+        constexpr int DV_MFMAS = 4 * DV_BLOCKS;
+        static_assert(RING <= DV_MFMAS && RING <= S_MFMAS, "a ring of fragments must fit each product");
+        bf16x8 ring[RING];
+        // S fragment K: k-step K/2 of query half K%2; dV fragment K: 16-query step K / DV_BLOCKS, column block K % DV_BLOCKS
+        auto s_fragment = [&](const unsigned (&q_at)[TileReads<C::Q_ROW>::NAT], auto k_tag) -> bf16x8 {
+            constexpr int K = decltype(k_tag)::value;
+            return natural_fragment<C::Q_ROW, 32 * (K % 2), K / 2>(lds, q_at);
+        };
+        auto dv_fragment = [&](const unsigned (&o_at)[2][TileReads<C::O_ROW>::TR], auto k_tag) -> bf16x8 {
+            constexpr int K = decltype(k_tag)::value;
+            return transposed_fragment<C::O_ROW, 16 * (K / DV_BLOCKS), K % DV_BLOCKS>(lds, o_at);
+        };
 
-        for (int index = 0; index <= tiles; ++index) {
+        for (int index = 0; index < tiles; ++index) {
             wait_vector_memory<0>();   // this wave's share of tile `index` has landed
             workgroup_barrier();       // ... and everybody's; every wave has left tile index - 2
             if (index + 1 < tiles) {
                 request_tile(index + 1);
             }
-            if (index < tiles) {
+            {
                 const unsigned stage = (index % 3) * C::STAGE_BYTES;
                 unsigned q_at[TileReads<C::Q_ROW>::NAT], o_at[2][TileReads<C::O_ROW>::TR];
                 rebase(q_at, q_reads.natural, stage);
                 rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
                 const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g);
 
-                // S of both query halves: two independent accumulation chains
+                // S of both query halves (two independent accumulation chains), fragments
+                // through the ring; its tail reads the first dV fragments ahead
                 f32x16 s_acc[2];
-                static_for<0, QK_STEPS>([&](auto ks_tag) {
-                    constexpr int KS = decltype(ks_tag)::value;
-                    s_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::Q_ROW, 0, KS>(lds, q_at), kf[KS],
-                                                                       KS == 0 ? zero : s_acc[0], 0, 0, 0);
-                    s_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::Q_ROW, 32, KS>(lds, q_at), kf[KS],
-                                                                       KS == 0 ? zero : s_acc[1], 0, 0, 0);
+                static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = s_fragment(q_at, k_tag); });
+                static_for<0, S_MFMAS>([&](auto k_tag) {
+                    constexpr int K = decltype(k_tag)::value;
+                    constexpr int KS = K / 2;
+                    s_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[K % RING], kf[KS],
+                                                                           KS == 0 ? zero : s_acc[K % 2], 0, 0, 0);
+                    if constexpr (K + RING < S_MFMAS) {
+                        ring[K % RING] = s_fragment(q_at, std::integral_constant<int, K + RING>{});
+                    } else {
+                        ring[K % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING - S_MFMAS>{});
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 });
 
                 // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
@@ -493,17 +514,20 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                     });
                 }
                 // dV += P^T dO (contraction over the tile's 64 queries)
-                static_for<0, 4>([&](auto step_tag) {
-                    constexpr int STEP = decltype(step_tag)::value;   // 16-query step
-                    static_for<0, DV_BLOCKS>([&](auto d_tag) {
-                        constexpr int D = decltype(d_tag)::value;
-                        dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
-                            transposed_fragment<C::O_ROW, 16 * STEP, D>(lds, o_at), dv_acc[D], 0, 0, 0);
-                    });
+                static_for<0, DV_MFMAS>([&](auto k_tag) {
+                    constexpr int K = decltype(k_tag)::value;
+                    constexpr int STEP = K / DV_BLOCKS;   // 16-query step
+                    constexpr int D = K % DV_BLOCKS;
+                    dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
+                                                                        ring[(K + S_MFMAS) % RING], dv_acc[D], 0, 0, 0);
+                    if constexpr (K + RING < DV_MFMAS) {
+                        ring[(K + S_MFMAS) % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING>{});
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 });
             }
         }
+        workgroup_barrier();   // the key waves' last iteration
 
         // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
         __syncthreads();
@@ -538,14 +562,65 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         f32x16 dp_acc[2];
         clear(dp_acc[0]);
         clear(dp_acc[1]);
+        constexpr int DK_MFMAS = 4 * DK_BLOCKS;
+        constexpr int DP_MFMAS = 2 * V_STEPS;
+        static_assert(RING <= DK_MFMAS && RING <= DP_MFMAS, "a ring of fragments must fit each product");
+        static_assert((DK_MFMAS + DP_MFMAS) % RING == 0, "the ring must close over an iteration");
+        bf16x8 ring[RING];
+        // dK fragment K: 16-query step K / DK_BLOCKS, column block K % DK_BLOCKS; dP fragment K: k-step K/2 of query half K%2
+        auto dk_fragment = [&](const unsigned (&q_at)[2][TileReads<C::Q_ROW>::TR], auto k_tag) -> bf16x8 {
+            constexpr int K = decltype(k_tag)::value;
+            return transposed_fragment<C::Q_ROW, 16 * (K / DK_BLOCKS), K % DK_BLOCKS>(lds, q_at);
+        };
+        auto dp_fragment = [&](const unsigned (&o_at)[TileReads<C::O_ROW>::NAT], auto k_tag) -> bf16x8 {
+            constexpr int K = decltype(k_tag)::value;
+            return natural_fragment<C::O_ROW, 32 * (K % 2), K / 2>(lds, o_at);
+        };
 
-        for (int index = 0; index <= tiles; ++index) {
+        // dP of tile `index` (consumed in the next iteration; at index == tiles a harmless
+        // repeat over stale data, so that every iteration has one shape); the tail reads
+        // the first dK fragments of the same tile ahead
+        auto dp_stream = [&](int index) {
+            const unsigned stage = (index % 3) * C::STAGE_BYTES;
+            unsigned o_at[TileReads<C::O_ROW>::NAT], q_next[2][TileReads<C::Q_ROW>::TR];
+            rebase(o_at, o_reads.natural, stage + C::Q_BYTES);
+            rebase(q_next, q_reads.transposed, stage);
+            static_for<0, DP_MFMAS>([&](auto k_tag) {
+                constexpr int K = decltype(k_tag)::value;
+                constexpr int KS = K / 2;
+                dp_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[(K + DK_MFMAS) % RING], vf[KS],
+                                                                        KS == 0 ? zero : dp_acc[K % 2], 0, 0, 0);
+                if constexpr (K + RING < DP_MFMAS) {
+                    ring[(K + DK_MFMAS) % RING] = dp_fragment(o_at, std::integral_constant<int, K + RING>{});
+                } else {
+                    ring[(K + DK_MFMAS) % RING] = dk_fragment(q_next, std::integral_constant<int, K + RING - DP_MFMAS>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+
+        // first iteration: only dP of tile 0
+        wait_vector_memory<0>();
+        workgroup_barrier();
+        if (1 < tiles) {
+            request_tile(1);
+        }
+        {
+            unsigned o_at[TileReads<C::O_ROW>::NAT];
+            rebase(o_at, o_reads.natural, C::Q_BYTES);
+            static_for<0, RING>([&](auto k_tag) {
+                ring[(decltype(k_tag)::value + DK_MFMAS) % RING] = dp_fragment(o_at, k_tag);
+            });
+        }
+        dp_stream(0);
+
+        for (int index = 1; index <= tiles; ++index) {
             wait_vector_memory<0>();
             workgroup_barrier();
             if (index + 1 < tiles) {
                 request_tile(index + 1);
             }
-            if (index > 0) {
+            {
                 // tile index - 1: dS = P (dP - delta), dK += dS^T Q
                 const int previous = index - 1;
                 const unsigned stage = (previous % 3) * C::STAGE_BYTES;
@@ -579,29 +654,24 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                     *reinterpret_cast<u32x4*>(block + ((group * 2 + QB) * 2 + N) * 1024 + 16 * (lane ^ (4 * g + 8 * N))) =
                         dsf[QB][N];
                 });
-                static_for<0, 4>([&](auto step_tag) {
-                    constexpr int STEP = decltype(step_tag)::value;
-                    static_for<0, DK_BLOCKS>([&](auto d_tag) {
-                        constexpr int D = decltype(d_tag)::value;
-                        dk_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, dsf[STEP / 2][STEP % 2]),
-                            transposed_fragment<C::Q_ROW, 16 * STEP, D>(lds, q_at), dk_acc[D], 0, 0, 0);
-                    });
-                });
-            }
-            if (index < tiles) {
-                // dP of tile `index`, consumed in the next iteration
-                const unsigned stage = (index % 3) * C::STAGE_BYTES;
+                // dK += dS^T Q; the tail reads the first dP fragments of tile `index` ahead
                 unsigned o_at[TileReads<C::O_ROW>::NAT];
-                rebase(o_at, o_reads.natural, stage + C::Q_BYTES);
-                static_for<0, V_STEPS>([&](auto ks_tag) {
-                    constexpr int KS = decltype(ks_tag)::value;
-                    dp_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::O_ROW, 0, KS>(lds, o_at), vf[KS],
-                                                                        KS == 0 ? zero : dp_acc[0], 0, 0, 0);
-                    dp_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<C::O_ROW, 32, KS>(lds, o_at), vf[KS],
-                                                                        KS == 0 ? zero : dp_acc[1], 0, 0, 0);
+                rebase(o_at, o_reads.natural, (index % 3) * C::STAGE_BYTES + C::Q_BYTES);
+                static_for<0, DK_MFMAS>([&](auto k_tag) {
+                    constexpr int K = decltype(k_tag)::value;
+                    constexpr int STEP = K / DK_BLOCKS;
+                    constexpr int D = K % DK_BLOCKS;
+                    dk_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, dsf[STEP / 2][STEP % 2]),
+                                                                        ring[K % RING], dk_acc[D], 0, 0, 0);
+                    if constexpr (K + RING < DK_MFMAS) {
+                        ring[K % RING] = dk_fragment(q_at, std::integral_constant<int, K + RING>{});
+                    } else {
+                        ring[K % RING] = dp_fragment(o_at, std::integral_constant<int, K + RING - DK_MFMAS>{});
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 });
             }
+            dp_stream(index);
         }
 
         // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
