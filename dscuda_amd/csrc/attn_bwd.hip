@@ -319,17 +319,14 @@ __global__ __launch_bounds__(256) void attention_backward_statistics_kernel(
 //   key wave (g + 4)    dP = dO V^T (V rows in registers)  ->  dS = P (dP - delta)
 //                       ->  dK += dS^T Q;  dS goes to the workspace
 //
-// A wave cannot overlap its own MFMAs with its own vector arithmetic, but the two
-// waves of a SIMD can: the key wave runs one tile behind and in the opposite order
-// (arithmetic first), so while one wave forms probabilities the other feeds the
-// matrix pipeline.  One workgroup barrier per tile keeps the pair, the tile stages
-// and the P hand-over in step:
+// The two waves of a SIMD run different instruction streams, so while one wave
+// forms probabilities the other feeds the matrix pipeline.  Two workgroup barriers
+// per tile keep the pair, the tile stages and the P hand-over in step:
 //
-//   iteration i    value wave: S(i) | P(i) -> LDS | dV(i)
-//                  key wave:   dS(i-1) from P(i-1), dP(i-1) | dK(i-1) | dP(i)
+//   barrier A (tile landed)   value wave: S | P -> LDS        key wave: dP
+//   barrier B (P visible)     value wave: dV                  key wave: dS, dK
 //
-// Tile i lives in stage i % 3 and is requested one iteration ahead; P(i) lives in
-// hand-over buffer i % 2 of its key group.
+// Tile i lives in stage i % 3 and is requested two tiles ahead.
 
 constexpr int KV_THREADS = 512;
 
@@ -344,7 +341,7 @@ struct KeyValueGradConfig {
     static constexpr int STAGES = 3;
     static constexpr int P_BYTES = QTILE * 32 * 2;                  // P of one tile and key group, bf16
     static constexpr int HANDOVER_AT = STAGES * STAGE_BYTES;
-    static constexpr int LDS_BYTES = HANDOVER_AT + 4 * 2 * P_BYTES;  // 4 key groups x 2 buffers
+    static constexpr int LDS_BYTES = HANDOVER_AT + 4 * P_BYTES;   // one buffer per key group
     static constexpr int DK_PITCH = 2 * DQK;   // epilogue staging
     static constexpr int DV_PITCH = 2 * DV;
     static_assert(4 * 32 * (DK_PITCH + DV_PITCH) <= HANDOVER_AT, "epilogue staging must fit");
@@ -376,8 +373,25 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     const int g = lane / 32;
     const int S = sequence_length;
 
-    int bh, kb;  // key block 0 sees every query: heaviest first in natural order
-    xcd_order(blockIdx.x, gridDim.x / key_blocks, key_blocks, bh, kb);
+    // Work order.  The key blocks of a (batch, head) pair all stream the same query
+    // tiles, so they are kept together: pairs are dealt to the XCDs (private L2s), one
+    // pair at a time per XCD, key block 0 (which sees every query: the heaviest) first.
+    // Every key block walks the tiles from the last one down to its diagonal: blocks
+    // started together then read the same tile at the same time, and one fetch from
+    // memory serves them all.
+    int bh, kb;
+    {
+        constexpr int XCDS = 8;
+        const int pairs = gridDim.x / key_blocks;
+        if (pairs % XCDS == 0) {
+            const int slot = blockIdx.x / XCDS;
+            bh = blockIdx.x % XCDS + XCDS * (slot / key_blocks);
+            kb = slot % key_blocks;
+        } else {
+            bh = blockIdx.x / key_blocks;
+            kb = blockIdx.x % key_blocks;
+        }
+    }
     const int b = bh / heads;
     const int h = bh % heads;
     const int k0 = kb * KBLOCK;
@@ -394,24 +408,28 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     const float* stat_base = statistics + (size_t)bh * query_tiles * STAT_FLOATS;
     const unsigned lds_base = lds_offset_of(lds);
 
-    const int first_tile = 2 * kb;
-    const int tiles = query_tiles - first_tile;   // >= 1
+    const int tiles = query_tiles - 2 * kb;   // >= 1; step `index` works on tile query_tiles - 1 - index
 
-    TileRequests<C::Q_ROW, WAVES> q_requests;
-    TileRequests<C::O_ROW, WAVES> o_requests;
-    q_requests.init(q_stride_bytes, wave, lane);
-    o_requests.init(o_stride_bytes, wave, lane);
+    // Tiles are requested by the four value waves, each the same number of loads per
+    // tile: a value wave then knows that all but its last REQUEST_LOADS loads have
+    // landed, and the key waves' vector-memory counter only ever holds their dS
+    // stores, which nothing has to wait for.
+    TileRequests<C::Q_ROW, 4> q_requests;
+    TileRequests<C::O_ROW, 4> o_requests;
+    q_requests.init(q_stride_bytes, wave % 4, lane);
+    o_requests.init(o_stride_bytes, wave % 4, lane);
+    constexpr int REQUEST_LOADS = TileRequests<C::Q_ROW, 4>::LOADS + TileRequests<C::O_ROW, 4>::LOADS + 1;
     auto request_tile = [&](int index) {
-        const int tile = first_tile + index;
+        const int tile = query_tiles - 1 - index;
         const int row0 = tile * QTILE;
         const int row_limit = S - 1 - row0;
         const unsigned target = lds_base + (index % 3) * C::STAGE_BYTES;
         q_requests.request(q_base + (size_t)row0 * q_stride_bytes, q_stride_bytes, row_limit, target, wave);
         o_requests.request(do_base + (size_t)row0 * o_stride_bytes, o_stride_bytes, row_limit, target + C::Q_BYTES, wave);
-        if (wave < 2) {
-            direct_load_4_offset(stat_base + (size_t)tile * STAT_FLOATS + 64 * wave, 4u * lane,
-                                 target + C::Q_BYTES + C::O_BYTES + 256 * wave);
-        }
+        // statistics: 128 floats = two loads; waves 2 and 3 repeat those of waves 0 and 1
+        // (same bytes to the same place) so that every value wave issues the same count
+        direct_load_4_offset(stat_base + (size_t)tile * STAT_FLOATS + 64 * (wave % 2), 4u * lane,
+                             target + C::Q_BYTES + C::O_BYTES + 256 * (wave % 2));
     };
 
     // per-lane read offsets inside a stage
@@ -420,14 +438,16 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     q_reads.init(lane);
     o_reads.init(lane);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    // hand-over buffers of this key group: P as the value wave's registers hold it,
+    // hand-over buffer of this key group: P as the value wave's registers hold it,
     // piece (query half, 16-query step) of 1 KB, 16 bytes per lane
-    const unsigned handover = C::HANDOVER_AT + group * 2 * C::P_BYTES + 16 * lane;
-
-    request_tile(0);
+    const unsigned handover = C::HANDOVER_AT + group * C::P_BYTES + 16 * lane;
 
     if (!key_wave) {
         // ================= value wave: S, P, dV =================
+        request_tile(0);
+        if (tiles > 1) {
+            request_tile(1);
+        }
         const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
         bf16x8 kf[QK_STEPS];   // B operand: column = key lq
         load_row_fragments<DQK>(kf, k_base, qk_stride, key_row, key_row < S, g);
@@ -448,86 +468,107 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             constexpr int K = decltype(k_tag)::value;
             return transposed_fragment<C::O_ROW, 16 * (K / DV_BLOCKS), K % DV_BLOCKS>(lds, o_at);
         };
+        // the K row loads are waited for here: the counted waits below assume that only
+        // tile requests are in flight (the two requests above are older and land first)
+        wait_vector_memory<0>();
 
-        for (int index = 0; index < tiles; ++index) {
-            wait_vector_memory<0>();   // this wave's share of tile `index` has landed
-            workgroup_barrier();       // ... and everybody's; every wave has left tile index - 2
+        // One tile.  MASKED applies the causal mask: it can only bite in the two tiles at
+        // the diagonal, the last ones of the walk (and all the tiles a ragged last block has).
+        auto value_tile = [&](auto masked_tag, int index) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            // this wave's share of tile `index` has landed; the request of tile index + 1
+            // (if there is one) may stay in flight
             if (index + 1 < tiles) {
-                request_tile(index + 1);
+                wait_vector_memory<REQUEST_LOADS>();
+            } else {
+                wait_vector_memory<0>();
             }
-            {
-                const unsigned stage = (index % 3) * C::STAGE_BYTES;
-                unsigned q_at[TileReads<C::Q_ROW>::NAT], o_at[2][TileReads<C::O_ROW>::TR];
-                rebase(q_at, q_reads.natural, stage);
-                rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
-                const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g);
+            workgroup_barrier();       // ... and everybody's; every wave has left tile index - 1
+            const unsigned stage = (index % 3) * C::STAGE_BYTES;
+            unsigned q_at[TileReads<C::Q_ROW>::NAT], o_at[2][TileReads<C::O_ROW>::TR];
+            rebase(q_at, q_reads.natural, stage);
+            const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g);
 
-                // S of both query halves (two independent accumulation chains), fragments
-                // through the ring; its tail reads the first dV fragments ahead
-                f32x16 s_acc[2];
-                static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = s_fragment(q_at, k_tag); });
-                static_for<0, S_MFMAS>([&](auto k_tag) {
-                    constexpr int K = decltype(k_tag)::value;
-                    constexpr int KS = K / 2;
-                    s_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[K % RING], kf[KS],
-                                                                           KS == 0 ? zero : s_acc[K % 2], 0, 0, 0);
-                    if constexpr (K + RING < S_MFMAS) {
-                        ring[K % RING] = s_fragment(q_at, std::integral_constant<int, K + RING>{});
-                    } else {
-                        ring[K % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING - S_MFMAS>{});
+            // S of both query halves (two independent accumulation chains), fragments
+            // through the ring; its tail reads the first dV fragments and the statistics
+            // of the tile's queries ahead.  The tile after the next is requested while the
+            // first fragments are on their way.
+            f32x16 s_acc[2];
+            f32x4 lse4[2][4];   // queries 32*qb + 8*i4 + 4*g + (0..3)
+            static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = s_fragment(q_at, k_tag); });
+            if (index + 2 < tiles) {
+                request_tile(index + 2);
+            }
+            rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
+            static_for<0, S_MFMAS>([&](auto k_tag) {
+                constexpr int K = decltype(k_tag)::value;
+                constexpr int KS = K / 2;
+                s_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[K % RING], kf[KS],
+                                                                       KS == 0 ? zero : s_acc[K % 2], 0, 0, 0);
+                if constexpr (K + RING < S_MFMAS) {
+                    ring[K % RING] = s_fragment(q_at, std::integral_constant<int, K + RING>{});
+                } else {
+                    ring[K % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING - S_MFMAS>{});
+                }
+                if constexpr (K >= S_MFMAS - 8) {
+                    constexpr int J = K - (S_MFMAS - 8);
+                    lse4[J / 4][J % 4] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * (J / 4) + 8 * (J % 4)));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+
+            // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
+            // local index below `threshold` lies before this lane's key.
+            u32x4 pf[2][2];
+            const int threshold = key_row - 4 * g - (query_tiles - 1 - index) * QTILE;
+            static_for<0, 2>([&](auto qb_tag) {
+                constexpr int QB = decltype(qb_tag)::value;
+                static_for<0, 4>([&](auto i4_tag) {
+                    constexpr int I4 = decltype(i4_tag)::value;
+                    float p[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        p[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[QB][4 * I4 + e], c, -lse4[QB][I4][e]));
                     }
-                    __builtin_amdgcn_sched_barrier(0);
-                });
-
-                // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
-                // local index below `threshold` lies before this lane's key (only the
-                // first two tiles of a key block can meet the diagonal).
-                u32x4 pf[2][2];
-                const bool masked = index < 2;
-                const int threshold = key_row - 4 * g - (first_tile + index) * QTILE;
-                static_for<0, 2>([&](auto qb_tag) {
-                    constexpr int QB = decltype(qb_tag)::value;
-                    static_for<0, 4>([&](auto i4_tag) {
-                        constexpr int I4 = decltype(i4_tag)::value;
-                        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
-                        float p[4];
+                    if constexpr (MASKED) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            p[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[QB][4 * I4 + e], c, -lse4[e]));
+                            if (32 * QB + 8 * I4 + e < threshold) p[e] = 0.f;
                         }
-                        if (masked) {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                if (32 * QB + 8 * I4 + e < threshold) p[e] = 0.f;
-                            }
-                        }
-                        pf[QB][I4 / 2][2 * (I4 % 2)] = pack_bf16(p[0], p[1]);
-                        pf[QB][I4 / 2][2 * (I4 % 2) + 1] = pack_bf16(p[2], p[3]);
-                    });
-                });
-                // hand P to the key wave
-                {
-                    unsigned char* buffer = lds + opaque(handover + (index % 2) * C::P_BYTES);
-                    static_for<0, 4>([&](auto piece_tag) {
-                        constexpr int PIECE = decltype(piece_tag)::value;
-                        *reinterpret_cast<u32x4*>(buffer + PIECE * 1024) = pf[PIECE / 2][PIECE % 2];
-                    });
-                }
-                // dV += P^T dO (contraction over the tile's 64 queries)
-                static_for<0, DV_MFMAS>([&](auto k_tag) {
-                    constexpr int K = decltype(k_tag)::value;
-                    constexpr int STEP = K / DV_BLOCKS;   // 16-query step
-                    constexpr int D = K % DV_BLOCKS;
-                    dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
-                                                                        ring[(K + S_MFMAS) % RING], dv_acc[D], 0, 0, 0);
-                    if constexpr (K + RING < DV_MFMAS) {
-                        ring[(K + S_MFMAS) % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING>{});
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+                    pf[QB][I4 / 2][2 * (I4 % 2)] = pack_bf16(p[0], p[1]);
+                    pf[QB][I4 / 2][2 * (I4 % 2) + 1] = pack_bf16(p[2], p[3]);
                 });
+            });
+            // hand P to the key wave
+            static_for<0, 4>([&](auto piece_tag) {
+                constexpr int PIECE = decltype(piece_tag)::value;
+                *reinterpret_cast<u32x4*>(lds + handover + PIECE * 1024) = pf[PIECE / 2][PIECE % 2];
+            });
+            workgroup_barrier();   // P is visible; the key waves have their dP
+
+            // dV += P^T dO (contraction over the tile's 64 queries)
+            static_for<0, DV_MFMAS>([&](auto k_tag) {
+                constexpr int K = decltype(k_tag)::value;
+                constexpr int STEP = K / DV_BLOCKS;   // 16-query step
+                constexpr int D = K % DV_BLOCKS;
+                dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
+                                                                    ring[(K + S_MFMAS) % RING], dv_acc[D], 0, 0, 0);
+                if constexpr (K + RING < DV_MFMAS) {
+                    ring[(K + S_MFMAS) % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        {
+            int index = 0;
+            for (; index < tiles - 2; ++index) {
+                value_tile(std::false_type{}, index);
+            }
+            for (; index < tiles; ++index) {
+                value_tile(std::true_type{}, index);
             }
         }
-        workgroup_barrier();   // the key waves' last iteration
 
         // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
         __syncthreads();
@@ -559,13 +600,9 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
 #pragma unroll
         for (int d = 0; d < DK_BLOCKS; ++d) clear(dk_acc[d]);
         unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
-        f32x16 dp_acc[2];
-        clear(dp_acc[0]);
-        clear(dp_acc[1]);
         constexpr int DK_MFMAS = 4 * DK_BLOCKS;
         constexpr int DP_MFMAS = 2 * V_STEPS;
         static_assert(RING <= DK_MFMAS && RING <= DP_MFMAS, "a ring of fragments must fit each product");
-        static_assert((DK_MFMAS + DP_MFMAS) % RING == 0, "the ring must close over an iteration");
         bf16x8 ring[RING];
         // dK fragment K: 16-query step K / DK_BLOCKS, column block K % DK_BLOCKS; dP fragment K: k-step K/2 of query half K%2
         auto dk_fragment = [&](const unsigned (&q_at)[2][TileReads<C::Q_ROW>::TR], auto k_tag) -> bf16x8 {
@@ -576,102 +613,84 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             constexpr int K = decltype(k_tag)::value;
             return natural_fragment<C::O_ROW, 32 * (K % 2), K / 2>(lds, o_at);
         };
+        // per-lane part of the dS store addresses: slot (lane ^ (4g + 8n)) of the 1 KB
+        // piece (group, qb, n) of the tile's block
+        unsigned ds_slot[2];
+        ds_slot[0] = group * 4096 + 16 * (lane ^ (4 * g));
+        ds_slot[1] = group * 4096 + 1024 + 16 * (lane ^ (4 * g + 8));
+        wait_vector_memory<0>();   // the V rows
 
-        // dP of tile `index` (consumed in the next iteration; at index == tiles a harmless
-        // repeat over stale data, so that every iteration has one shape); the tail reads
-        // the first dK fragments of the same tile ahead
-        auto dp_stream = [&](int index) {
+        for (int index = 0; index < tiles; ++index) {
+            workgroup_barrier();   // tile `index` has landed
             const unsigned stage = (index % 3) * C::STAGE_BYTES;
-            unsigned o_at[TileReads<C::O_ROW>::NAT], q_next[2][TileReads<C::Q_ROW>::TR];
+            unsigned o_at[TileReads<C::O_ROW>::NAT], q_at[2][TileReads<C::Q_ROW>::TR];
             rebase(o_at, o_reads.natural, stage + C::Q_BYTES);
-            rebase(q_next, q_reads.transposed, stage);
+            const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g + 4 * QTILE);
+
+            // dP of both query halves; the tail reads the first dK fragments and the
+            // tile's delta values ahead
+            f32x16 dp_acc[2];
+            f32x4 delta4[2][4];   // queries 32*qb + 8*i4 + 4*g + (0..3)
+            static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = dp_fragment(o_at, k_tag); });
+            rebase(q_at, q_reads.transposed, stage);
             static_for<0, DP_MFMAS>([&](auto k_tag) {
                 constexpr int K = decltype(k_tag)::value;
                 constexpr int KS = K / 2;
-                dp_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[(K + DK_MFMAS) % RING], vf[KS],
+                dp_acc[K % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[K % RING], vf[KS],
                                                                         KS == 0 ? zero : dp_acc[K % 2], 0, 0, 0);
                 if constexpr (K + RING < DP_MFMAS) {
-                    ring[(K + DK_MFMAS) % RING] = dp_fragment(o_at, std::integral_constant<int, K + RING>{});
+                    ring[K % RING] = dp_fragment(o_at, std::integral_constant<int, K + RING>{});
                 } else {
-                    ring[(K + DK_MFMAS) % RING] = dk_fragment(q_next, std::integral_constant<int, K + RING - DP_MFMAS>{});
+                    ring[K % RING] = dk_fragment(q_at, std::integral_constant<int, K + RING - DP_MFMAS>{});
+                }
+                if constexpr (K >= DP_MFMAS - 8) {
+                    constexpr int J = K - (DP_MFMAS - 8);
+                    delta4[J / 4][J % 4] = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * (J / 4) + 8 * (J % 4)));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
-        };
+            workgroup_barrier();   // P of this tile is in the hand-over buffer
 
-        // first iteration: only dP of tile 0
-        wait_vector_memory<0>();
-        workgroup_barrier();
-        if (1 < tiles) {
-            request_tile(1);
-        }
-        {
-            unsigned o_at[TileReads<C::O_ROW>::NAT];
-            rebase(o_at, o_reads.natural, C::Q_BYTES);
-            static_for<0, RING>([&](auto k_tag) {
-                ring[(decltype(k_tag)::value + DK_MFMAS) % RING] = dp_fragment(o_at, k_tag);
+            // dS = P (dP - delta): lane holds key lq and queries 32*qb + 8*i4 + 4*g + e
+            u32x4 packed[4];      // pieces (query half, 16-query step)
+            static_for<0, 4>([&](auto piece_tag) {
+                constexpr int PIECE = decltype(piece_tag)::value;
+                packed[PIECE] = *reinterpret_cast<const u32x4*>(lds + handover + PIECE * 1024);
             });
-        }
-        dp_stream(0);
-
-        for (int index = 1; index <= tiles; ++index) {
-            wait_vector_memory<0>();
-            workgroup_barrier();
-            if (index + 1 < tiles) {
-                request_tile(index + 1);
-            }
-            {
-                // tile index - 1: dS = P (dP - delta), dK += dS^T Q
-                const int previous = index - 1;
-                const unsigned stage = (previous % 3) * C::STAGE_BYTES;
-                unsigned q_at[2][TileReads<C::Q_ROW>::TR];
-                rebase(q_at, q_reads.transposed, stage);
-                const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g + 4 * QTILE);
-                const unsigned char* buffer = lds + opaque(handover + (previous % 2) * C::P_BYTES);
-                unsigned char* block =
-                    ds_head + (size_t)ds_block_index(kb, first_tile + previous, query_tiles) * DS_BLOCK_BYTES;
-                u32x4 dsf[2][2];
-                static_for<0, 4>([&](auto piece_tag) {
-                    constexpr int PIECE = decltype(piece_tag)::value;   // (query half, 16-query step)
-                    constexpr int QB = PIECE / 2;
-                    constexpr int N = PIECE % 2;
-                    const u32x4 packed = *reinterpret_cast<const u32x4*>(buffer + PIECE * 1024);
-                    static_for<0, 2>([&](auto half_tag) {
-                        constexpr int HALF = decltype(half_tag)::value;
-                        constexpr int I4 = 2 * N + HALF;
-                        const f32x4 delta4 = *reinterpret_cast<const f32x4*>(lds + stats_at + 4 * (32 * QB + 8 * I4));
-                        float ds[4];
+            unsigned char* block =
+                ds_head + (size_t)ds_block_index(kb, query_tiles - 1 - index, query_tiles) * DS_BLOCK_BYTES;
+            u32x4 dsf[2][2];
+            static_for<0, 4>([&](auto piece_tag) {
+                constexpr int PIECE = decltype(piece_tag)::value;
+                constexpr int QB = PIECE / 2;
+                constexpr int N = PIECE % 2;
+                static_for<0, 2>([&](auto half_tag) {
+                    constexpr int HALF = decltype(half_tag)::value;
+                    constexpr int I4 = 2 * N + HALF;
+                    float ds[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t pair = packed[2 * HALF + e / 2];
-                            const float p = (e % 2) ? __uint_as_float(pair & 0xffff0000u) : __uint_as_float(pair << 16);
-                            ds[e] = p * (dp_acc[QB][4 * I4 + e] - delta4[e]);
-                        }
-                        dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
-                        dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
-                    });
-                    // 16 bytes per lane, slot (lane ^ (4g + 8n)) of the 1 KB piece (group, qb, n)
-                    *reinterpret_cast<u32x4*>(block + ((group * 2 + QB) * 2 + N) * 1024 + 16 * (lane ^ (4 * g + 8 * N))) =
-                        dsf[QB][N];
-                });
-                // dK += dS^T Q; the tail reads the first dP fragments of tile `index` ahead
-                unsigned o_at[TileReads<C::O_ROW>::NAT];
-                rebase(o_at, o_reads.natural, (index % 3) * C::STAGE_BYTES + C::Q_BYTES);
-                static_for<0, DK_MFMAS>([&](auto k_tag) {
-                    constexpr int K = decltype(k_tag)::value;
-                    constexpr int STEP = K / DK_BLOCKS;
-                    constexpr int D = K % DK_BLOCKS;
-                    dk_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, dsf[STEP / 2][STEP % 2]),
-                                                                        ring[K % RING], dk_acc[D], 0, 0, 0);
-                    if constexpr (K + RING < DK_MFMAS) {
-                        ring[K % RING] = dk_fragment(q_at, std::integral_constant<int, K + RING>{});
-                    } else {
-                        ring[K % RING] = dp_fragment(o_at, std::integral_constant<int, K + RING - DK_MFMAS>{});
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t pair = packed[PIECE][2 * HALF + e / 2];
+                        const float p = (e % 2) ? __uint_as_float(pair & 0xffff0000u) : __uint_as_float(pair << 16);
+                        ds[e] = p * (dp_acc[QB][4 * I4 + e] - delta4[QB][I4][e]);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+                    dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
+                    dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
                 });
-            }
-            dp_stream(index);
+                *reinterpret_cast<u32x4*>(block + (ds_slot[N] + QB * 2048)) = dsf[QB][N];
+            });
+            // dK += dS^T Q
+            static_for<0, DK_MFMAS>([&](auto k_tag) {
+                constexpr int K = decltype(k_tag)::value;
+                constexpr int STEP = K / DK_BLOCKS;
+                constexpr int D = K % DK_BLOCKS;
+                dk_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, dsf[STEP / 2][STEP % 2]),
+                                                                    ring[(K + DP_MFMAS) % RING], dk_acc[D], 0, 0, 0);
+                if constexpr (K + RING < DK_MFMAS) {
+                    ring[(K + DP_MFMAS) % RING] = dk_fragment(q_at, std::integral_constant<int, K + RING>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
         }
 
         // ---- epilogue: lane holds column 32*d + lq and keys 8*(i/4) + 4*g + i%4
