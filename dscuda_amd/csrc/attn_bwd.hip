@@ -731,15 +731,23 @@ struct QueryGradConfig {
     static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     static constexpr int D_BLOCKS = DQK / 64;            // 32-column blocks per wave
     static_assert(LDS_BYTES <= 160 * 1024, "stages must fit the LDS");
+    static_assert(4 * D_BLOCKS * 2 * 16 * 64 * 4 <= LDS_BYTES, "the final sums must fit the LDS");
 };
 
 // dQ^T (d x queries) = sum over keys of K^T (d x keys) dS^T (keys x queries).
-// Wave w owns query tile w%2 of the workgroup's two and the 32-column blocks 2*d + w/2.
+// Eight waves, two per SIMD: wave w owns query tile w%2 of the workgroup's two, the
+// 32-column blocks 2*d + (w/2)%2, and the 16-key steps 2*(w/4), 2*(w/4)+1 of every
+// 64-key step; the two key halves are added through LDS at the end.  The pass is
+// bound by the dS stream from memory: steps are requested two ahead and a wave only
+// waits for the older of its two requests in flight.
+constexpr int DQ_THREADS = 512;
+
 template <int DQK>
-__global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
+__global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
     bf16_t* __restrict__ query_gradient, const unsigned char* __restrict__ ds_blocks, const bf16_t* __restrict__ key,
     int sequence_length, int heads, int query_blocks, int key_blocks, int query_tiles, float scale) {
     using C = QueryGradConfig<DQK>;
+    constexpr int WAVES = DQ_THREADS / 64;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -756,7 +764,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
     const int b = bh / heads;
     const int h = bh % heads;
     const int tile_of_wave = wave % 2;
-    const int column_half = wave / 2;
+    const int column_half = (wave / 2) % 2;
+    const int key_half = wave / 4;
 
     const unsigned k_stride_bytes = (unsigned)heads * DQK * 2;
     const unsigned char* k_base = reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * heads + h) * DQK);
@@ -770,8 +779,10 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
     tile_index[1] = min(2 * jb + 1, query_tiles - 1);
 
     const int steps = 2 * (jb + 1);   // 64-key steps up to the end of key block jb
-    TileRequests<C::K_ROW, BWD_THREADS / 64> k_requests;
+    TileRequests<C::K_ROW, WAVES> k_requests;
     k_requests.init(k_stride_bytes, wave, lane);
+    constexpr int DS_LOADS = 2 * C::DS_HALF / 1024 / WAVES;   // 1 KB pieces of the two query tiles' halves per wave
+    constexpr int STEP_LOADS = TileRequests<C::K_ROW, WAVES>::LOADS + DS_LOADS;
     auto request_step = [&](int step, int stage) {
         const int kb = step / 2;
         const int half = step % 2;
@@ -781,8 +792,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
         k_requests.request(k_base + (size_t)min(row0, S - 1) * k_stride_bytes, k_stride_bytes, max(S - 1 - row0, 0),
                            target, wave);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int load = 4 * wave + i;   // 16 pieces of 1 KB: two query tiles x 8
+        for (int i = 0; i < DS_LOADS; ++i) {
+            const int load = DS_LOADS * wave + i;   // 16 pieces of 1 KB: two query tiles x 8
             const int t = load / 8;
             const int part = load % 8;
             const unsigned char* block =
@@ -801,7 +812,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
 
     // K^T operand (ds_read_b64_tr_b16 on the row-major K rows).  A wave's column
     // blocks are 2*d + column_half, so the swizzle-dependent part of the address
-    // (block % TR) is fixed per wave up to d, and the rest is an immediate.
+    // (block % TR) is fixed per wave up to d, and the rest is an immediate.  The
+    // wave's key half (32 rows down) is folded into the per-lane part as well.
     constexpr int TR = TileReads<C::K_ROW>::TR;
     constexpr int SEL = TR / 2;
     unsigned k_reads[2][SEL];
@@ -812,7 +824,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
         for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
             for (int j = 0; j < SEL; ++j) {
-                k_reads[h2][j] = column_half ? reads.transposed[h2][2 * j + 1] : reads.transposed[h2][2 * j];
+                k_reads[h2][j] = (column_half ? reads.transposed[h2][2 * j + 1] : reads.transposed[h2][2 * j]) +
+                                 key_half * 32 * C::K_ROW;
             }
         }
     }
@@ -821,6 +834,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
     // of a 16-lane group fetches the 8 bytes that hold queries 4*(s%4).. of key s/4
     // (+8 for the second read): slot ((key%32 + 32*g') ^ (4*g' + 8*n)) of the 1 KB piece
     // (key/32, qb, n), n = (lane/16)%2, g' = s%2, second half of the slot if (s%4)/2.
+    // The wave's key half selects key/32.
     unsigned ds_reads[2];
     {
         const int s = lane % 16;
@@ -829,14 +843,20 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
             const int slot = s / 4 + 4 * (g ^ gp) + 8 * (h2 ^ n) + 32 * gp;
-            ds_reads[h2] = C::K_BYTES + tile_of_wave * C::DS_HALF + n * 1024 + 16 * slot + 8 * ((s % 4) / 2);
+            ds_reads[h2] = C::K_BYTES + tile_of_wave * C::DS_HALF + key_half * 4096 + n * 1024 + 16 * slot +
+                           8 * ((s % 4) / 2);
         }
     }
 
     request_step(0, 0);
     request_step(1, 1);   // steps >= 2 always
     for (int step = 0; step < steps; ++step) {
-        wait_vector_memory<0>();
+        // this wave's share of step `step` has landed; the request of step + 1 may stay in flight
+        if (step + 1 < steps) {
+            wait_vector_memory<STEP_LOADS>();
+        } else {
+            wait_vector_memory<0>();
+        }
         workgroup_barrier();
         if (step + 2 < steps) {
             request_step(step + 2, (step + 2) % 3);
@@ -846,11 +866,11 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
         rebase(k_at, k_reads, stage_offset);
         rebase(ds_at, ds_reads, stage_offset);
 #pragma unroll
-        for (int kk = 0; kk < C::STEP_KEYS / 16; ++kk) {
+        for (int kk = 0; kk < 2; ++kk) {   // the wave's two 16-key steps
             bf16x8 ds[2];
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-                const int constant = (kk / 2) * 4096 + qb * 2048 + (kk % 2) * 256;
+                const int constant = qb * 2048 + kk * 256;
                 const s16x4 low =
                     __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(lds + ds_at[0] + constant));
                 const s16x4 high =
@@ -868,6 +888,35 @@ __global__ __launch_bounds__(BWD_THREADS) void attention_query_gradient_kernel(
                     __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
                 dq_acc[d][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, ds[0], dq_acc[d][0], 0, 0, 0);
                 dq_acc[d][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, ds[1], dq_acc[d][1], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- the upper key half hands its sums to the lower one: register r of lane l at
+    // float (r * 64 + l) of the wave pair's area
+    __syncthreads();
+    {
+        float* area = reinterpret_cast<float*>(lds) + (wave % 4) * (C::D_BLOCKS * 2 * 16 * 64) + lane;
+        if (key_half == 1) {
+#pragma unroll
+            for (int d = 0; d < C::D_BLOCKS; ++d) {
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) area[((d * 2 + qb) * 16 + i) * 64] = dq_acc[d][qb][i];
+                }
+            }
+        }
+        __syncthreads();
+        if (key_half == 1) {
+            return;
+        }
+#pragma unroll
+        for (int d = 0; d < C::D_BLOCKS; ++d) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) dq_acc[d][qb][i] += area[((d * 2 + qb) * 16 + i) * 64];
             }
         }
     }
@@ -958,7 +1007,7 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
                        shape.query_tiles, scale);
     HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>), dim3((unsigned)(groups * shape.query_blocks)),
-                       dim3(BWD_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
+                       dim3(DQ_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
                        heads, shape.query_blocks, shape.key_blocks, shape.query_tiles, scale);
     HIP_CHECK(hipGetLastError());
 }
