@@ -26,6 +26,14 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch of the forward kernel at the headline workload, from the two
+# rocprofv3 --pmc runs whose summaries are profiles/pmc_fwd_fetch.txt (FETCH_SIZE 675103.5 KiB)
+# and profiles/pmc_fwd_write.txt (WRITE_SIZE 214073.0 KiB), each scaled by what the same counter
+# reads for a 1 GiB device copy (profiles/pmc_copy_*.txt: FETCH_SIZE reports half the bytes
+# read -> factor 2.0, WRITE_SIZE reports them all -> factor 1.0).  A recorded measurement, not
+# something this script can observe itself.
+FORWARD_TRAFFIC_BYTES = (675103.5 * 2.0 + 214073.0 * 1.0) * 1024
+
 
 def event_time_ms(function, steps, warmup):
     """Average duration of `function` over `steps` launches, from events on torch's
@@ -126,7 +134,7 @@ def main():
         "config": {"workload": "MLA prefill forward, B=1 S=4096 H=128, d_qk=128+64, d_v=128, causal, "
                                "0.5*N(0,1) seed 1, RoPE theta=10000, scale 1/sqrt(192)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": FORWARD_TRAFFIC_BYTES,
                      "kernel": "attention_forward_pingpong_kernel<192,128>", "kernel_ms": kernel_ms,
                      "flops_per_launch": flops},
         "cpu_baseline": baseline,
