@@ -75,6 +75,18 @@ def mla_prefill_dout(batch=1, seq=4096, heads=128, dv=128, seed=2, factor=1.0):
     return _randn(g, (batch, seq, heads, dv), factor).bfloat16()
 
 
+def mla_long_context_inputs(batch=1, seq=16384, heads=128, nope=128, rope=64, dv=128, seed=4):
+    """Workload 5: Q, K [B,S,H,192], V [B,S,H,128] ~ 0.5*N(0,1) and dO [B,S,H,128] ~ N(0,1), all from
+    one generator seeded with 4, no rotation; scale 1/sqrt(192)."""
+    g = torch.Generator().manual_seed(seed)
+    dqk = nope + rope
+    q = _randn(g, (batch, seq, heads, dqk), 0.5).bfloat16()
+    k = _randn(g, (batch, seq, heads, dqk), 0.5).bfloat16()
+    v = _randn(g, (batch, seq, heads, dv), 0.5).bfloat16()
+    dout = _randn(g, (batch, seq, heads, dv), 1.0).bfloat16()
+    return q, k, v, dout, c_float(dqk ** -0.5)
+
+
 def decode_lengths(batch=64, low=1024, high=8192, seed=3):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(low, high + 1, (batch,), generator=g, dtype=torch.int64).to(torch.int32), g

@@ -52,6 +52,30 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3)
         "kernels": "mla_decode_split + mla_decode_combine"}
     del paged, workspace
 
+    # long context: MLA prefill forward + backward, B=1 S=16384 H=128.  Timing does not depend on the
+    # values, so the inputs are drawn on the GPU (the seeded CPU inputs are what the parity test uses).
+    generator = torch.Generator(device=device).manual_seed(4)
+    long_seq = 16384
+    draw = lambda shape, factor: (torch.randn(shape, device=device, generator=generator) * factor).bfloat16()
+    lq, lk = draw((1, long_seq, heads, dqk), 0.5), draw((1, long_seq, heads, dqk), 0.5)
+    lv, ldo = draw((1, long_seq, heads, dv), 0.5), draw((1, long_seq, heads, dv), 1.0)
+    lout = torch.empty(1, long_seq, heads, dv, device=device, dtype=torch.bfloat16)
+    llse = torch.empty(1, heads, long_seq, device=device, dtype=torch.float32)
+    ms, _ = event_time_ms(lambda: ops.mla_prefill_forward(lq, lk, lv, scale, lout, llse), 3, 1)
+    flops = configs.forward_flops(1, heads, long_seq, dqk, dv)
+    results["mla_forward_S16384_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
+                                          "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,
+                                          "data": "synthetic, GPU generator"}
+    grads = (torch.empty_like(lq), torch.empty_like(lk), torch.empty_like(lv))
+    workspace = ops.mla_prefill_backward_workspace(1, long_seq, heads, dqk, dv, device)
+    ms, _ = event_time_ms(lambda: ops.mla_prefill_backward(ldo, lout, llse, lq, lk, lv, scale, workspace, grads), 3, 1)
+    flops = configs.backward_flops(1, heads, long_seq, dqk, dv)
+    results["mla_backward_S16384_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
+                                           "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,
+                                           "workspace_gib": workspace.numel() * 4 / 2 ** 30,
+                                           "data": "synthetic, GPU generator"}
+    del lq, lk, lv, ldo, lout, llse, grads, workspace
+
     # flash attention forward, B=1 H=8 S=512 D=64 (latency bound: report time)
     fq, fk, fv, fscale = configs.flash_forward_inputs()
     fq, fk, fv = fq.to(device), fk.to(device), fv.to(device)
