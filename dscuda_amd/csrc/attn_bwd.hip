@@ -323,10 +323,12 @@ __global__ __launch_bounds__(256) void attention_backward_statistics_kernel(
 // forms probabilities the other feeds the matrix pipeline.  Two workgroup barriers
 // per tile keep the pair, the tile stages and the P hand-over in step:
 //
-//   barrier A (tile landed)   value wave: S | P -> LDS        key wave: dP
-//   barrier B (P visible)     value wave: dV                  key wave: dS, dK
+//   barrier A   value wave: P(i) -> LDS               key wave: dP(i)
+//   barrier B   value wave: dV(i), S(i+1)            key wave: dS(i), dK(i)
 //
-// Tile i lives in stage i % 3 and is requested two tiles ahead.
+// so that in either phase one wave of a SIMD has vector work while the other has
+// matrix work.  Tile i lives in stage i % 3 and is requested two tiles ahead; it is
+// complete one phase before its first use.
 
 constexpr int KV_THREADS = 512;
 
@@ -468,38 +470,16 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             constexpr int K = decltype(k_tag)::value;
             return transposed_fragment<C::O_ROW, 16 * (K / DV_BLOCKS), K % DV_BLOCKS>(lds, o_at);
         };
-        // the K row loads are waited for here: the counted waits below assume that only
-        // tile requests are in flight (the two requests above are older and land first)
-        wait_vector_memory<0>();
-
-        // One tile.  MASKED applies the causal mask: it can only bite in the two tiles at
-        // the diagonal, the last ones of the walk (and all the tiles a ragged last block has).
-        auto value_tile = [&](auto masked_tag, int index) {
-            constexpr bool MASKED = decltype(masked_tag)::value;
-            // this wave's share of tile `index` has landed; the request of tile index + 1
-            // (if there is one) may stay in flight
-            if (index + 1 < tiles) {
-                wait_vector_memory<REQUEST_LOADS>();
-            } else {
-                wait_vector_memory<0>();
-            }
-            workgroup_barrier();       // ... and everybody's; every wave has left tile index - 1
+        // S of tile `index` (both query halves: two independent accumulation chains),
+        // fragments through the ring; the tail reads the statistics of the tile's queries.
+        f32x16 s_acc[2];
+        f32x4 lse4[2][4];   // queries 32*qb + 8*i4 + 4*g + (0..3)
+        auto score_stream = [&](int index) {
             const unsigned stage = (index % 3) * C::STAGE_BYTES;
-            unsigned q_at[TileReads<C::Q_ROW>::NAT], o_at[2][TileReads<C::O_ROW>::TR];
+            unsigned q_at[TileReads<C::Q_ROW>::NAT];
             rebase(q_at, q_reads.natural, stage);
             const unsigned stats_at = opaque(stage + C::Q_BYTES + C::O_BYTES + 16 * g);
-
-            // S of both query halves (two independent accumulation chains), fragments
-            // through the ring; its tail reads the first dV fragments and the statistics
-            // of the tile's queries ahead.  The tile after the next is requested while the
-            // first fragments are on their way.
-            f32x16 s_acc[2];
-            f32x4 lse4[2][4];   // queries 32*qb + 8*i4 + 4*g + (0..3)
             static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = s_fragment(q_at, k_tag); });
-            if (index + 2 < tiles) {
-                request_tile(index + 2);
-            }
-            rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
             static_for<0, S_MFMAS>([&](auto k_tag) {
                 constexpr int K = decltype(k_tag)::value;
                 constexpr int KS = K / 2;
@@ -507,8 +487,6 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                                                                        KS == 0 ? zero : s_acc[K % 2], 0, 0, 0);
                 if constexpr (K + RING < S_MFMAS) {
                     ring[K % RING] = s_fragment(q_at, std::integral_constant<int, K + RING>{});
-                } else {
-                    ring[K % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING - S_MFMAS>{});
                 }
                 if constexpr (K >= S_MFMAS - 8) {
                     constexpr int J = K - (S_MFMAS - 8);
@@ -516,7 +494,21 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
+        };
 
+        // One tile, in two phases separated by barriers:
+        //   after barrier A   P of the tile from its scores (formed one phase earlier) -> hand-over
+        //   after barrier B   dV of the tile, then the scores of the next tile
+        // so that in either phase one wave of the SIMD has vector work and the other
+        // matrix work.  MASKED applies the causal mask: it can only bite in the two
+        // tiles at the diagonal, the last ones of the walk (and all the tiles a ragged
+        // last block has).
+        auto value_tile = [&](auto masked_tag, int index) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            workgroup_barrier();   // A: every wave has left tile index - 1
+            if (index + 2 < tiles) {
+                request_tile(index + 2);
+            }
             // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
             // local index below `threshold` lies before this lane's key.
             u32x4 pf[2][2];
@@ -545,21 +537,39 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 constexpr int PIECE = decltype(piece_tag)::value;
                 *reinterpret_cast<u32x4*>(lds + handover + PIECE * 1024) = pf[PIECE / 2][PIECE % 2];
             });
-            workgroup_barrier();   // P is visible; the key waves have their dP
+            // this wave's share of tile index + 1 has landed (the request of tile index + 2,
+            // if there is one, may stay in flight)
+            if (index + 2 < tiles) {
+                wait_vector_memory<REQUEST_LOADS>();
+            } else {
+                wait_vector_memory<0>();
+            }
+            workgroup_barrier();   // B: P is visible, and so is all of tile index + 1
 
             // dV += P^T dO (contraction over the tile's 64 queries)
+            const unsigned stage = (index % 3) * C::STAGE_BYTES;
+            unsigned o_at[2][TileReads<C::O_ROW>::TR];
+            rebase(o_at, o_reads.transposed, stage + C::Q_BYTES);
+            static_for<0, RING>([&](auto k_tag) { ring[decltype(k_tag)::value] = dv_fragment(o_at, k_tag); });
             static_for<0, DV_MFMAS>([&](auto k_tag) {
                 constexpr int K = decltype(k_tag)::value;
                 constexpr int STEP = K / DV_BLOCKS;   // 16-query step
                 constexpr int D = K % DV_BLOCKS;
                 dv_acc[D] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pf[STEP / 2][STEP % 2]),
-                                                                    ring[(K + S_MFMAS) % RING], dv_acc[D], 0, 0, 0);
+                                                                    ring[K % RING], dv_acc[D], 0, 0, 0);
                 if constexpr (K + RING < DV_MFMAS) {
-                    ring[(K + S_MFMAS) % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING>{});
+                    ring[K % RING] = dv_fragment(o_at, std::integral_constant<int, K + RING>{});
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
+            if (index + 1 < tiles) {
+                score_stream(index + 1);
+            }
         };
+        // tile 0 has landed for everybody; its scores
+        wait_vector_memory<0>();
+        workgroup_barrier();
+        score_stream(0);
         {
             int index = 0;
             for (; index < tiles - 2; ++index) {
@@ -619,9 +629,10 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         ds_slot[0] = group * 4096 + 16 * (lane ^ (4 * g));
         ds_slot[1] = group * 4096 + 1024 + 16 * (lane ^ (4 * g + 8));
         wait_vector_memory<0>();   // the V rows
+        workgroup_barrier();       // tile 0 has landed
 
         for (int index = 0; index < tiles; ++index) {
-            workgroup_barrier();   // tile `index` has landed
+            workgroup_barrier();   // A: every wave has left tile index - 1 (tile `index` landed a phase ago)
             const unsigned stage = (index % 3) * C::STAGE_BYTES;
             unsigned o_at[TileReads<C::O_ROW>::NAT], q_at[2][TileReads<C::Q_ROW>::TR];
             rebase(o_at, o_reads.natural, stage + C::Q_BYTES);
@@ -649,7 +660,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
-            workgroup_barrier();   // P of this tile is in the hand-over buffer
+            workgroup_barrier();   // B: P of this tile is in the hand-over buffer
 
             // dS = P (dP - delta): lane holds key lq and queries 32*qb + 8*i4 + 4*g + e
             u32x4 packed[4];      // pieces (query half, 16-query step)
