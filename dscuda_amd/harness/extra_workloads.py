@@ -8,7 +8,7 @@ PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 
-def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3):
+def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15):
     """q, k, v: the S=4096 H=128 prefill inputs already on `device`; out / lse: the
     forward's results for them (the backward's saved tensors)."""
     import torch
@@ -44,7 +44,7 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3)
     dout_o = torch.empty(b, 1, h, 512, device=device, dtype=torch.bfloat16)
     dlse = torch.empty(b, h, 1, device=device, dtype=torch.float32)
     ms, _ = event_time_ms(lambda: ops.mla_decode(dq, paged, table, dl, data["scale"], splits=8, workspace=workspace,
-                                                 out=dout_o, lse=dlse), 3 * steps, warmup)
+                                                 out=dout_o, lse=dlse), 5 * steps, 3 * warmup)
     nbytes = configs.decode_bytes(total, b, h)
     results["mla_decode_B64_H128"] = {
         "us": ms * 1000.0, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
@@ -80,7 +80,7 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=10, warmup=3)
     fq, fk, fv, fscale = configs.flash_forward_inputs()
     fq, fk, fv = fq.to(device), fk.to(device), fv.to(device)
     fo, fl = torch.empty_like(fq), torch.empty(1, 8, 512, device=device)
-    ms, _ = event_time_ms(lambda: ops.flash_forward(fq, fk, fv, fscale, fo, fl), 50, 10)
+    ms, _ = event_time_ms(lambda: ops.flash_forward(fq, fk, fv, fscale, fo, fl), 200, 50)
     results["flash_forward_B1_H8_S512_D64"] = {"us": ms * 1000.0,
                                                "tflops": configs.forward_flops(1, 8, 512, 64, 64) / ms / 1e9}
     return results
