@@ -212,10 +212,6 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-// Order of the score MFMAs of one half: S and dP steps alternate while dP lasts.
-__host__ __device__ constexpr bool score_slot_is_s(int k, int v_steps) { return k >= 2 * v_steps || k % 2 == 0; }
-__host__ __device__ constexpr int score_slot_step(int k, int v_steps) { return k >= 2 * v_steps ? k - v_steps : k / 2; }
-
 // at = reads + offset, as values the optimiser cannot take apart again: the
 // fragment reads then keep the form (per-lane register) + (immediate) instead of
 // one address computation per read.
@@ -250,16 +246,6 @@ __device__ __forceinline__ void load_row_fragments(bf16x8 (&fragments)[D / 16], 
         }
         fragments[ks] = __builtin_bit_cast(bf16x8, bits);
     }
-}
-
-// Element of an MFMA result that lives in the accumulation registers, copied where
-// it is needed (the compiler would otherwise copy all sixteen at the first use and
-// hold them).  Two further MFMAs must have been issued since the one that produced it.
-template <int I>
-__device__ __forceinline__ float accumulator_element(const f32x16& accumulator) {
-    float value;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(value) : "a"(accumulator[I]));
-    return value;
 }
 
 __device__ __forceinline__ void clear(f32x16& value) {
