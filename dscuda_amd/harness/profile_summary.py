@@ -38,18 +38,45 @@ def kernel_stats(path: Path, patterns: list[str]) -> list[str]:
     return lines
 
 
-def counter_averages(path: Path, patterns: list[str]) -> list[str]:
+def mean(values) -> float:
+    values = list(values)
+    return sum(values) / len(values)
+
+
+def counter_averages(path: Path, patterns: list[str], xcds: int = 8) -> list[str]:
+    """Counter means per kernel.  Where the file carries dispatch timestamps, also
+    the dispatch duration of the first launches and of the second half of them
+    (the chip's clock takes some tens of launches to settle), and, if
+    GRBM_GUI_ACTIVE was collected (it is summed over the `xcds` dies), the clock
+    those cycles imply."""
     table = collections.defaultdict(lambda: collections.defaultdict(list))
+    spans = collections.defaultdict(lambda: collections.defaultdict(list))
     with open(path, newline="") as handle:
         for row in csv.DictReader(handle):
             if not wanted(row["Kernel_Name"], patterns):
                 continue
-            table[short_name(row["Kernel_Name"])][row["Counter_Name"]].append(float(row["Counter_Value"]))
+            kernel = short_name(row["Kernel_Name"])
+            table[kernel][row["Counter_Name"]].append(float(row["Counter_Value"]))
+            if row.get("Start_Timestamp") and row.get("End_Timestamp"):
+                spans[kernel][row["Counter_Name"]].append(int(row["End_Timestamp"]) - int(row["Start_Timestamp"]))
     lines = []
     for kernel, counters in table.items():
         lines.append(kernel[:100])
         for counter, values in counters.items():
-            lines.append(f"    {counter:32s} {sum(values) / len(values):18.1f}   (mean of {len(values)} dispatches)")
+            lines.append(f"    {counter:32s} {mean(values):18.1f}   (mean of {len(values)} dispatches)")
+        durations = next(iter(spans[kernel].values()), [])
+        if len(durations) >= 8:
+            head, tail = durations[:5], durations[len(durations) // 2:]
+            lines.append(f"    dispatch duration: first {len(head)} launches {mean(head) / 1e3:.1f} us, "
+                         f"second half ({len(tail)} launches) {mean(tail) / 1e3:.1f} us")
+            cycles = counters.get("GRBM_GUI_ACTIVE")
+            if cycles and len(cycles) == len(durations):
+                half = len(cycles) // 2
+                lines.append(f"    clock from GRBM_GUI_ACTIVE / {xcds} dies: first launches "
+                             f"{mean(cycles[:5]) / xcds / mean(head):.2f} GHz, second half "
+                             f"{mean(cycles[half:]) / xcds / mean(tail):.2f} GHz")
+        elif durations:
+            lines.append(f"    dispatch duration: {mean(durations) / 1e3:.1f} us (mean of {len(durations)})")
     return lines
 
 
