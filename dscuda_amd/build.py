@@ -4,7 +4,10 @@ Outputs ``build/libdscuda_mla_bench.so`` and
 ``build/libdscuda_flash_attention_bench.so`` under the repository root: the
 file names the reference's harness loads (``benchmarks/common.py:19-20``,
 ``CMakeLists.txt:56-61``).  Objects are compiled in parallel, one hipcc
-process per translation unit.
+process per translation unit.  The standalone profiler programs
+(``dscuda_amd/profiler/*.cpp``, the counterparts of the reference's
+``benchmarks/attention/benchmark_*.cu`` launchers, ``CMakeLists.txt:43-50``) are
+linked against them into ``build/`` as well.
 
 Run ``python -m dscuda_amd.build`` (add ``--resource-usage`` to print the
 compiler's per-kernel register / LDS / spill report).
@@ -36,6 +39,16 @@ LIBRARIES = {
     "libdscuda_mla_bench.so": ["api_mla", "attn_fwd", "attn_bwd", "mla_absorbed", "mla_decode"],
     "libdscuda_flash_attention_bench.so": ["api_flash", "attn_fwd"],
 }
+
+
+# executable -> (source under dscuda_amd/profiler, library it links)
+PROGRAMS = {
+    "benchmark_mla": ("benchmark_mla.cpp", "libdscuda_mla_bench.so"),
+    "benchmark_mla_decode": ("benchmark_mla_decode.cpp", "libdscuda_mla_bench.so"),
+    "benchmark_mla_prefill": ("benchmark_mla_prefill.cpp", "libdscuda_mla_bench.so"),
+    "benchmark_flash_attention": ("benchmark_flash_attention.cpp", "libdscuda_flash_attention_bench.so"),
+}
+PROFILER = ROOT / "dscuda_amd" / "profiler"
 
 
 def _hipcc() -> str:
@@ -78,6 +91,16 @@ def build_all(resource_usage: bool = False, jobs: int | None = None) -> dict[str
         _run([_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(target),
               *[str(objects[p]) for p in parts]])
         outputs[library] = target
+
+    def link_program(item):
+        program, (source, library) = item
+        target = BUILD / program
+        _run([_hipcc(), *COMMON_FLAGS, f"-I{PROFILER}", str(PROFILER / source), "-o", str(target),
+              f"-L{BUILD}", f"-l:{library}", "-Wl,-rpath,$ORIGIN"])
+        return program, target
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        outputs.update(dict(pool.map(link_program, PROGRAMS.items())))
     return outputs
 
 

@@ -122,8 +122,11 @@ void mla_prefill_forward_cuda(
     float scale,
     hipStream_t stream = nullptr);
 
-// FP32 elements of workspace the prefill backward needs (row-wise
-// delta = sum(dO * O), [B,H,S]).
+// FP32 elements of workspace the prefill backward needs: per-row statistics
+// (logsumexp in log2 units and delta = sum(dO * O), 128 floats per 64-query
+// tile) followed by the BF16 dS blocks the key/value-gradient pass hands to the
+// query-gradient pass, 16 KB per causal (128-key block, 64-query tile) pair --
+// about S*S bytes per (batch, head).  0 for non-positive sizes.
 std::size_t mla_prefill_backward_workspace_elements(
     int batch_size,
     int sequence_length,
