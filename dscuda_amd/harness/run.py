@@ -4,7 +4,7 @@ expression of the same mathematics on the same GPU, then both are timed by HIP
 graph replay and reported in the six-column table (``report.py``).
 
     python -m dscuda_amd.harness.run mla --suite quick
-    python -m dscuda_amd.harness.run all --suite full --output gpurun_out/runtime
+    python -m dscuda_amd.harness.run all --suite full --output /tmp/runtime
     python -m dscuda_amd.harness.run mla_prefill --suite metric --operation forward --no-reference
 
 Families: ``flash_attention`` and ``mla`` (the reference's shapes,
@@ -274,7 +274,7 @@ def main(argv=None):
     parser.add_argument("--warmup-ms", type=int, default=1000)
     parser.add_argument("--sample-ms", type=int, default=20)
     parser.add_argument("--trials", type=int, default=9)
-    parser.add_argument("--output", default=str(ROOT / "gpurun_out" / "runtime"), help="directory of the report files")
+    parser.add_argument("--output", default=str(ROOT / "build" / "runtime"), help="directory of the report files")
     args = parser.parse_args(argv)
 
     import torch
