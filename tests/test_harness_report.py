@@ -94,3 +94,49 @@ def test_entry_point_needs_a_gpu():
         pytest.skip("a GPU is present")
     result = harness("mla")
     assert result.returncode != 0 and "needs a GPU" in result.stderr
+
+
+# ---- the PyTorch expressions run.py times and checks against, pinned on the CPU against the oracle ----------
+
+def test_harness_reference_matches_the_oracle_for_causal_attention():
+    import torch
+    from dscuda_amd.harness import configs, run
+    from oracle import attention_oracle as oracle
+    q, k, v, scale = configs.mla_prefill_inputs(batch=2, seq=96, heads=3, seed=5)
+    out, lse = run._sdpa(q, k, v, scale, causal=True)
+    expected, expected_lse = oracle.causal_attention_forward(q, k, v, scale)
+    assert out.shape == expected.shape and lse.shape == expected_lse.shape == (2, 3, 96)
+    torch.testing.assert_close(out, expected.float(), atol=2e-5, rtol=1e-4)
+    torch.testing.assert_close(lse, expected_lse, atol=2e-5, rtol=1e-5)
+
+
+def test_harness_reference_broadcasts_shared_keys_and_masks_lengths():
+    import torch
+    from dscuda_amd.harness import configs, run
+    from oracle import attention_oracle as oracle
+    # grouped-query heads: 4 query heads on 2 key/value heads
+    q, k, v, scale = configs.flash_forward_inputs(1, 64, 4, 2, 64, seed=3, factor=0.5)
+    out, lse = run._sdpa(q, k, v, scale, causal=True)
+    expected, expected_lse = oracle.causal_attention_forward(q, k.repeat_interleave(2, dim=2), v.repeat_interleave(2, dim=2), scale)
+    torch.testing.assert_close(out, expected.float(), atol=2e-5, rtol=1e-4)
+    torch.testing.assert_close(lse, expected_lse, atol=2e-5, rtol=1e-5)
+    # decode: one query token per sequence against a shared 576-wide cache cut to per-sequence lengths
+    q_lat, q_rope, latent, k_rope, scale = configs.mla_absorbed_inputs(3, 70, 5, query_tokens=1)
+    lengths = torch.tensor([1, 37, 70], dtype=torch.int32)
+    packed, cache = torch.cat((q_lat, q_rope), -1), torch.cat((latent, k_rope), -1)
+    mask = (torch.arange(70)[None] < lengths[:, None])[:, None, None]
+    out, lse = run._sdpa(packed, cache[:, :, None], cache[:, :, None, :512], scale, mask=mask)
+    expected, expected_lse = oracle.mla_decode_unrounded(packed, cache, lengths, scale)
+    torch.testing.assert_close(out, expected.float().reshape(out.shape), atol=2e-5, rtol=1e-4)
+    torch.testing.assert_close(lse.reshape(-1), expected_lse.float().reshape(-1), atol=2e-5, rtol=1e-5)
+
+
+def test_harness_check_uses_per_output_tolerances():
+    import torch
+    from dscuda_amd.harness import run
+    expected = (torch.zeros(4), torch.zeros(4))
+    run._close((torch.full((4,), 5e-3), torch.full((4,), 5e-5)), expected, (8e-3, 1e-4), (8e-3, 1e-4))
+    with pytest.raises(AssertionError):
+        run._close((torch.full((4,), 5e-3), torch.full((4,), 5e-3)), expected, (8e-3, 1e-4), (8e-3, 1e-4))
+    with pytest.raises(AssertionError):
+        run._close(torch.zeros(4), expected, 1e-2, 1e-2)      # one output where two are expected
