@@ -35,10 +35,20 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 FORWARD_TRAFFIC_BYTES = (675103.5 * 2.0 + 214073.0 * 1.0) * 1024
 
 
-def event_time_ms(function, steps, warmup):
+SETTLE_MS = 40.0   # back-to-back launches before any timing: the chip's clock needs ~25 ms of load to settle
+
+
+def event_time_ms(function, steps, warmup, settle_ms=SETTLE_MS):
     """Average duration of `function` over `steps` launches, from events on torch's
-    current stream (the stream the kernels are enqueued on)."""
+    current stream (the stream the kernels are enqueued on).  Before the `warmup`
+    untimed launches the function is run back to back for `settle_ms` of wall time,
+    so that a small `warmup` still times the kernel at the clock a loaded chip runs at."""
     import torch
+    deadline = time.perf_counter() + settle_ms / 1000.0
+    while time.perf_counter() < deadline:
+        for _ in range(8):
+            function()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         function()
     torch.cuda.synchronize()
@@ -81,8 +91,6 @@ def cpu_baseline_forward(q, k, v, scale, gpu_out, gpu_lse, sample_heads):
 def main():
     parser = argparse.ArgumentParser(description=__doc__)
     parser.add_argument("--gpus", type=int, default=1)
-    # the chip's clock needs some 30 back-to-back launches (~25 ms) to settle: fewer warm-up steps
-    # time the ramp, not the kernel
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--cpu-heads", type=int, default=128, help="heads in the CPU baseline sample")
@@ -127,6 +135,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": SETTLE_MS,
         "ms_per_step": wall_ms,
         "higher_is_better": True,
         "scaling": "weak",
