@@ -33,6 +33,7 @@
 // pass reads them back transposed without bank conflicts).
 #include "attn_kernels.h"
 #include "hip_common.h"
+#include "index_math.h"
 
 #include <stdexcept>
 #include <string>
@@ -52,27 +53,9 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4* transposing_read_pointer;
 
-// Position of dS block (key block kb, query tile qt), qt >= 2*kb, key block major.
-__host__ __device__ inline long long ds_block_index(int kb, int qt, int query_tiles) {
-    return (long long)kb * query_tiles - (long long)kb * (kb - 1) + (qt - 2 * kb);
-}
-
-__host__ __device__ inline long long ds_block_count(int key_blocks, int query_tiles) {
-    return (long long)key_blocks * query_tiles - (long long)key_blocks * (key_blocks - 1);
-}
-
-// Chunk permutation of a row-major LDS tile whose rows are ROW_BYTES long.
-// Row bytes = 0 (mod 256): the four bits of the row, pairs exchanged.
-// Row bytes = 128 (mod 256): the three bits of row>>1, bits 0 and 2 exchanged.
-template <int ROW_BYTES>
-__device__ __forceinline__ constexpr int tile_swizzle(int row) {
-    if constexpr (ROW_BYTES % 256 == 0) {
-        return ((row & 3) << 2) | ((row >> 2) & 3);
-    } else {
-        const int u = row >> 1;
-        return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
-    }
-}
+using index_math::ds_block_count;
+using index_math::ds_block_index;
+using index_math::tile_swizzle;
 
 // global_load_lds with 4 bytes per lane (256 consecutive LDS bytes per wave instruction)
 __device__ __forceinline__ void direct_load_4_offset(const void* uniform_base, unsigned byte_offset, unsigned lds_base) {
@@ -83,57 +66,36 @@ __device__ __forceinline__ void direct_load_4_offset(const void* uniform_base, u
 }
 
 // One wave's share of the global_load_lds requests of a [64][ROW_BYTES] tile that
-// WAVES waves fetch together.  LDS slot 64*load + lane (16 bytes each) holds chunk
-// (slot % CHUNKS) ^ f(row) of row slot / CHUNKS.  PERIOD loads cover PERIOD_ROWS
-// whole rows; from one period to the next only the low bits of f change, so load
-// L = PERIOD*m + r reads at
-//     tile + m * PERIOD_ROWS * row_stride  +  (offset of load r) ^ 16 * (m % XOR_STEPS)
-// The periods of a wave's LOADS consecutive loads are m = wave * LOADS/PERIOD + j;
-// LOADS/PERIOD and XOR_STEPS are powers of two, so the two parts of m touch
-// different bits of the XOR term: the wave's part is folded into base[r] once and
-// j's part is a compile-time constant.  At a ragged end rows past `row_limit`
-// repeat that row (slow path).
+// WAVES waves fetch together; the offsets are those of index_math::TileRequestMath.
+// Full tiles take the fast form (a per-lane base per residue, computed once, plus
+// compile-time constants); at a ragged end rows past `row_limit` repeat that row
+// (general form).
 template <int ROW_BYTES, int WAVES>
 struct TileRequests {
-    static constexpr int CHUNKS = ROW_BYTES / 16;
-    static constexpr int LOADS = QTILE * ROW_BYTES / 1024 / WAVES;
-    static constexpr int PERIOD = CHUNKS == 24 ? 3 : 1;
-    static constexpr int PERIOD_ROWS = 64 * PERIOD / CHUNKS;
-    static constexpr int XOR_STEPS = CHUNKS == 16 ? 4 : 2;
-    static constexpr int PERIODS = LOADS / PERIOD;   // per wave
-    static_assert(CHUNKS == 8 || CHUNKS == 16 || CHUNKS == 24, "rows of 128, 256 or 384 bytes");
-    static_assert(QTILE * ROW_BYTES % (1024 * WAVES) == 0 && LOADS % PERIOD == 0, "tile must divide evenly over the waves");
-    static_assert(PERIODS == 1 || PERIODS == 2 || PERIODS == 4, "periods per wave must be a power of two");
+    using Math = index_math::TileRequestMath<ROW_BYTES, WAVES, QTILE>;
+    static constexpr int LOADS = Math::LOADS;
+    static constexpr int PERIOD = Math::PERIOD;
     unsigned base[PERIOD];
 
-    __device__ __forceinline__ static unsigned offset_of(int load, int lane, unsigned row_stride, int row_limit) {
-        const int slot = 64 * load + lane;
-        const int row = slot / CHUNKS;
-        const int chunk = (slot % CHUNKS) ^ tile_swizzle<ROW_BYTES>(row);
-        return (unsigned)min(row, row_limit) * row_stride + 16u * chunk;
-    }
     __device__ __forceinline__ void init(unsigned row_stride, int wave, int lane) {
 #pragma unroll
-        for (int r = 0; r < PERIOD; ++r) {
-            base[r] = offset_of(r, lane, row_stride, QTILE) ^ (16u * ((wave * PERIODS) % XOR_STEPS));
-        }
+        for (int r = 0; r < PERIOD; ++r) base[r] = Math::base_of(r, lane, row_stride, wave);
     }
     // `tile` = address of the tile's first row (uniform)
     __device__ __forceinline__ void request(const unsigned char* tile, unsigned row_stride, int row_limit,
                                             unsigned lds_target, int wave) const {
         if (row_limit >= QTILE - 1) {
-            const unsigned char* rows = tile + (size_t)(wave * PERIODS * PERIOD_ROWS) * row_stride;
+            const unsigned char* rows = tile + (size_t)Math::rows_before(0, wave) * row_stride;
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
-                direct_load_16_offset(rows + (size_t)(i / PERIOD * PERIOD_ROWS) * row_stride,
-                                      base[i % PERIOD] ^ (16u * ((i / PERIOD) % XOR_STEPS)),
-                                      lds_target + (wave * LOADS + i) * 1024);
+                direct_load_16_offset(rows + (size_t)Math::rows_before(i, 0) * row_stride,
+                                      Math::lane_part(base[i % PERIOD], i), lds_target + (wave * LOADS + i) * 1024);
             }
         } else {
             const int lane = fresh_lane_id();
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
-                direct_load_16_offset(tile, offset_of(wave * LOADS + i, lane, row_stride, row_limit),
+                direct_load_16_offset(tile, Math::offset_of(wave * LOADS + i, lane, row_stride, row_limit),
                                       lds_target + (wave * LOADS + i) * 1024);
             }
         }

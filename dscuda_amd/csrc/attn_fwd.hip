@@ -43,6 +43,7 @@
 //   by s_waitcnt vmcnt + one workgroup barrier per tile.
 #include "attn_kernels.h"
 #include "hip_common.h"
+#include "index_math.h"
 
 #include <cmath>
 #include <stdexcept>
@@ -378,27 +379,8 @@ struct PingPong {
     static constexpr int CLUSTERS = 8;
 };
 
-struct ForwardItem {
-    int batch_head;
-    int query_block;
-};
-
-// item `round` of workgroup `member` (of `members`) of a cluster that owns
-// `cluster_heads` (batch, head) pairs; false past the end of the list
-__device__ __forceinline__ bool forward_item(int round, int member, int members, int cluster, int clusters,
-                                             int cluster_heads, int query_blocks, ForwardItem& item) {
-    const int position = (round & 1) ? members - 1 - member : member;
-    const int index = round * members + position;
-    if (index >= cluster_heads * query_blocks) {
-        return false;
-    }
-    const int interleave = (cluster_heads % 2 == 0) ? 2 : 1;
-    const int group = index / (interleave * query_blocks);
-    const int rest = index % (interleave * query_blocks);
-    item.batch_head = cluster + clusters * (interleave * group + rest % interleave);
-    item.query_block = query_blocks - 1 - rest / interleave;
-    return true;
-}
+using index_math::forward_item;
+using index_math::ForwardItem;
 
 template <int DQK, int DV>
 __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(

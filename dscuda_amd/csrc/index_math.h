@@ -1,0 +1,145 @@
+// Integer arithmetic of the attention kernels that decides where data lives and
+// which workgroup does what: LDS chunk permutations, tile-request offsets, the
+// position of a dS block in the backward workspace, the work order of the
+// persistent forward kernel and the split of the decode tile list.  Kept free
+// of anything device-specific so that the same definitions compile for the
+// host, where tests enumerate them exhaustively (coverage, uniqueness,
+// fast path == general path).
+#pragma once
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define DSCUDA_HOST_DEVICE __host__ __device__
+#else
+#define DSCUDA_HOST_DEVICE
+#endif
+
+namespace dscuda {
+namespace index_math {
+
+// ---- LDS chunk permutations -------------------------------------------------
+// A row-major LDS tile keeps 16-byte chunk c of row r at position c ^ f(r).
+// Row bytes = 0 (mod 256): the four bits of the row, pairs exchanged.
+// Row bytes = 128 (mod 256): the three bits of row>>1, bits 0 and 2 exchanged.
+template <int ROW_BYTES>
+DSCUDA_HOST_DEVICE constexpr int tile_swizzle(int row) {
+    if constexpr (ROW_BYTES % 256 == 0) {
+        return ((row & 3) << 2) | ((row >> 2) & 3);
+    } else {
+        const int u = row >> 1;
+        return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
+    }
+}
+
+// ---- backward workspace -----------------------------------------------------
+// Position of dS block (key block kb of 128 keys, query tile qt of 64 queries),
+// qt >= 2*kb, key block major; and the number of such blocks of one head.
+DSCUDA_HOST_DEVICE inline long long ds_block_index(int kb, int qt, int query_tiles) {
+    return (long long)kb * query_tiles - (long long)kb * (kb - 1) + (qt - 2 * kb);
+}
+
+DSCUDA_HOST_DEVICE inline long long ds_block_count(int key_blocks, int query_tiles) {
+    return (long long)key_blocks * query_tiles - (long long)key_blocks * (key_blocks - 1);
+}
+
+// ---- tile requests of the backward kernels ------------------------------------
+// One wave's share of the global -> LDS requests of a [ROWS][ROW_BYTES] tile that
+// WAVES waves fetch together.  LDS slot 64*load + lane (16 bytes each) holds chunk
+// (slot % CHUNKS) ^ f(row) of row slot / CHUNKS.  PERIOD loads cover PERIOD_ROWS
+// whole rows; from one period to the next only the low bits of f change, so load
+// L = PERIOD*m + r reads at
+//     tile + m * PERIOD_ROWS * row_stride  +  (offset of load r) ^ 16 * (m % XOR_STEPS)
+// The periods of a wave's LOADS consecutive loads are m = wave * LOADS/PERIOD + j;
+// LOADS/PERIOD and XOR_STEPS are powers of two, so the two parts of m touch
+// different bits of the XOR term: the wave's part is folded into a per-lane base
+// once and j's part is a compile-time constant.
+template <int ROW_BYTES, int WAVES, int ROWS = 64>
+struct TileRequestMath {
+    static constexpr int CHUNKS = ROW_BYTES / 16;
+    static constexpr int LOADS = ROWS * ROW_BYTES / 1024 / WAVES;
+    static constexpr int PERIOD = CHUNKS == 24 ? 3 : 1;
+    static constexpr int PERIOD_ROWS = 64 * PERIOD / CHUNKS;
+    static constexpr int XOR_STEPS = CHUNKS == 16 ? 4 : 2;
+    static constexpr int PERIODS = LOADS / PERIOD;   // per wave
+    static_assert(CHUNKS == 8 || CHUNKS == 16 || CHUNKS == 24, "rows of 128, 256 or 384 bytes");
+    static_assert(ROWS * ROW_BYTES % (1024 * WAVES) == 0 && LOADS % PERIOD == 0, "tile must divide evenly over the waves");
+    static_assert(PERIODS == 1 || PERIODS == 2 || PERIODS == 4, "periods per wave must be a power of two");
+
+    // general form: byte offset of lane `lane` of load `load` from the tile's first row; rows past
+    // `row_limit` repeat that row
+    DSCUDA_HOST_DEVICE static unsigned offset_of(int load, int lane, unsigned row_stride, int row_limit) {
+        const int slot = 64 * load + lane;
+        const int row = slot / CHUNKS;
+        const int chunk = (slot % CHUNKS) ^ tile_swizzle<ROW_BYTES>(row);
+        return (unsigned)(row_limit < row ? row_limit : row) * row_stride + 16u * chunk;
+    }
+    // fast form, full tiles only: per-lane base of residue r (computed once per kernel) ...
+    DSCUDA_HOST_DEVICE static unsigned base_of(int r, int lane, unsigned row_stride, int wave) {
+        return offset_of(r, lane, row_stride, ROWS) ^ (16u * ((wave * PERIODS) % XOR_STEPS));
+    }
+    // ... the rows (from the tile's first) the uniform part of the address of the wave's load i skips ...
+    DSCUDA_HOST_DEVICE static constexpr int rows_before(int i, int wave) {
+        return wave * PERIODS * PERIOD_ROWS + i / PERIOD * PERIOD_ROWS;
+    }
+    // ... and the per-lane part of that load
+    DSCUDA_HOST_DEVICE static constexpr unsigned lane_part(unsigned base, int i) {
+        return base ^ (16u * ((i / PERIOD) % XOR_STEPS));
+    }
+};
+
+// ---- work order of the persistent forward kernel ------------------------------
+struct ForwardItem {
+    int batch_head;
+    int query_block;
+};
+
+// Item `round` of workgroup `member` (of `members`) of a cluster that owns
+// `cluster_heads` (batch, head) pairs (pairs cluster, cluster + clusters, ...);
+// false past the end of the list.  Inside a cluster the items are laid out two
+// heads at a time (one if the count is odd), blocks from the heaviest (last) to
+// the lightest, and cut into rounds of one item per workgroup; odd rounds are
+// handed out in reverse.
+DSCUDA_HOST_DEVICE inline bool forward_item(int round, int member, int members, int cluster, int clusters,
+                                            int cluster_heads, int query_blocks, ForwardItem& item) {
+    const int position = (round & 1) ? members - 1 - member : member;
+    const int index = round * members + position;
+    if (index >= cluster_heads * query_blocks) {
+        return false;
+    }
+    const int interleave = (cluster_heads % 2 == 0) ? 2 : 1;
+    const int group = index / (interleave * query_blocks);
+    const int rest = index % (interleave * query_blocks);
+    item.batch_head = cluster + clusters * (interleave * group + rest % interleave);
+    item.query_block = query_blocks - 1 - rest / interleave;
+    return true;
+}
+
+// ---- decode: cutting the tile list -------------------------------------------
+// The 64-token tiles of all sequences form one list (sequence after sequence),
+// cut into `workgroups` equal ranges.  A range that holds only part of a
+// sequence leaves a partial result in slot workgroup + sequence: ranges and
+// sequences both advance monotonically, so no two (range, sequence) pairs that
+// intersect share a slot, and every slot is below workgroups + sequences.
+DSCUDA_HOST_DEVICE inline int tiles_per_range(int total_tiles, int workgroups) {
+    return (total_tiles + workgroups - 1) / workgroups;
+}
+
+DSCUDA_HOST_DEVICE inline int range_begin_of(int total_tiles, int workgroups, int workgroup) {
+    const int first = workgroup * tiles_per_range(total_tiles, workgroups);
+    return first < total_tiles ? first : total_tiles;
+}
+
+DSCUDA_HOST_DEVICE inline int range_end_of(int total_tiles, int workgroups, int begin) {
+    const int last = begin + tiles_per_range(total_tiles, workgroups);
+    return last < total_tiles ? last : total_tiles;
+}
+
+// First and last range that hold tiles of a sequence of `own` > 0 tiles that starts at tile `before`.
+DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total_tiles, int workgroups, int before, int own, int& first,
+                                                  int& last) {
+    const int per = tiles_per_range(total_tiles, workgroups);
+    first = before / per;
+    last = (before + own - 1) / per;
+}
+
+}  // namespace index_math
+}  // namespace dscuda

@@ -45,6 +45,7 @@
 //   call stays capturable.
 #include "attn_kernels.h"
 #include "hip_common.h"
+#include "index_math.h"
 
 #include <algorithm>
 #include <stdexcept>
@@ -71,8 +72,7 @@ constexpr int EPILOGUE_PITCH = 1024 + 16;   // bytes per staged output row
 typedef const __attribute__((address_space(1))) void* global_pointer;
 
 __device__ __forceinline__ int swizzle_of_row(int row) {
-    const int u = row >> 1;
-    return ((u & 1) << 2) | (u & 2) | ((u >> 2) & 1);
+    return index_math::tile_swizzle<ROW_BYTES>(row);
 }
 
 __device__ __forceinline__ float uniform(float value) {
@@ -659,9 +659,8 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         range_begin = prefix[sequence];
         range_end = prefix[sequence + 1];
     } else {
-        const int per = (total + workgroups - 1) / workgroups;
-        range_begin = min(workgroup * per, total);
-        range_end = min(range_begin + per, total);
+        range_begin = index_math::range_begin_of(total, workgroups, workgroup);
+        range_end = index_math::range_end_of(total, workgroups, range_begin);
         // first sequence whose tiles reach past range_begin
         int low = 0, high = batch_size;
         while (low < high) {
@@ -772,9 +771,8 @@ __global__ __launch_bounds__(128) void mla_decode_combine_kernel(
     total = sums[0][1] + sums[1][1];
     const int own = tiles_of(cache_lengths[sequence]);
     if (own == 0) return;
-    const int per = (total + workgroups - 1) / workgroups;
-    const int first = before / per;
-    const int last = (before + own - 1) / per;
+    int first, last;
+    index_math::ranges_of_sequence(total, workgroups, before, own, first, last);
     if (first == last) return;  // finished in place by the split kernel
 
     const size_t slots = (size_t)workgroups + batch_size;

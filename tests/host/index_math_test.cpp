@@ -1,0 +1,236 @@
+// Exhaustive host-side checks of dscuda_amd/csrc/index_math.h, the integer arithmetic the kernels share with
+// this test: compiled with the host compiler and run by tests/test_index_math.py.  Every check enumerates its
+// whole domain; a failure prints the first counterexample and the program exits non-zero.
+#include "index_math.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <set>
+#include <utility>
+#include <vector>
+
+using namespace dscuda::index_math;
+
+static int failures = 0;
+#define EXPECT(condition, ...)                                  \
+    do {                                                        \
+        if (!(condition)) {                                     \
+            if (failures++ < 20) {                              \
+                std::printf("FAIL %s:%d %s: ", __FILE__, __LINE__, #condition); \
+                std::printf(__VA_ARGS__);                       \
+                std::printf("\n");                              \
+            }                                                   \
+        }                                                       \
+    } while (0)
+
+// ---- chunk permutation: stays inside the row, is a permutation, and spreads the two read patterns over the banks
+template <int ROW_BYTES>
+void check_swizzle() {
+    constexpr int CHUNKS = ROW_BYTES / 16;
+    constexpr int SPAN = ROW_BYTES % 256 == 0 ? 16 : 8;
+    for (int row = 0; row < 128; ++row) {
+        const int f = tile_swizzle<ROW_BYTES>(row);
+        EXPECT(f >= 0 && f < SPAN, "ROW_BYTES %d row %d f %d", ROW_BYTES, row, f);
+        std::set<int> seen;
+        for (int chunk = 0; chunk < CHUNKS; ++chunk) {
+            const int position = chunk ^ f;
+            EXPECT(position >= 0 && position < CHUNKS, "ROW_BYTES %d row %d chunk %d -> %d", ROW_BYTES, row, chunk, position);
+            seen.insert(position);
+        }
+        EXPECT((int)seen.size() == CHUNKS, "ROW_BYTES %d row %d not a permutation", ROW_BYTES, row);
+    }
+    // 16-byte reads down a column: 16 lanes (rows r0 .. r0+15, the same chunk c of each) are served together and
+    // must touch 16 different 16-byte bank groups of the 256-byte bank line
+    for (int r0 = 0; r0 < 64; r0 += 16) {
+        for (int chunk = 0; chunk < CHUNKS; ++chunk) {
+            std::set<int> groups;
+            for (int lane = 0; lane < 16; ++lane) {
+                const int row = r0 + lane;
+                const int address = row * ROW_BYTES + 16 * (chunk ^ tile_swizzle<ROW_BYTES>(row));
+                groups.insert(address / 16 % 16);
+            }
+            EXPECT(groups.size() == 16, "ROW_BYTES %d rows %d.. chunk %d: %zu of 16 bank groups", ROW_BYTES, r0, chunk, groups.size());
+        }
+    }
+    // transposing 8-byte reads: 16 lanes cover 4 rows (r0 .. r0+3, r0 a multiple of 4) x one 64-byte column block
+    // (chunks 4b .. 4b+3, two lanes per chunk): the 16 chunks touched must lie in 16 different bank groups
+    for (int r0 = 0; r0 < 64; r0 += 4) {
+        for (int block = 0; block < CHUNKS / 4; ++block) {
+            std::set<int> groups;
+            for (int row = r0; row < r0 + 4; ++row) {
+                for (int c = 0; c < 4; ++c) {
+                    const int address = row * ROW_BYTES + 16 * ((4 * block + c) ^ tile_swizzle<ROW_BYTES>(row));
+                    groups.insert(address / 16 % 16);
+                }
+            }
+            EXPECT(groups.size() == 16, "ROW_BYTES %d rows %d.. block %d: %zu of 16 bank groups", ROW_BYTES, r0, block, groups.size());
+        }
+    }
+}
+
+// ---- tile requests: the fast form equals the general form, and the loads of all waves tile the LDS copy exactly
+template <int ROW_BYTES, int WAVES>
+void check_requests() {
+    using Math = TileRequestMath<ROW_BYTES, WAVES, 64>;
+    for (unsigned heads : {1u, 3u, 128u}) {
+        const unsigned row_stride = heads * ROW_BYTES;
+        std::vector<int> covered(64 * Math::CHUNKS, 0);
+        for (int wave = 0; wave < WAVES; ++wave) {
+            for (int i = 0; i < Math::LOADS; ++i) {
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int load = wave * Math::LOADS + i;
+                    const unsigned general = Math::offset_of(load, lane, row_stride, 63);
+                    const unsigned base = Math::base_of(i % Math::PERIOD, lane, row_stride, wave);
+                    const unsigned long long fast = (unsigned long long)Math::rows_before(i, wave) * row_stride + Math::lane_part(base, i);
+                    EXPECT(fast == general, "ROW_BYTES %d WAVES %d stride %u wave %d load %d lane %d: fast %llu general %u",
+                           ROW_BYTES, WAVES, row_stride, wave, i, lane, fast, general);
+                    // LDS slot 64*load + lane must receive chunk (slot % CHUNKS) ^ f(row) of row slot / CHUNKS
+                    const int slot = 64 * load + lane;
+                    const int row = slot / Math::CHUNKS;
+                    const unsigned expected = (unsigned)row * row_stride + 16u * ((slot % Math::CHUNKS) ^ tile_swizzle<ROW_BYTES>(row));
+                    EXPECT(general == expected, "slot %d", slot);
+                    const int source_chunk = (int)((general - (unsigned)row * row_stride) / 16);
+                    ++covered[row * Math::CHUNKS + source_chunk];
+                }
+            }
+        }
+        for (int index = 0; index < 64 * Math::CHUNKS; ++index) {
+            EXPECT(covered[index] == 1, "ROW_BYTES %d WAVES %d: chunk %d of the tile fetched %d times", ROW_BYTES, WAVES, index, covered[index]);
+        }
+        // ragged end: rows past the limit repeat the limit row, nothing before the tile or past that row is read
+        for (int row_limit : {0, 1, 17, 62}) {
+            for (int load = 0; load < WAVES * Math::LOADS; ++load) {
+                for (int lane = 0; lane < 64; ++lane) {
+                    const unsigned offset = Math::offset_of(load, lane, row_stride, row_limit);
+                    EXPECT(offset < (unsigned)row_limit * row_stride + ROW_BYTES, "row_limit %d load %d lane %d offset %u", row_limit, load, lane, offset);
+                }
+            }
+        }
+    }
+}
+
+// ---- dS blocks: key-block-major enumeration of the causal (key block, query tile) pairs, without gaps
+void check_ds_blocks() {
+    for (int sequence = 1; sequence <= 4200; sequence += (sequence < 600 ? 1 : 97)) {
+        const int query_tiles = (sequence + 63) / 64, key_blocks = (sequence + 127) / 128;
+        long long next = 0;
+        for (int kb = 0; kb < key_blocks; ++kb) {
+            for (int qt = 2 * kb; qt < query_tiles; ++qt) {
+                EXPECT(ds_block_index(kb, qt, query_tiles) == next, "S %d kb %d qt %d", sequence, kb, qt);
+                ++next;
+            }
+        }
+        EXPECT(ds_block_count(key_blocks, query_tiles) == next, "S %d count %lld enumerated %lld", sequence,
+               ds_block_count(key_blocks, query_tiles), next);
+    }
+}
+
+// ---- forward work order: every (batch*head, query block) exactly once, heads stay with their cluster, and with an
+// even number of heads per cluster and rounds that divide evenly every workgroup gets the same number of key tiles
+void check_forward_items() {
+    for (int clusters : {1, 8}) {
+        for (int batch_heads : {1, 2, 7, 8, 16, 24, 40, 128, 136}) {
+            if (batch_heads % clusters != 0) continue;
+            for (int query_blocks : {1, 2, 3, 5, 16, 64}) {
+                const int cluster_heads = batch_heads / clusters;
+                for (int members : {1, 2, 3, 5, 32}) {
+                    if (members > cluster_heads * query_blocks) continue;
+                    std::vector<int> visits(batch_heads * query_blocks, 0);
+                    long long lightest = -1, heaviest = -1;
+                    for (int cluster = 0; cluster < clusters; ++cluster) {
+                        for (int member = 0; member < members; ++member) {
+                            long long work = 0;
+                            ForwardItem item;
+                            int round = 0;
+                            for (; forward_item(round, member, members, cluster, clusters, cluster_heads, query_blocks, item); ++round) {
+                                EXPECT(item.batch_head >= 0 && item.batch_head < batch_heads && item.batch_head % clusters == cluster,
+                                       "head %d cluster %d", item.batch_head, cluster);
+                                EXPECT(item.query_block >= 0 && item.query_block < query_blocks, "block %d", item.query_block);
+                                ++visits[item.batch_head * query_blocks + item.query_block];
+                                work += item.query_block + 1;
+                            }
+                            // the list ends for good: no item reappears after the first miss
+                            EXPECT(!forward_item(round + 1, member, members, cluster, clusters, cluster_heads, query_blocks, item) ||
+                                       round * members + members > cluster_heads * query_blocks - members,
+                                   "item after the end");
+                            lightest = lightest < 0 ? work : std::min(lightest, work);
+                            heaviest = std::max(heaviest, work);
+                        }
+                    }
+                    for (int index = 0; index < batch_heads * query_blocks; ++index) {
+                        EXPECT(visits[index] == 1, "clusters %d heads %d blocks %d members %d: item %d visited %d times", clusters,
+                               batch_heads, query_blocks, members, index, visits[index]);
+                    }
+                    const int rounds = cluster_heads * query_blocks / members;
+                    if (cluster_heads % 2 == 0 && (cluster_heads * query_blocks) % members == 0 && rounds % 2 == 0 &&
+                        (2 * query_blocks) % members == 0) {
+                        EXPECT(lightest == heaviest, "clusters %d heads %d blocks %d members %d: work %lld .. %lld", clusters, batch_heads,
+                               query_blocks, members, lightest, heaviest);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- decode: the ranges partition the tile list; (range, sequence) pairs that intersect own distinct slots
+void check_decode_ranges() {
+    unsigned state = 12345;
+    auto random = [&](int low, int high) { state = state * 1664525u + 1013904223u; return low + (int)((state >> 8) % (unsigned)(high - low + 1)); };
+    for (int trial = 0; trial < 400; ++trial) {
+        const int sequences = random(1, 70);
+        const int workgroups = random(1, 300);
+        std::vector<int> prefix(sequences + 1, 0);
+        for (int s = 0; s < sequences; ++s) prefix[s + 1] = prefix[s] + random(trial % 3 == 0 ? 0 : 1, trial % 2 ? 130 : 5);
+        const int total = prefix[sequences];
+        if (total == 0) continue;
+        int expected_begin = 0;
+        std::set<int> slots;
+        std::vector<int> covered(total, 0);
+        for (int w = 0; w < workgroups; ++w) {
+            const int begin = range_begin_of(total, workgroups, w), end = range_end_of(total, workgroups, begin);
+            EXPECT(begin == std::min(expected_begin, total) && end >= begin && end <= total, "workgroup %d range %d..%d", w, begin, end);
+            expected_begin = end;
+            for (int s = 0; s < sequences; ++s) {
+                const int low = std::max(begin, prefix[s]), high = std::min(end, prefix[s + 1]);
+                if (low >= high) continue;
+                for (int tile = low; tile < high; ++tile) ++covered[tile];
+                const bool whole = low == prefix[s] && high == prefix[s + 1];
+                int first, last;
+                ranges_of_sequence(total, workgroups, prefix[s], prefix[s + 1] - prefix[s], first, last);
+                EXPECT(first <= w && w <= last, "sequence %d is in range %d but its ranges are %d..%d", s, w, first, last);
+                EXPECT(whole == (first == last), "sequence %d whole %d first %d last %d", s, (int)whole, first, last);
+                if (!whole) {
+                    const int slot = w + s;
+                    EXPECT(slot < workgroups + sequences, "slot %d", slot);
+                    EXPECT(slots.insert(slot).second, "slot %d used twice (workgroup %d sequence %d)", slot, w, s);
+                }
+            }
+        }
+        EXPECT(expected_begin == total, "ranges end at %d of %d", expected_begin, total);
+        for (int tile = 0; tile < total; ++tile) EXPECT(covered[tile] == 1, "tile %d covered %d times", tile, covered[tile]);
+    }
+}
+
+int main() {
+    check_swizzle<128>();
+    check_swizzle<256>();
+    check_swizzle<384>();
+    check_swizzle<1152>();
+    check_requests<384, 4>();
+    check_requests<256, 4>();
+    check_requests<128, 4>();
+    check_requests<384, 8>();
+    check_requests<256, 8>();
+    check_requests<128, 8>();
+    check_ds_blocks();
+    check_forward_items();
+    check_decode_ranges();
+    if (failures) {
+        std::printf("%d check(s) failed\n", failures);
+        return 1;
+    }
+    std::printf("index_math: all checks passed\n");
+    return 0;
+}
