@@ -113,6 +113,33 @@ DSCUDA_HOST_DEVICE inline bool forward_item(int round, int member, int members, 
     return true;
 }
 
+// ---- decode: tile loads -------------------------------------------------------
+// A [64][ROW_BYTES] tile of consecutive rows is fetched by four waves, wave w
+// filling rows 16w .. 16w+15 with 1 KB instructions: LDS slot 64*i + lane of the
+// wave's share (16 bytes each) holds chunk (slot % CHUNKS) ^ f(row) of local row
+// slot / CHUNKS.  With i a compile-time constant a wave instruction spans at most
+// two rows, so the row part of the offset is wave-uniform and the lane part costs
+// an add, an xor and a shift-add per candidate row.  Rows past `row_limit` (of
+// the tile) repeat that row.  f depends on bits 1..3 of the row only, which
+// 16*wave leaves alone.
+template <int ROW_BYTES>
+DSCUDA_HOST_DEVICE inline unsigned contiguous_load_offset(int wave, int i, int lane, int row_limit) {
+    constexpr int CHUNKS = ROW_BYTES / 16;
+    const int first_row = (64 * i) / CHUNKS;                 // row of lane 0 (within the wave's 16 rows)
+    const int boundary = CHUNKS * (first_row + 1) - 64 * i;  // first lane of the next row (may be >= 64)
+    const int tile_row_a = 16 * wave + first_row;
+    const unsigned row_a = (unsigned)(tile_row_a < row_limit ? tile_row_a : row_limit) * ROW_BYTES;
+    unsigned offset = row_a + 16u * (unsigned)((lane + 64 * i - CHUNKS * first_row) ^ tile_swizzle<ROW_BYTES>(first_row));
+    if (boundary < 64) {
+        const int tile_row_b = 16 * wave + first_row + 1;
+        const unsigned row_b = (unsigned)(tile_row_b < row_limit ? tile_row_b : row_limit) * ROW_BYTES;
+        const unsigned other =
+            row_b + 16u * (unsigned)((lane + 64 * i - CHUNKS * (first_row + 1)) ^ tile_swizzle<ROW_BYTES>(first_row + 1));
+        offset = lane >= boundary ? other : offset;
+    }
+    return offset;
+}
+
 // ---- decode: cutting the tile list -------------------------------------------
 // The 64-token tiles of all sequences form one list (sequence after sequence),
 // cut into `workgroups` equal ranges.  A range that holds only part of a

@@ -134,22 +134,11 @@ __device__ __forceinline__ TileSource locate_tile(unsigned char* stage_base, con
     return source;
 }
 
-// Load number i (0..17) of a contiguous tile; i is a constant after unrolling,
-// which leaves scalar arithmetic for the row part of the address and three
-// cheap vector ops (add, xor, shift-add) per candidate row for the lane part.
+// Load number i (0..17) of a contiguous tile; i is a constant after unrolling
+// (offsets: index_math::contiguous_load_offset).
 __device__ __forceinline__ void issue_contiguous_load(const TileSource& source, int wave, int i, int lane) {
-    const int first_row = (64 * i) / CHUNKS;                 // row of lane 0 (within the wave's 16 rows)
-    const int boundary = CHUNKS * (first_row + 1) - 64 * i;  // first lane of the next row (may be >= 64)
-    // f depends on bits 1..3 of the row; 16*wave leaves them alone
-    const unsigned row_a = (unsigned)min(16 * wave + first_row, source.row_limit) * ROW_BYTES;        // scalar
-    unsigned offset = row_a + 16u * (unsigned)((lane + 64 * i - CHUNKS * first_row) ^ swizzle_of_row(first_row));
-    if (boundary < 64) {
-        const unsigned row_b = (unsigned)min(16 * wave + first_row + 1, source.row_limit) * ROW_BYTES;
-        const unsigned other =
-            row_b + 16u * (unsigned)((lane + 64 * i - CHUNKS * (first_row + 1)) ^ swizzle_of_row(first_row + 1));
-        offset = lane >= boundary ? other : offset;
-    }
-    direct_load_16_offset(source.tile_base, offset, source.lds_base + i * 1024);
+    direct_load_16_offset(source.tile_base, index_math::contiguous_load_offset<ROW_BYTES>(wave, i, lane, source.row_limit),
+                          source.lds_base + i * 1024);
 }
 
 // All 18 loads of a tile at once (first tile of a walk, and every tile of the

@@ -174,6 +174,31 @@ void check_forward_items() {
     }
 }
 
+// ---- decode tile loads: the two-candidate-row form equals the general form for every wave, load, lane and limit
+void check_decode_loads() {
+    constexpr int ROW_BYTES = 1152, CHUNKS = ROW_BYTES / 16, LOADS = 18;
+    for (int row_limit : {0, 1, 15, 16, 17, 31, 40, 62, 63, 64, 1000}) {
+        std::vector<int> fetched(64 * CHUNKS, 0);
+        for (int wave = 0; wave < 4; ++wave) {
+            for (int i = 0; i < LOADS; ++i) {
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int slot = 64 * i + lane;                  // of the wave's 18 KB
+                    const int local_row = slot / CHUNKS, position = slot % CHUNKS;
+                    const int row = 16 * wave + local_row;
+                    const int chunk = position ^ tile_swizzle<ROW_BYTES>(row);
+                    const unsigned general = (unsigned)std::min(row, row_limit) * ROW_BYTES + 16u * chunk;
+                    const unsigned fast = contiguous_load_offset<ROW_BYTES>(wave, i, lane, row_limit);
+                    EXPECT(fast == general, "row_limit %d wave %d load %d lane %d: %u vs %u", row_limit, wave, i, lane, fast, general);
+                    if (row_limit >= 63) ++fetched[row * CHUNKS + chunk];
+                }
+            }
+        }
+        if (row_limit >= 63) {
+            for (int index = 0; index < 64 * CHUNKS; ++index) EXPECT(fetched[index] == 1, "chunk %d fetched %d times", index, fetched[index]);
+        }
+    }
+}
+
 // ---- decode: the ranges partition the tile list; (range, sequence) pairs that intersect own distinct slots
 void check_decode_ranges() {
     unsigned state = 12345;
@@ -226,6 +251,7 @@ int main() {
     check_requests<128, 8>();
     check_ds_blocks();
     check_forward_items();
+    check_decode_loads();
     check_decode_ranges();
     if (failures) {
         std::printf("%d check(s) failed\n", failures);
