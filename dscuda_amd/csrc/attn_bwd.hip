@@ -102,45 +102,24 @@ struct TileRequests {
     }
 };
 
-// Per-lane byte offsets of the fragment reads of a row-major swizzled tile.
-// The swizzle only touches the low SPAN chunk positions of a row, so a handful
-// of per-lane values plus compile-time immediates reach every fragment; a user
-// adds the (run-time) tile base to the per-lane values once per tile.
-//
-//   natural[i]        row lane%32, chunk (2i + g) ^ f(row): the operand whose
-//                     contraction index is the tile column (k-step ks = NAT*m + i
-//                     lies NAT*32*m bytes further, 32 rows down 32*ROW_BYTES)
-//   transposed[h][i]  for ds_read_b64_tr_b16: row 4g + s/4 + 8h (s = lane%16),
-//                     chunk (4i + 2*((lane/16)%2) + (s%4)/2) ^ f(row), byte 8*(s%2):
-//                     the operand whose contraction index is the tile row; MFMA
-//                     row/column lane%32 = tile column 32*block + lane%32, k = rows
-//                     {4g..4g+3, 8+4g..8+4g+3} of a 16-row step -- the order a
-//                     C-layout register block carries (block = TR*m + i lies
-//                     TR*64*m bytes further)
+// Per-lane byte offsets of the fragment reads of a row-major swizzled tile
+// (index_math::TileReadMath); a user adds the (run-time) tile base to the per-lane
+// values once per tile.
 template <int ROW_BYTES>
 struct TileReads {
-    static constexpr int SPAN = (ROW_BYTES % 256 == 0) ? 16 : 8;
-    static constexpr int NAT = SPAN / 2;
-    static constexpr int TR = SPAN / 4;
+    using Math = index_math::TileReadMath<ROW_BYTES>;
+    static constexpr int NAT = Math::NAT;
+    static constexpr int TR = Math::TR;
     unsigned natural[NAT];
     unsigned transposed[2][TR];
 
     __device__ __forceinline__ void init(int lane) {
-        const int lq = lane % 32;
-        const int g = lane / 32;
 #pragma unroll
-        for (int i = 0; i < NAT; ++i) {
-            natural[i] = lq * ROW_BYTES + 16 * ((2 * i + g) ^ tile_swizzle<ROW_BYTES>(lq));
-        }
-        const int s = lane % 16;
-        const int low = 2 * ((lane / 16) % 2) + (s % 4) / 2;
+        for (int i = 0; i < NAT; ++i) natural[i] = Math::natural(i, lane);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int row = 4 * g + s / 4 + 8 * h;
 #pragma unroll
-            for (int i = 0; i < TR; ++i) {
-                transposed[h][i] = row * ROW_BYTES + 16 * ((4 * i + low) ^ tile_swizzle<ROW_BYTES>(row)) + 8 * (s % 2);
-            }
+            for (int i = 0; i < TR; ++i) transposed[h][i] = Math::transposed(h, i, lane);
         }
     }
 };
@@ -148,20 +127,20 @@ struct TileReads {
 // `at` = TileReads::natural plus the tile's LDS offset; rows ROW0 + lane%32, k-step KS
 template <int ROW_BYTES, int ROW0, int KS>
 __device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* lds, const unsigned (&at)[TileReads<ROW_BYTES>::NAT]) {
-    constexpr int NAT = TileReads<ROW_BYTES>::NAT;
-    return *reinterpret_cast<const bf16x8*>(lds + at[KS % NAT] + (ROW0 * ROW_BYTES + (KS / NAT) * (NAT * 32)));
+    using Math = index_math::TileReadMath<ROW_BYTES>;
+    return *reinterpret_cast<const bf16x8*>(lds + at[KS % Math::NAT] + Math::natural_constant(ROW0, KS));
 }
 
 // `at` = TileReads::transposed plus the tile's LDS offset; 16 rows from ROW0, column block BLOCK
 template <int ROW_BYTES, int ROW0, int BLOCK>
 __device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* lds,
                                                       const unsigned (&at)[2][TileReads<ROW_BYTES>::TR]) {
-    constexpr int TR = TileReads<ROW_BYTES>::TR;
-    constexpr int CONSTANT = ROW0 * ROW_BYTES + (BLOCK / TR) * (TR * 64);
+    using Math = index_math::TileReadMath<ROW_BYTES>;
+    constexpr int CONSTANT = Math::transposed_constant(ROW0, BLOCK);
     const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (transposing_read_pointer)(lds + at[0][BLOCK % TR] + CONSTANT));
+        (transposing_read_pointer)(lds + at[0][BLOCK % Math::TR] + CONSTANT));
     const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (transposing_read_pointer)(lds + at[1][BLOCK % TR] + CONSTANT));
+        (transposing_read_pointer)(lds + at[1][BLOCK % Math::TR] + CONSTANT));
     return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 

@@ -86,6 +86,49 @@ struct TileRequestMath {
     }
 };
 
+// ---- fragment reads of the backward kernels ------------------------------------
+// Per-lane byte offsets of the MFMA operand fragments inside a row-major swizzled
+// LDS tile.  The swizzle only touches the low SPAN chunk positions of a row, so a
+// handful of per-lane values plus compile-time constants reach every fragment.
+//
+//   natural(i, lane)        row lane%32, chunk (2i + g) ^ f(row), g = lane/32: the
+//                           operand whose contraction index is the tile column;
+//                           k-step ks = NAT*m + i lies NAT*32*m bytes further, 32
+//                           rows down 32*ROW_BYTES (natural_constant)
+//   transposed(h, i, lane)  for ds_read_b64_tr_b16: row 4g + s/4 + 8h (s = lane%16),
+//                           chunk (4i + 2*((lane/16)%2) + (s%4)/2) ^ f(row), byte
+//                           8*(s%2): the operand whose contraction index is the
+//                           tile row; MFMA row/column lane%32 = tile column
+//                           32*block + lane%32, k = rows {4g..4g+3, 8+4g..8+4g+3}
+//                           of a 16-row step -- the order a C-layout register block
+//                           carries; block = TR*m + i lies TR*64*m bytes further
+//                           (transposed_constant)
+template <int ROW_BYTES>
+struct TileReadMath {
+    static constexpr int SPAN = (ROW_BYTES % 256 == 0) ? 16 : 8;
+    static constexpr int NAT = SPAN / 2;
+    static constexpr int TR = SPAN / 4;
+
+    DSCUDA_HOST_DEVICE static unsigned natural(int i, int lane) {
+        const int lq = lane % 32;
+        const int g = lane / 32;
+        return lq * ROW_BYTES + 16 * ((2 * i + g) ^ tile_swizzle<ROW_BYTES>(lq));
+    }
+    DSCUDA_HOST_DEVICE static unsigned transposed(int h, int i, int lane) {
+        const int g = lane / 32;
+        const int s = lane % 16;
+        const int low = 2 * ((lane / 16) % 2) + (s % 4) / 2;
+        const int row = 4 * g + s / 4 + 8 * h;
+        return row * ROW_BYTES + 16 * ((4 * i + low) ^ tile_swizzle<ROW_BYTES>(row)) + 8 * (s % 2);
+    }
+    DSCUDA_HOST_DEVICE static constexpr int natural_constant(int row0, int ks) {
+        return row0 * ROW_BYTES + (ks / NAT) * (NAT * 32);
+    }
+    DSCUDA_HOST_DEVICE static constexpr int transposed_constant(int row0, int block) {
+        return row0 * ROW_BYTES + (block / TR) * (TR * 64);
+    }
+};
+
 // ---- work order of the persistent forward kernel ------------------------------
 struct ForwardItem {
     int batch_head;

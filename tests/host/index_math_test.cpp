@@ -110,6 +110,61 @@ void check_requests() {
     }
 }
 
+// ---- fragment reads: which tile element ends up in which operand register
+// A byte address inside a swizzled LDS tile -> (row, first column) of the 16-bit elements stored there.
+template <int ROW_BYTES>
+void locate(unsigned address, int& row, int& column) {
+    row = (int)(address / ROW_BYTES);
+    const int in_row = (int)(address % ROW_BYTES);
+    const int chunk = (in_row / 16) ^ tile_swizzle<ROW_BYTES>(row);
+    column = 8 * chunk + (in_row % 16) / 2;
+}
+
+// MFMA 32x32x16 operand layout: lane l holds row (or column) l % 32 of the operand and the eight contraction
+// indices 8 * (l / 32) + j.  ds_read_b64_tr_b16: within a block of 16 lanes, lane i receives, as element e of its
+// four, 16-bit element i % 4 of the eight bytes that lane i / 4 + 4 * e addressed.
+template <int ROW_BYTES>
+void check_fragment_reads() {
+    using Math = TileReadMath<ROW_BYTES>;
+    constexpr int COLUMNS = ROW_BYTES / 2;
+    // natural: operand row = tile row ROW0 + l % 32, contraction index = tile column 16 * KS + 8 * (l / 32) + j
+    for (int row0 : {0, 32}) {
+        for (int ks = 0; ks < COLUMNS / 16; ++ks) {
+            for (int lane = 0; lane < 64; ++lane) {
+                int row, column;
+                locate<ROW_BYTES>(Math::natural(ks % Math::NAT, lane) + Math::natural_constant(row0, ks), row, column);
+                EXPECT(row == row0 + lane % 32 && column == 16 * ks + 8 * (lane / 32),
+                       "natural ROW_BYTES %d row0 %d ks %d lane %d -> row %d column %d", ROW_BYTES, row0, ks, lane, row, column);
+            }
+        }
+    }
+    // transposed: operand row = tile column 32 * BLOCK + l % 32, contraction index j -> tile row
+    // ROW0 + {4g .. 4g+3, 8+4g .. 8+4g+3}[j], g = l / 32 (two reads, h = 0 for j < 4, h = 1 for j >= 4)
+    for (int row0 : {0, 16, 32, 48}) {
+        for (int block = 0; block < COLUMNS / 32; ++block) {
+            for (int h = 0; h < 2; ++h) {
+                unsigned address[64];
+                for (int lane = 0; lane < 64; ++lane) {
+                    address[lane] = Math::transposed(h, block % Math::TR, lane) + Math::transposed_constant(row0, block);
+                    EXPECT(address[lane] % 8 == 0, "transposed read not 8-byte aligned");
+                }
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int block16 = lane / 16, i = lane % 16, g = lane / 32;
+                    for (int e = 0; e < 4; ++e) {
+                        const int source = 16 * block16 + i / 4 + 4 * e;
+                        int row, column;
+                        locate<ROW_BYTES>(address[source], row, column);
+                        column += i % 4;
+                        EXPECT(column == 32 * block + lane % 32 && row == row0 + 8 * h + 4 * g + e,
+                               "transposed ROW_BYTES %d row0 %d block %d h %d lane %d e %d -> row %d column %d", ROW_BYTES, row0,
+                               block, h, lane, e, row, column);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- dS blocks: key-block-major enumeration of the causal (key block, query tile) pairs, without gaps
 void check_ds_blocks() {
     for (int sequence = 1; sequence <= 4200; sequence += (sequence < 600 ? 1 : 97)) {
@@ -249,6 +304,9 @@ int main() {
     check_requests<384, 8>();
     check_requests<256, 8>();
     check_requests<128, 8>();
+    check_fragment_reads<128>();
+    check_fragment_reads<256>();
+    check_fragment_reads<384>();
     check_ds_blocks();
     check_forward_items();
     check_decode_loads();
