@@ -76,6 +76,21 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
                                            "data": "synthetic, GPU generator"}
     del lq, lk, lv, ldo, lout, llse, grads, workspace
 
+    # for scale only: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this chip with random
+    # operands, timed the same way; a plain GEMM is the practical ceiling of any MFMA-bound kernel here
+    try:
+        size = 8192
+        left = draw((size, size), 0.5)
+        right = draw((size, size), 0.5)
+        product = torch.empty(size, size, device=device, dtype=torch.bfloat16)
+        ms, _ = event_time_ms(lambda: torch.matmul(left, right, out=product), 40, 10)
+        results["bf16_gemm_8192_for_scale"] = {"ms": ms, "tflops": 2.0 * size ** 3 / ms / 1e9,
+                                               "frac_of_bf16_peak": 2.0 * size ** 3 / ms / 1e9 / PEAK_BF16_TFLOPS,
+                                               "what": "torch.matmul bf16, 0.5*N(0,1) operands"}
+        del left, right, product
+    except Exception as error:   # the comparison is optional; never let it break the measurement
+        results["bf16_gemm_8192_for_scale"] = {"error": str(error)}
+
     # flash attention forward, B=1 H=8 S=512 D=64 (latency bound: report time)
     fq, fk, fv, fscale = configs.flash_forward_inputs()
     fq, fk, fv = fq.to(device), fk.to(device), fv.to(device)
