@@ -7,7 +7,7 @@
 // fast path == general path).
 #pragma once
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define DSCUDA_HOST_DEVICE __host__ __device__
 #else
 #define DSCUDA_HOST_DEVICE
@@ -209,6 +209,42 @@ DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total_tiles, int workgroup
     const int per = tiles_per_range(total_tiles, workgroups);
     first = before / per;
     last = (before + own - 1) / per;
+}
+
+// ---- decode: how a call uses the caller's workspace ---------------------------
+// The workspace holds batch * heads * splits * (rank + 2) floats.  It is used as
+// `slots` partial-result slots of heads * (rank + 2) floats (slot = workgroup +
+// sequence, so slots = workgroups + batch) followed by one flag word per launched
+// workgroup.  The number of workgroups is capped so that slots stays at least one
+// below batch * splits and the flags fit the slot left over; when not even two
+// workgroups fit under that cap (splits == 1, batch == 1 with splits == 2, a single
+// compute unit) no
+// sequence is cut: one workgroup per sequence, no slots, flags at the start.
+struct DecodeLayout {
+    int workgroups;
+    int whole_sequences;
+    long long slots;
+    long long flag_offset;   // in floats from the start of the workspace
+    long long flag_words;
+};
+
+DSCUDA_HOST_DEVICE inline DecodeLayout decode_layout(int batch, int heads, int splits, int compute_units,
+                                                     int rows_per_group, int rank) {
+    DecodeLayout layout;
+    const long long head_groups = (heads + rows_per_group - 1) / rows_per_group;
+    const long long by_workspace = (long long)batch * (splits - 1) - 1;
+    const long long cutting = by_workspace < compute_units ? by_workspace : compute_units;
+    layout.whole_sequences = cutting < 2 ? 1 : 0;
+    if (layout.whole_sequences) {
+        layout.workgroups = batch;
+        layout.slots = 0;
+    } else {
+        layout.workgroups = (int)cutting;
+        layout.slots = (long long)layout.workgroups + batch;
+    }
+    layout.flag_offset = layout.slots * heads * (rank + 2);
+    layout.flag_words = head_groups * layout.workgroups;
+    return layout;
 }
 
 }  // namespace index_math

@@ -883,16 +883,10 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
         allow_large_lds(mla_decode_split_kernel<true>);
         prepared = true;
     }
-    // Workspace B*H*splits*(C+2) floats holds workgroups + batch partial-result
-    // slots of H*(C+2) floats and, behind them, one flag word per workgroup (the
-    // flags fit one more slot).  With splits == 1 every sequence is finished by
-    // one workgroup, no slot is used and the flags sit at the start.
-    const int whole_sequences = splits == 1 ? 1 : 0;
-    int workgroups = batch_size;
-    if (!whole_sequences) {
-        const long long by_workspace = (long long)batch_size * (splits - 1) - 1;
-        workgroups = (int)std::max<long long>(1, std::min<long long>(compute_units(), by_workspace));
-    }
+    // How the caller's B*H*splits*(C+2) floats are used: index_math::decode_layout.
+    const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
+    const int whole_sequences = layout.whole_sequences;
+    const int workgroups = layout.workgroups;
     const int head_groups = (heads + ROWS - 1) / ROWS;
     const dim3 grid(workgroups, head_groups);
     hipLaunchKernelGGL(mla_decode_split_kernel<false>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,

@@ -293,6 +293,35 @@ void check_decode_ranges() {
     }
 }
 
+// ---- decode workspace: slots and flag words stay inside the batch * heads * splits * (rank + 2) floats the caller
+// provides, for every batch size, head count and split count
+void check_decode_layout() {
+    constexpr int RANK = 512, ROWS = 128;
+    for (int compute_units : {1, 8, 256, 304}) {
+        for (int batch = 1; batch <= 80; ++batch) {
+            for (int heads : {1, 2, 16, 127, 128, 129, 160, 256}) {
+                for (int splits = 1; splits <= 34; ++splits) {
+                    const DecodeLayout layout = decode_layout(batch, heads, splits, compute_units, ROWS, RANK);
+                    const long long workspace = (long long)batch * heads * splits * (RANK + 2);
+                    EXPECT(layout.workgroups >= 1 && layout.workgroups <= std::max(batch, compute_units), "B %d H %d splits %d: %d workgroups",
+                           batch, heads, splits, layout.workgroups);
+                    EXPECT(layout.flag_offset + layout.flag_words <= workspace, "B %d H %d splits %d CUs %d: flags end at %lld of %lld floats",
+                           batch, heads, splits, compute_units, layout.flag_offset + layout.flag_words, workspace);
+                    if (layout.whole_sequences) {
+                        EXPECT(layout.workgroups == batch && layout.slots == 0 && layout.flag_offset == 0, "B %d splits %d", batch, splits);
+                    } else {
+                        EXPECT(layout.workgroups >= 2 && layout.slots == layout.workgroups + batch, "B %d splits %d", batch, splits);
+                        EXPECT(layout.flag_offset == layout.slots * heads * (RANK + 2), "B %d splits %d", batch, splits);
+                    }
+                }
+            }
+        }
+    }
+    // the case that used to put its flag word one float past the end
+    const DecodeLayout single = decode_layout(1, 128, 2, 256, ROWS, RANK);
+    EXPECT(single.whole_sequences == 1 && single.flag_offset == 0, "B 1 splits 2 must not cut the sequence");
+}
+
 int main() {
     check_swizzle<128>();
     check_swizzle<256>();
@@ -311,6 +340,7 @@ int main() {
     check_forward_items();
     check_decode_loads();
     check_decode_ranges();
+    check_decode_layout();
     if (failures) {
         std::printf("%d check(s) failed\n", failures);
         return 1;
