@@ -13,6 +13,7 @@
 #include "hip_common.h"
 
 #include <exception>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 
@@ -29,6 +30,35 @@ void check_positive(const char* what, int batch_size, int tokens, int heads) {
     if (batch_size <= 0 || tokens <= 0 || heads <= 0) {
         throw std::invalid_argument(std::string(what) + " requires positive batch, sequence and head counts");
     }
+}
+
+// Workspace of mla_decode_forward_static: one array per GPU, part of the loaded code
+// object, so it exists from module load to process exit and no call ever allocates.
+// In host code the array's name only stands for the symbol; the device address is
+// looked up once per device and every use below goes through that pointer.
+__device__ __align__(256) unsigned char static_decode_scratch[MLA_DECODE_STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+
+float* static_decode_scratch_of_current_device() {
+    static std::mutex guard;
+    static void* address_of_device[MAX_DEVICES] = {};
+    int device = 0;
+    HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= MAX_DEVICES) {
+        throw std::runtime_error("MLA decode (static workspace): device index " + std::to_string(device) +
+                                 " is beyond the " + std::to_string(MAX_DEVICES) + " devices supported");
+    }
+    std::lock_guard<std::mutex> lock(guard);
+    if (address_of_device[device] == nullptr) {
+        void* address = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(static_decode_scratch)));
+        if (address == nullptr) {
+            throw std::runtime_error("MLA decode (static workspace): the workspace symbol has no device address");
+        }
+        address_of_device[device] = address;
+    }
+    return static_cast<float*>(address_of_device[device]);
 }
 
 void check_prefill_heads(int qk_head_size, int v_head_size) {
@@ -79,6 +109,27 @@ void mla_decode_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __h
         throw std::invalid_argument(
             "MLA decode requires positive batch, head, page_size, pages_per_sequence and splits");
     }
+    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
+                        heads, page_size, pages_per_sequence, splits, scale, stream);
+}
+
+void mla_decode_forward_static(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                               const __hip_bfloat16* paged_kv_cache, const int* block_table, const int* cache_lengths,
+                               int batch_size, int heads, int kv_rank, int rope_size, int page_size,
+                               int pages_per_sequence, int splits, float scale, hipStream_t stream) {
+    check_shape(kv_rank, rope_size);
+    if (batch_size <= 0 || heads <= 0 || page_size <= 0 || pages_per_sequence <= 0 || splits <= 0) {
+        throw std::invalid_argument(
+            "MLA decode requires positive batch, head, page_size, pages_per_sequence and splits");
+    }
+    const std::size_t needed = mla_decode_workspace_elements(batch_size, heads, splits, kv_rank) * sizeof(float);
+    if (needed > MLA_DECODE_STATIC_SCRATCH_BYTES) {
+        throw std::invalid_argument(
+            "MLA decode (static workspace): batch*heads*splits*(rank+2) floats = " + std::to_string(needed) +
+            " bytes exceed the built-in workspace of " + std::to_string(MLA_DECODE_STATIC_SCRATCH_BYTES) +
+            " bytes; lower splits or call the variant that takes a caller workspace");
+    }
+    float* workspace = static_decode_scratch_of_current_device();
     mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
                         heads, page_size, pages_per_sequence, splits, scale, stream);
 }
@@ -172,6 +223,16 @@ extern "C" int dscuda_mla_decode(__hip_bfloat16* output, float* lse, const __hip
     return guarded([&] {
         dscuda::mla_decode_forward_cuda(output, lse, query, paged_cache, block_table, lengths, workspace, batch,
                                         heads, rank, rope, page_size, pages, splits, scale, stream);
+    });
+}
+
+extern "C" int dscuda_mla_decode_static(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
+                                        const __hip_bfloat16* paged_cache, const int* block_table,
+                                        const int* lengths, int batch, int heads, int rank, int rope, int page_size,
+                                        int pages, int splits, float scale, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_decode_forward_static(output, lse, query, paged_cache, block_table, lengths, batch, heads, rank,
+                                          rope, page_size, pages, splits, scale, stream);
     });
 }
 

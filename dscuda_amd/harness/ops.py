@@ -32,6 +32,7 @@ class _Mla:
         self.forward = bind(lib, "dscuda_mla_forward", [P] * 6 + [I] * 5 + [F, P])
         self.backward = bind(lib, "dscuda_mla_backward", [P] * 11 + [I] * 5 + [F, P])
         self.decode = bind(lib, "dscuda_mla_decode", [P] * 7 + [I] * 7 + [F, P])
+        self.decode_static = bind(lib, "dscuda_mla_decode_static", [P] * 6 + [I] * 7 + [F, P])
         self.workspace = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
         self.prefill_forward = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
         self.prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
@@ -161,4 +162,16 @@ def mla_decode(packed_query, paged_cache, block_table, lengths, scale, splits=8,
     checked(lib.lib, "mla", lib.decode(
         *pointers((out, lse, packed_query, paged_cache, block_table, lengths, workspace)),
         b, h, rank, rope, page_size, pages, splits, scale, stream()))
+    return out, lse
+
+
+def mla_decode_static(packed_query, paged_cache, block_table, lengths, scale, splits, out, lse, rank=512):
+    """dscuda_mla_decode_static: the decode call for callers that cannot allocate.  The caller passes every
+    input and output; partial results go to the workspace built into the library."""
+    _require_cuda(packed_query, paged_cache, block_table, lengths, out, lse)
+    b, _, h, width = packed_query.shape
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.decode_static(
+        *pointers((out, lse, packed_query, paged_cache, block_table, lengths)),
+        b, h, rank, width - rank, paged_cache.shape[1], block_table.shape[1], splits, scale, stream()))
     return out, lse

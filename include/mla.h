@@ -103,6 +103,39 @@ void mla_decode_forward_cuda(
     float scale,
     hipStream_t stream = nullptr);
 
+// Bytes of the workspace built into the library for mla_decode_forward_static
+// (one copy per GPU the library is loaded on, held until the process ends).
+constexpr std::size_t MLA_DECODE_STATIC_SCRATCH_BYTES = std::size_t(64) << 20;
+
+// mla_decode_forward_cuda for callers that cannot allocate or pass a workspace
+// (code under HIP graph capture, tight serving loops, harnesses that forbid
+// hipMalloc).  No counterpart in the reference.  Same arguments without the
+// workspace: the partial results and flags live in a fixed array inside the
+// library, and the call performs no allocation of any kind.  Sizes for which
+// batch*heads*splits*(kv_rank+2) floats exceed MLA_DECODE_STATIC_SCRATCH_BYTES
+// are rejected with std::invalid_argument (lower `splits`: the result does not
+// depend on it).  All calls on one GPU share that GPU's array: calls that
+// overlap in time on one GPU (different streams or threads) race; calls in
+// stream order do not, and nothing has to be cleared between them.  The first
+// call on a device looks up the array's address and must not be made under
+// stream capture.
+void mla_decode_forward_static(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* paged_kv_cache,
+    const int* block_table,
+    const int* cache_lengths,
+    int batch_size,
+    int heads,
+    int kv_rank,
+    int rope_size,
+    int page_size,
+    int pages_per_sequence,
+    int splits,
+    float scale,
+    hipStream_t stream = nullptr);
+
 // ---- additive: per-head MLA prefill (no counterpart in the reference) ------
 //
 // query/key [B,S,H,d_qk] with the rope slice stored after the nope slice,
@@ -191,6 +224,15 @@ int dscuda_mla_decode(  // mla_bridge.cu:58-73
     __hip_bfloat16* output, float* lse,
     const __hip_bfloat16* query, const __hip_bfloat16* paged_cache,
     const int* block_table, const int* lengths, float* workspace,
+    int batch, int heads, int rank, int rope, int page_size, int pages, int splits,
+    float scale, hipStream_t stream);
+
+// No counterpart in the reference: dscuda_mla_decode without the workspace argument, for
+// callers that cannot allocate (see dscuda::mla_decode_forward_static above for the limit).
+int dscuda_mla_decode_static(
+    __hip_bfloat16* output, float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* paged_cache,
+    const int* block_table, const int* lengths,
     int batch, int heads, int rank, int rope, int page_size, int pages, int splits,
     float scale, hipStream_t stream);
 
