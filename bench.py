@@ -26,13 +26,25 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch of the forward kernel at the headline workload, from the two
-# rocprofv3 --pmc runs whose summaries are profiles/pmc_fwd_fetch.txt (FETCH_SIZE 675103.5 KiB)
-# and profiles/pmc_fwd_write.txt (WRITE_SIZE 214073.0 KiB), each scaled by what the same counter
-# reads for a 1 GiB device copy (profiles/pmc_copy_*.txt: FETCH_SIZE reports half the bytes
-# read -> factor 2.0, WRITE_SIZE reports them all -> factor 1.0).  A recorded measurement, not
-# something this script can observe itself.
-FORWARD_TRAFFIC_BYTES = (675103.5 * 2.0 + 214073.0 * 1.0) * 1024
+PROFILES = ROOT / "profiles"
+
+
+def profiled_figures(stem, kernel_prefix):
+    """(HBM bytes per launch, settled microseconds) of the first kernel whose name starts with `kernel_prefix` in
+    profiles/<stem>.md, the summary `python -m dscuda_amd.profiler.capture` writes from rocprofv3's FETCH_SIZE /
+    WRITE_SIZE passes (each scaled by what the same counter reads for a 1 GiB device copy) and its kernel trace.
+    A recorded measurement of the committed kernels, not something this script can observe; (None, None) if the
+    summary is missing."""
+    path = PROFILES / f"{stem}.md"
+    if not path.is_file():
+        return None, None
+    for line in path.read_text().splitlines():
+        line = line.strip()
+        if line.startswith(kernel_prefix) and " :: " in line:
+            fields = dict(part.strip().split(" = ") for part in line.split(" :: ", 1)[1].split(" ; "))
+            nbytes = float(fields["hbm_bytes"])
+            return (None if nbytes != nbytes else nbytes), float(fields["time_us"])
+    return None, None
 
 
 SETTLE_MS = 40.0   # back-to-back launches before any timing: the chip's clock needs ~25 ms of load to settle
@@ -81,11 +93,48 @@ def cpu_baseline_forward(q, k, v, scale, gpu_out, gpu_lse, sample_heads):
     baseline = {
         "value": flops / seconds / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"{len(heads)} of {q.shape[2]} heads of the same workload, unfused fp32 PyTorch oracle, "
-                  f"{seconds:.1f} s, os.cpu_count()={os.cpu_count()}, torch {torch.__version__}",
+                  f"{seconds:.1f} s, {torch.get_num_threads()} intra-op threads (the cores counted), "
+                  f"os.cpu_count()={os.cpu_count()}, torch {torch.__version__}",
     }
     parity = {"heads_checked": len(heads), "o_max_abs": worst, "o_mean_abs": mean, "lse_max_abs": lse_err,
               "ok": bool(worst <= 2e-2 and mean <= 2e-3 and lse_err <= 1e-3)}
     return baseline, parity
+
+
+def cpu_baselines_of_the_other_legs(q, k, v, scale, gpu_out, gpu_lse, backward_heads=8):
+    """The fp32 oracle timed on the host cores for the backward (a sample of heads of the S=4096 workload) and the
+    decode (all 64 sequences of the B=64 workload): reported beside the GPU figures of `extra`, never a target."""
+    import torch
+    from dscuda_amd.harness import configs
+    from oracle import attention_oracle as oracle
+
+    results = {}
+    batch, seq, heads, dqk = q.shape
+    dv = v.shape[-1]
+    sample = list(range(0, heads, max(1, heads // backward_heads)))[:backward_heads]
+    dout = configs.mla_prefill_dout(batch, seq, heads, dv, seed=2)
+    sub = lambda t: t[:, :, sample]
+    saved_out, saved_lse = gpu_out[:, :, sample].cpu(), gpu_lse[:, sample].cpu()
+    begin = time.perf_counter()
+    oracle.attention_backward(sub(dout), saved_out, saved_lse, sub(q), sub(k), sub(v), scale)
+    seconds = time.perf_counter() - begin
+    flops = configs.backward_flops(batch, len(sample), seq, dqk, dv)
+    results["cpu_baseline_mla_backward_S4096"] = {
+        "value": flops / seconds / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{len(sample)} of {heads} heads, analytic fp32 backward of the oracle, {seconds:.1f} s"}
+
+    data = configs.mla_decode_inputs()
+    lengths = data["lengths"]
+    begin = time.perf_counter()
+    for b in range(lengths.numel()):
+        n = int(lengths[b])
+        oracle.mla_decode_unrounded(data["query"][b:b + 1], data["cache"][b:b + 1, :n], lengths[b:b + 1], data["scale"])
+    seconds = time.perf_counter() - begin
+    nbytes = configs.decode_bytes(int(lengths.sum()), lengths.numel(), data["query"].shape[2])
+    results["cpu_baseline_mla_decode_B64_H128"] = {
+        "value": nbytes / seconds / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"all {lengths.numel()} sequences, fp32 oracle one sequence at a time, {seconds:.1f} s"}
+    return results
 
 
 def main():
@@ -127,6 +176,9 @@ def main():
         extra = extra_workloads.measure(device, event_time_ms, dq, dk, dvv, scale, out, lse)
 
     baseline, parity = cpu_baseline_forward(q, k, v, scale, out, lse, args.cpu_heads)
+    if not args.no_extra:
+        extra.update(cpu_baselines_of_the_other_legs(q, k, v, scale, out, lse))
+    traffic, profiled_us = profiled_figures("mla_prefill_forward_S4096_H128", "attention_forward_pingpong_kernel")
 
     line = {
         "metric": "MLA fwd/bwd TFLOP/s (% bf16 MFMA peak); decode HBM GB/s, 1xMI355X",
@@ -145,8 +197,10 @@ def main():
         "config": {"workload": "MLA prefill forward, B=1 S=4096 H=128, d_qk=128+64, d_v=128, causal, "
                                "0.5*N(0,1) seed 1, RoPE theta=10000, scale 1/sqrt(192)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": FORWARD_TRAFFIC_BYTES,
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic,
+                     "traffic_source": "profiles/mla_prefill_forward_S4096_H128.md (rocprofv3 FETCH_SIZE + WRITE_SIZE)",
                      "kernel": "attention_forward_pingpong_kernel<192,128>", "kernel_ms": kernel_ms,
+                     "profiled_kernel_ms": None if profiled_us is None else profiled_us / 1000.0,
                      "flops_per_launch": flops},
         "cpu_baseline": baseline,
         "parity": parity,

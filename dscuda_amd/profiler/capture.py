@@ -1,0 +1,359 @@
+"""Two-pass rocprofv3 capture of the attention kernels and the table built from it.
+
+Counterpart of the reference's ``scripts/profile.sh`` (a timing pass and a
+counter pass per case around the standalone programs, ``profile.sh:143-185``)
+and ``scripts/extract_ncu.py`` (the per-kernel duration / DRAM traffic /
+throughput / registers / spills table, ``extract_ncu.py:193-326``), on rocprofv3:
+
+    python -m dscuda_amd.profiler.capture {metric|mla|flash_attention} [quick|full] [profile|extract]
+        [--out DIR] [--profiles DIR] [--only STEM] [--passes time,fetch,write,mfma[,waits]]
+
+``profile`` runs every case of the family once per pass, each pass a rocprofv3
+process of its own (a kernel trace, or one ``--pmc`` group that fits the
+hardware's counter blocks), raw CSV under ``--out``; then extracts.  ``extract``
+only rebuilds the tables from raw output that is already there.  The tables go
+to ``--profiles`` as one ``<stem>.md`` per case plus ``capture_<family>.md``.
+
+What a row holds, per kernel of a case:
+
+* launches and duration: mean over the second half of the launches of the
+  timing pass (the chip's clock needs some tens of back-to-back launches to
+  settle, so the first launches are reported separately);
+* HBM bytes read / written per launch: ``FETCH_SIZE`` / ``WRITE_SIZE`` (KiB per
+  dispatch) times the factor the same counter shows for a plain device copy
+  of known size (the ``copy`` case of the metric family);
+* matrix-pipe utilisation ``SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / XCDS *
+  SIMDS)`` and the shader clock ``GRBM_GUI_ACTIVE / XCDS / duration`` of the
+  counter pass, LDS bank-conflict cycles;
+* registers per lane (rocprofv3's VGPR_Count is in units of two registers of
+  the unified arch + accumulator file on this part, so it is doubled here),
+  scratch bytes per lane (spills) and the statically declared LDS bytes per
+  workgroup as the dispatch packets report them (dynamic LDS is not in them).
+"""
+
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+import os
+import shlex
+import subprocess
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parents[2]
+BUILD = ROOT / "build"
+CASE_SCRIPT = ROOT / "dscuda_amd" / "harness" / "profile_case.py"
+
+XCDS = 8
+SIMDS = 256 * 4
+COPY_KIB = float(1 << 20)   # the copy case moves 1 GiB each way
+
+PASSES = {
+    "time": ["--kernel-trace", "--stats"],
+    "fetch": ["--pmc", "FETCH_SIZE"],
+    "write": ["--pmc", "WRITE_SIZE"],
+    "mfma": ["--pmc", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES", "SQ_WAVE_CYCLES", "SQ_INSTS_LDS",
+             "SQ_LDS_BANK_CONFLICT", "SQ_INSTS_VALU", "GRBM_GUI_ACTIVE"],
+    "waits": ["--pmc", "SQ_WAIT_ANY", "SQ_WAIT_INST_ANY", "SQ_WAIT_INST_LDS", "SQ_ACTIVE_INST_ANY",
+              "SQ_ACTIVE_INST_VALU", "SQ_ACTIVE_INST_LDS", "SQ_WAVE_CYCLES", "SQ_INSTS_VMEM"],
+}
+DEFAULT_PASSES = ("time", "fetch", "write", "mfma")
+
+Case = collections.namedtuple("Case", "stem label command counter_command kernels")
+
+
+def _python_case(workload, steps, counter_steps, *extra):
+    base = [sys.executable, str(CASE_SCRIPT), workload, *map(str, extra)]
+    return base + ["--steps", str(steps)], base + ["--steps", str(counter_steps)]
+
+
+def copy_case():
+    """A plain device copy of 1 GiB: what FETCH_SIZE / WRITE_SIZE read for a known amount of traffic."""
+    command, counter_command = _python_case("copy", 12, 6)
+    return Case("copy_1GiB", "device copy of 1 GiB (FETCH_SIZE / WRITE_SIZE calibration)", command, counter_command,
+                ["copyBuffer"])
+
+
+def metric_cases(suite):
+    """The workloads of the headline metric (synthetic inputs drawn on the GPU) and the copy calibration."""
+    cases = []
+
+    def add(stem, label, workload, steps, counter_steps, kernels, *extra):
+        command, counter_command = _python_case(workload, steps, counter_steps, *extra)
+        cases.append(Case(stem, label, command, counter_command, kernels))
+
+    add("mla_prefill_forward_S4096_H128", "MLA prefill forward B=1 S=4096 H=128 192/128", "forward", 160, 60,
+        ["attention_forward"])
+    add("mla_prefill_backward_S4096_H128", "MLA prefill backward B=1 S=4096 H=128 192/128", "backward", 80, 30,
+        ["attention_backward", "attention_key_value", "attention_query"])
+    add("mla_decode_B64_H128", "absorbed MLA decode B=64 H=128 lengths U[1024,8192] seed 3", "decode", 300, 100,
+        ["mla_decode"])
+    add("flash_forward_S512_H8_D64", "flash forward B=1 H=8 S=512 D=64", "flash", 300, 100, ["attention_forward"])
+    if suite == "full":
+        add("mla_prefill_forward_S16384_H128", "MLA prefill forward B=1 S=16384 H=128 192/128", "forward", 16, 8,
+            ["attention_forward"], "--seq", 16384)
+        add("mla_prefill_backward_S16384_H128", "MLA prefill backward B=1 S=16384 H=128 192/128", "backward", 8, 4,
+            ["attention_backward", "attention_key_value", "attention_query"], "--seq", 16384)
+    return cases
+
+
+def mla_cases(suite):
+    """The reference's profile_mla cases (scripts/profile.sh:281-296) on the standalone programs."""
+    cases = []
+    for sequence in ((128,) if suite == "quick" else (128, 256, 512)):
+        command = [str(BUILD / "benchmark_mla"), "1", str(sequence), "8", "512", "64"]
+        cases.append(Case(f"mla_T{sequence}_forward_backward", f"B=1,T={sequence},H=8,D=512,R=64/custom/forward_backward",
+                          command, command, ["mla_absorbed"]))
+        command = [str(BUILD / "benchmark_mla_decode"), "2", str(sequence), "16", "512", "64", "8"]
+        cases.append(Case(f"mla_KV{sequence}_decode", f"B=2,KV={sequence},H=16,D=512,R=64/custom/decode", command, command,
+                          ["mla_decode"]))
+    return cases
+
+
+def flash_cases(suite):
+    """The reference's profile_flash_attention shapes (scripts/profile.sh:232-279), custom side."""
+    cases = []
+    shapes = [(2, 512, 8, 128)] if suite == "quick" else [(2, 512, 8, 128), (1, 2048, 8, 128), (1, 512, 8, 64)]
+    for batch, sequence, heads, dimension in shapes:
+        command = [str(BUILD / "benchmark_flash_attention"), *map(str, (batch, sequence, heads, dimension)), "forward"]
+        cases.append(Case(f"flash_B{batch}_T{sequence}_H{heads}_D{dimension}_forward",
+                          f"B={batch},T={sequence},H={heads},D={dimension}/custom/forward", command, command,
+                          ["attention_forward"]))
+    return cases
+
+
+FAMILIES = {"metric": metric_cases, "mla": mla_cases, "flash_attention": flash_cases}
+
+
+def rocprof_command(pass_name, directory, program):
+    return ["rocprofv3", *PASSES[pass_name], "--output-format", "csv", "-d", str(directory), "-o", "x", "--", *program]
+
+
+def run_pass(case, pass_name, out, limit):
+    directory = out / case.stem / pass_name
+    directory.mkdir(parents=True, exist_ok=True)
+    program = case.command if pass_name == "time" else case.counter_command
+    command = rocprof_command(pass_name, directory, program)
+    (directory / "command.txt").write_text(shlex.join(command) + "\n")
+    print(f"[capture] {case.stem} / {pass_name}", flush=True)
+    environment = dict(os.environ, TMPDIR="/tmp", PYTHONPATH=str(ROOT))
+    # a rocprofv3 that asks for more counters than a block holds hangs after its error line: hard limit
+    result = subprocess.run(["timeout", "-s", "KILL", str(limit), *command], cwd="/tmp", env=environment,
+                            capture_output=True, text=True)
+    (directory / "log.txt").write_text(result.stdout[-4000:] + "\n--- stderr ---\n" + result.stderr[-4000:])
+    if result.returncode != 0:
+        raise RuntimeError(f"{case.stem}/{pass_name}: rocprofv3 exited with {result.returncode}; see {directory / 'log.txt'}")
+
+
+# ---- extraction ---------------------------------------------------------------------------------------------
+
+def short_name(name: str) -> str:
+    name = name.replace("void ", "").replace("(anonymous namespace)::", "").replace("dscuda::", "")
+    cut = name.find("(")
+    return name if cut < 0 else name[:cut]
+
+
+def mean(values):
+    values = list(values)
+    return sum(values) / len(values) if values else float("nan")
+
+
+def settled(values):
+    """Mean of the second half (all of them when there are fewer than four)."""
+    values = list(values)
+    return mean(values[len(values) // 2:] if len(values) >= 4 else values)
+
+
+def read_trace(directory, wanted):
+    rows = collections.OrderedDict()
+    for path in sorted(directory.rglob("*_kernel_trace.csv")):
+        with open(path, newline="") as handle:
+            for row in csv.DictReader(handle):
+                name = short_name(row["Kernel_Name"])
+                if not any(text in name for text in wanted):
+                    continue
+                entry = rows.setdefault(name, {"durations": [], "vgpr": 0, "scratch": 0, "lds": 0})
+                entry["durations"].append((int(row["End_Timestamp"]) - int(row["Start_Timestamp"])) / 1e3)
+                entry["vgpr"] = 2 * int(row["VGPR_Count"]) + int(row["Accum_VGPR_Count"])
+                entry["scratch"] = int(row["Scratch_Size"])
+                entry["lds"] = int(row["LDS_Block_Size"])
+    return rows
+
+
+def read_counters(directory, wanted):
+    """kernel -> counter -> list of per-dispatch values; kernel -> list of dispatch durations (us)."""
+    table = collections.OrderedDict()
+    spans = {}
+    for path in sorted(directory.rglob("*_counter_collection.csv")):
+        with open(path, newline="") as handle:
+            seen = set()
+            for row in csv.DictReader(handle):
+                name = short_name(row["Kernel_Name"])
+                if not any(text in name for text in wanted):
+                    continue
+                table.setdefault(name, collections.OrderedDict()).setdefault(row["Counter_Name"], []).append(
+                    float(row["Counter_Value"]))
+                key = (name, row["Dispatch_Id"])
+                if key not in seen and row.get("Start_Timestamp") and row.get("End_Timestamp"):
+                    seen.add(key)
+                    spans.setdefault(name, []).append((int(row["End_Timestamp"]) - int(row["Start_Timestamp"])) / 1e3)
+    return table, spans
+
+
+def calibration(out):
+    """(fetch factor, write factor) from the copy case: bytes moved / bytes the counter reports."""
+    factors = []
+    for pass_name, counter in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
+        table, _ = read_counters(out / "copy_1GiB" / pass_name, ["copyBuffer"])
+        values = [settled(counters[counter]) for counters in table.values() if counter in counters]
+        values = [value for value in values if value > COPY_KIB / 8]   # the 1 GiB copy, not the fills around it
+        factors.append(COPY_KIB / mean(values) if values else float("nan"))
+    return tuple(factors)
+
+
+def extract_case(case, out, factors):
+    directory = out / case.stem
+    trace = read_trace(directory / "time", case.kernels)
+    fetch, _ = read_counters(directory / "fetch", case.kernels)
+    write, _ = read_counters(directory / "write", case.kernels)
+    mfma, mfma_spans = read_counters(directory / "mfma", case.kernels)
+    rows = []
+    for kernel, entry in trace.items():
+        durations = entry["durations"]
+        row = {"kernel": kernel, "launches": len(durations), "first_us": mean(durations[:5]), "time_us": settled(durations),
+               "vgpr": entry["vgpr"], "scratch": entry["scratch"], "lds": entry["lds"],
+               "read_mb": float("nan"), "write_mb": float("nan"), "mfma_pct": float("nan"), "clock_ghz": float("nan"),
+               "bank_conflict": float("nan"), "counter_us": float("nan")}
+        if kernel in fetch and "FETCH_SIZE" in fetch[kernel]:
+            row["read_mb"] = settled(fetch[kernel]["FETCH_SIZE"]) * factors[0] * 1024 / 1e6
+        if kernel in write and "WRITE_SIZE" in write[kernel]:
+            row["write_mb"] = settled(write[kernel]["WRITE_SIZE"]) * factors[1] * 1024 / 1e6
+        if kernel in mfma:
+            counters = mfma[kernel]
+            span = settled(mfma_spans.get(kernel, []))
+            row["counter_us"] = span
+            if "GRBM_GUI_ACTIVE" in counters:
+                cycles = settled(counters["GRBM_GUI_ACTIVE"]) / XCDS
+                row["clock_ghz"] = cycles / span / 1e3 if span == span else float("nan")
+                if "SQ_VALU_MFMA_BUSY_CYCLES" in counters:
+                    row["mfma_pct"] = 100.0 * settled(counters["SQ_VALU_MFMA_BUSY_CYCLES"]) / (cycles * SIMDS)
+            if "SQ_LDS_BANK_CONFLICT" in counters:
+                row["bank_conflict"] = settled(counters["SQ_LDS_BANK_CONFLICT"])
+        rows.append(row)
+    return rows
+
+
+COLUMNS = [("kernel", "kernel", "{}"), ("launches", "launches", "{:d}"), ("first_us", "first 5 us", "{:.1f}"),
+           ("time_us", "settled us", "{:.1f}"), ("read_mb", "HBM read MB", "{:.1f}"), ("write_mb", "HBM write MB", "{:.1f}"),
+           ("mfma_pct", "MFMA busy %", "{:.1f}"), ("clock_ghz", "clock GHz", "{:.2f}"),
+           ("counter_us", "us in counter pass", "{:.1f}"), ("bank_conflict", "LDS bank conflict cycles", "{:.0f}"),
+           ("vgpr", "registers/lane", "{:d}"), ("scratch", "scratch B/lane", "{:d}"),
+           ("lds", "static LDS B", "{:d}")]
+
+
+def cell(pattern, value):
+    if isinstance(value, float) and value != value:
+        return "-"
+    return pattern.format(value)
+
+
+def markdown_table(rows):
+    lines = ["| " + " | ".join(title for _, title, _ in COLUMNS) + " |", "|" + "---|" * len(COLUMNS)]
+    for row in rows:
+        lines.append("| " + " | ".join(cell(pattern, row[key]) for key, _, pattern in COLUMNS) + " |")
+    return lines
+
+
+def portable(command: str) -> str:
+    """The recorded command with the checkout's location taken out: paths relative to the repository root,
+    the interpreter as `python3`."""
+    words = []
+    for word in shlex.split(command):
+        for anchor in ("gpurun_out/", "dscuda_amd/", "build/"):
+            cut = word.find("/" + anchor)
+            if cut >= 0:
+                word = word[cut + 1:]
+                break
+        if word.rsplit("/", 1)[-1] in ("python", "python3") or word.rsplit("/", 1)[-1].startswith("python3."):
+            word = "python3"
+        words.append(word)
+    return shlex.join(words)
+
+
+def write_case(case, rows, out, profiles, factors):
+    lines = [f"# {case.label}", ""]
+    lines.append("Commands (one rocprofv3 process per pass; raw CSV is not kept in the repository):")
+    lines.append("")
+    for pass_name in PASSES:
+        recorded = out / case.stem / pass_name / "command.txt"
+        if recorded.exists():
+            lines.append(f"- {pass_name}: `{portable(recorded.read_text().strip())}`")
+    lines += ["", f"Counter calibration from the 1 GiB copy: FETCH_SIZE x {factors[0]:.3f}, WRITE_SIZE x {factors[1]:.3f}.",
+              "Durations are the mean of the second half of the launches of the timing pass.", ""]
+    lines += markdown_table(rows)
+    lines += ["", "Machine-readable (bytes per launch from the two traffic columns, microseconds from the settled column):", ""]
+    for row in rows:
+        total = (row["read_mb"] + row["write_mb"]) * 1e6
+        lines.append(f"    {row['kernel']} :: time_us = {row['time_us']:.3f} ; hbm_bytes = "
+                     f"{'nan' if total != total else format(total, '.0f')}")
+    (profiles / f"{case.stem}.md").write_text("\n".join(lines) + "\n")
+
+
+def write_overview(family, suite, cases, results, profiles):
+    lines = [f"# rocprofv3 capture: family `{family}`, suite `{suite}`", "",
+             "One row per kernel of each case; `python -m dscuda_amd.profiler.capture " + family + " " + suite +
+             "` reproduces it.  The per-case files carry the exact commands.", ""]
+    for case in cases:
+        rows = results[case.stem]
+        if not rows:
+            continue
+        lines += [f"## {case.label}", ""] + markdown_table(rows)
+        total = sum(row["time_us"] for row in rows)
+        read = sum(row["read_mb"] for row in rows)
+        wrote = sum(row["write_mb"] for row in rows)
+        lines += ["", f"total: {len(rows)} kernels, {total:.1f} us, HBM read {cell('{:.1f}', read)} MB, "
+                      f"written {cell('{:.1f}', wrote)} MB", ""]
+    (profiles / f"capture_{family}.md").write_text("\n".join(lines) + "\n")
+
+
+def main(argv=None):
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("family", choices=sorted(FAMILIES))
+    parser.add_argument("suite", nargs="?", default="quick", choices=("quick", "full"))
+    parser.add_argument("mode", nargs="?", default="profile", choices=("profile", "extract"))
+    parser.add_argument("--out", type=Path, default=ROOT / "gpurun_out" / "capture")
+    parser.add_argument("--profiles", type=Path, default=ROOT / "profiles")
+    parser.add_argument("--only", action="append", default=[], help="case stems to run (default: all)")
+    parser.add_argument("--passes", default=",".join(DEFAULT_PASSES))
+    parser.add_argument("--limit", type=int, default=240, help="seconds before a pass is killed")
+    args = parser.parse_args(argv)
+
+    passes = [name for name in args.passes.split(",") if name]
+    for name in passes:
+        if name not in PASSES:
+            parser.error(f"unknown pass {name}")
+    cases = [copy_case()] + FAMILIES[args.family](args.suite)
+    if args.only:
+        cases = [case for case in cases if case.stem in args.only or case.stem == "copy_1GiB"]
+    out = args.out.resolve()
+    if args.mode == "profile":
+        for case in cases:
+            for name in passes:
+                run_pass(case, name, out, args.limit)
+    factors = calibration(out) if (out / "copy_1GiB").exists() else (float("nan"), float("nan"))
+    args.profiles.mkdir(parents=True, exist_ok=True)
+    results = {}
+    for case in cases:
+        rows = extract_case(case, out, factors)
+        results[case.stem] = rows
+        if rows:
+            write_case(case, rows, out, args.profiles, factors)
+            for line in markdown_table(rows):
+                print(line)
+    write_overview(args.family, args.suite, cases, results, args.profiles)
+
+
+if __name__ == "__main__":
+    main()
