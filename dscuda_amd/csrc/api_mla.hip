@@ -109,8 +109,44 @@ void mla_decode_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __h
         throw std::invalid_argument(
             "MLA decode requires positive batch, head, page_size, pages_per_sequence and splits");
     }
-    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
-                        heads, page_size, pages_per_sequence, splits, scale, stream);
+    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, nullptr,
+                        batch_size, heads, page_size, pages_per_sequence, splits, scale, stream);
+}
+
+std::size_t mla_decode_plan_elements(int batch_size, int heads, int splits, int kv_rank) {
+    if (batch_size <= 0 || heads <= 0 || splits <= 0 || kv_rank != MLA_KV_RANK) {
+        return 0;
+    }
+    return dscuda::mla_decode_plan_elements(batch_size, heads, splits);
+}
+
+void mla_decode_plan_cuda(int* plan, const int* cache_lengths, int batch_size, int heads, int kv_rank, int splits,
+                          hipStream_t stream) {
+    check_shape(kv_rank, MLA_ROPE_SIZE);
+    if (batch_size <= 0 || heads <= 0 || splits <= 0) {
+        throw std::invalid_argument("MLA decode plan requires positive batch, head and split counts");
+    }
+    if (plan == nullptr || cache_lengths == nullptr) {
+        throw std::invalid_argument("MLA decode plan requires a plan buffer and the cache lengths");
+    }
+    mla_decode_plan_dispatch(plan, cache_lengths, batch_size, heads, splits, stream);
+}
+
+void mla_decode_forward_planned_cuda(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
+                                     const __hip_bfloat16* paged_kv_cache, const int* block_table,
+                                     const int* cache_lengths, float* workspace, int* plan, int batch_size, int heads,
+                                     int kv_rank, int rope_size, int page_size, int pages_per_sequence, int splits,
+                                     float scale, hipStream_t stream) {
+    check_shape(kv_rank, rope_size);
+    if (batch_size <= 0 || heads <= 0 || page_size <= 0 || pages_per_sequence <= 0 || splits <= 0) {
+        throw std::invalid_argument(
+            "MLA decode requires positive batch, head, page_size, pages_per_sequence and splits");
+    }
+    if (plan == nullptr) {
+        throw std::invalid_argument("MLA decode (planned) requires the plan written by mla_decode_plan_cuda");
+    }
+    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, plan,
+                        batch_size, heads, page_size, pages_per_sequence, splits, scale, stream);
 }
 
 void mla_decode_forward_static(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
@@ -130,8 +166,8 @@ void mla_decode_forward_static(__hip_bfloat16* output, float* logsumexp, const _
             " bytes; lower splits or call the variant that takes a caller workspace");
     }
     float* workspace = static_decode_scratch_of_current_device();
-    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, batch_size,
-                        heads, page_size, pages_per_sequence, splits, scale, stream);
+    mla_decode_dispatch(output, logsumexp, query, paged_kv_cache, block_table, cache_lengths, workspace, nullptr,
+                        batch_size, heads, page_size, pages_per_sequence, splits, scale, stream);
 }
 
 void mla_prefill_forward_cuda(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
@@ -223,6 +259,25 @@ extern "C" int dscuda_mla_decode(__hip_bfloat16* output, float* lse, const __hip
     return guarded([&] {
         dscuda::mla_decode_forward_cuda(output, lse, query, paged_cache, block_table, lengths, workspace, batch,
                                         heads, rank, rope, page_size, pages, splits, scale, stream);
+    });
+}
+
+extern "C" std::size_t dscuda_mla_decode_plan_elements(int batch, int heads, int splits, int rank) {
+    return dscuda::mla_decode_plan_elements(batch, heads, splits, rank);
+}
+
+extern "C" int dscuda_mla_decode_plan(int* plan, const int* lengths, int batch, int heads, int rank, int splits,
+                                      hipStream_t stream) {
+    return guarded([&] { dscuda::mla_decode_plan_cuda(plan, lengths, batch, heads, rank, splits, stream); });
+}
+
+extern "C" int dscuda_mla_decode_planned(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
+                                         const __hip_bfloat16* paged_cache, const int* block_table, const int* lengths,
+                                         float* workspace, int* plan, int batch, int heads, int rank, int rope,
+                                         int page_size, int pages, int splits, float scale, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_decode_forward_planned_cuda(output, lse, query, paged_cache, block_table, lengths, workspace, plan,
+                                                batch, heads, rank, rope, page_size, pages, splits, scale, stream);
     });
 }
 

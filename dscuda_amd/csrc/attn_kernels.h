@@ -46,10 +46,18 @@ void mla_absorbed_backward_dispatch(__hip_bfloat16* query_latent_gradient, __hip
                                     const __hip_bfloat16* key_rope, int batch_size, int sequence_length, int heads,
                                     float scale, hipStream_t stream);
 
-// mla_decode.hip -- absorbed single-token decode over a paged latent cache.
+// mla_decode.hip -- absorbed single-token decode over a paged latent cache.  `plan` is
+// the int table mla_decode_plan_dispatch writes for the same batch, heads and splits
+// (mla_decode_plan_elements ints), or nullptr: the call then builds its own inside the
+// workspace.
+std::size_t mla_decode_plan_elements(int batch_size, int heads, int splits);
+
+void mla_decode_plan_dispatch(int* plan, const int* cache_lengths, int batch_size, int heads, int splits,
+                              hipStream_t stream);
+
 void mla_decode_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query,
                          const __hip_bfloat16* paged_kv_cache, const int* block_table, const int* cache_lengths,
-                         float* workspace, int batch_size, int heads, int page_size, int pages_per_sequence,
-                         int splits, float scale, hipStream_t stream);
+                         float* workspace, int* plan, int batch_size, int heads, int page_size,
+                         int pages_per_sequence, int splits, float scale, hipStream_t stream);
 
 }  // namespace dscuda

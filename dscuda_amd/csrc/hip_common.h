@@ -29,6 +29,7 @@
 #include <sstream>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 
 namespace dscuda {
 
@@ -169,6 +170,16 @@ __device__ __forceinline__ void xcd_order(int linear, int outer, int inner, int&
     } else {
         outer_index = linear / inner;
         inner_index = linear % inner;
+    }
+}
+
+// f(std::integral_constant<int, BEGIN>) ... f(std::integral_constant<int, END - 1>), in order:
+// a loop whose index is a compile-time constant inside the body.
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void unrolled(F&& f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        unrolled<BEGIN + 1, END>(f);
     }
 }
 

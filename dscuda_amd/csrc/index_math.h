@@ -157,27 +157,27 @@ DSCUDA_HOST_DEVICE inline bool forward_item(int round, int member, int members, 
 }
 
 // ---- decode: tile loads -------------------------------------------------------
-// A [64][ROW_BYTES] tile of consecutive rows is fetched by four waves, wave w
-// filling rows 16w .. 16w+15 with 1 KB instructions: LDS slot 64*i + lane of the
-// wave's share (16 bytes each) holds chunk (slot % CHUNKS) ^ f(row) of local row
-// slot / CHUNKS.  With i a compile-time constant a wave instruction spans at most
-// two rows, so the row part of the offset is wave-uniform and the lane part costs
-// an add, an xor and a shift-add per candidate row.  Rows past `row_limit` (of
-// the tile) repeat that row.  f depends on bits 1..3 of the row only, which
-// 16*wave leaves alone.
-template <int ROW_BYTES>
+// A [4 * ROWS_PER_WAVE][ROW_BYTES] tile of consecutive rows is fetched by four waves,
+// wave w filling rows ROWS_PER_WAVE*w .. +ROWS_PER_WAVE-1 with 1 KB instructions: LDS
+// slot 64*i + lane of the wave's share (16 bytes each) holds chunk (slot % CHUNKS) ^
+// f(row) of local row slot / CHUNKS.  With i a compile-time constant a wave
+// instruction spans at most two rows, so the row part of the offset is wave-uniform
+// and the lane part costs an add, an xor and a shift-add per candidate row.  Rows
+// past `row_limit` (of the tile) repeat that row.  ROWS_PER_WAVE = 16 is the 64-key
+// tile, 8 the 32-key unit.
+template <int ROW_BYTES, int ROWS_PER_WAVE = 16>
 DSCUDA_HOST_DEVICE inline unsigned contiguous_load_offset(int wave, int i, int lane, int row_limit) {
     constexpr int CHUNKS = ROW_BYTES / 16;
-    const int first_row = (64 * i) / CHUNKS;                 // row of lane 0 (within the wave's 16 rows)
+    const int first_row = (64 * i) / CHUNKS;                 // row of lane 0 (within the wave's rows)
     const int boundary = CHUNKS * (first_row + 1) - 64 * i;  // first lane of the next row (may be >= 64)
-    const int tile_row_a = 16 * wave + first_row;
+    const int tile_row_a = ROWS_PER_WAVE * wave + first_row;
     const unsigned row_a = (unsigned)(tile_row_a < row_limit ? tile_row_a : row_limit) * ROW_BYTES;
-    unsigned offset = row_a + 16u * (unsigned)((lane + 64 * i - CHUNKS * first_row) ^ tile_swizzle<ROW_BYTES>(first_row));
+    unsigned offset = row_a + 16u * (unsigned)((lane + 64 * i - CHUNKS * first_row) ^ tile_swizzle<ROW_BYTES>(tile_row_a));
     if (boundary < 64) {
-        const int tile_row_b = 16 * wave + first_row + 1;
+        const int tile_row_b = tile_row_a + 1;
         const unsigned row_b = (unsigned)(tile_row_b < row_limit ? tile_row_b : row_limit) * ROW_BYTES;
         const unsigned other =
-            row_b + 16u * (unsigned)((lane + 64 * i - CHUNKS * (first_row + 1)) ^ tile_swizzle<ROW_BYTES>(first_row + 1));
+            row_b + 16u * (unsigned)((lane + 64 * i - CHUNKS * (first_row + 1)) ^ tile_swizzle<ROW_BYTES>(tile_row_b));
         offset = lane >= boundary ? other : offset;
     }
     return offset;
@@ -211,30 +211,59 @@ DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total_tiles, int workgroup
     last = (before + own - 1) / per;
 }
 
-// ---- decode: how a call uses the caller's workspace ---------------------------
-// The workspace holds batch * heads * splits * (rank + 2) floats.  It is used as
-// `slots` partial-result slots of heads * (rank + 2) floats (slot = workgroup +
-// sequence, so slots = workgroups + batch) followed by one flag word per launched
-// workgroup.  The number of workgroups is capped so that slots stays at least one
-// below batch * splits and the flags fit the slot left over; when not even two
-// workgroups fit under that cap (splits == 1, batch == 1 with splits == 2, a single
-// compute unit) no
-// sequence is cut: one workgroup per sequence, no slots, flags at the start.
+// ---- decode: the plan and how a call uses the caller's workspace ---------------
+// The plan is what a decode call needs to know about the lengths of its batch
+// before any workgroup starts: an int table
+//     [0] total tiles   [1] workgroups   [2] tiles per range   [3] 1 = sequences are not cut
+//     [4 .. 4+B]        inclusive prefix of tiles per sequence (B + 1 entries)
+//     [.. + W]          first sequence whose tiles reach past the start of each range
+//     [.. + G*B]        one flag per (head group, sequence): some part needs the rescaling pass
+// with G = head groups of 128 heads.  The flags are zero between calls.
+constexpr int PLAN_TOTAL = 0;
+constexpr int PLAN_WORKGROUPS = 1;
+constexpr int PLAN_PER_RANGE = 2;
+constexpr int PLAN_WHOLE = 3;
+constexpr int PLAN_HEADER = 4;
+
+DSCUDA_HOST_DEVICE inline long long plan_prefix_at() { return PLAN_HEADER; }
+DSCUDA_HOST_DEVICE inline long long plan_first_sequence_at(int batch) { return PLAN_HEADER + (long long)batch + 1; }
+DSCUDA_HOST_DEVICE inline long long plan_flags_at(int batch, int workgroups) {
+    return plan_first_sequence_at(batch) + workgroups;
+}
+DSCUDA_HOST_DEVICE inline long long plan_elements(int batch, int workgroups, int head_groups) {
+    return plan_flags_at(batch, workgroups) + (long long)head_groups * batch;
+}
+
+// The caller's workspace holds batch * heads * splits * (rank + 2) floats.  A
+// range that holds only part of a sequence leaves its unnormalised result there:
+// slot workgroup + sequence (slots = workgroups + batch), each slot one bf16 row of
+// `rank` values plus two floats (reference exponent, sum) per head, heads rounded up
+// to whole waves of 32.  A call without a caller-provided plan keeps its plan behind
+// the slots.  The number of workgroups is the largest (up to one per compute unit)
+// for which all of that fits; when fewer than two fit, no sequence is cut: one
+// workgroup per sequence, no slots.
 struct DecodeLayout {
     int workgroups;
     int whole_sequences;
+    int head_groups;
+    long long slot_floats;
     long long slots;
-    long long flag_offset;   // in floats from the start of the workspace
-    long long flag_words;
+    long long plan_offset;   // in floats from the start of the workspace
+    long long plan_ints;
 };
 
 DSCUDA_HOST_DEVICE inline DecodeLayout decode_layout(int batch, int heads, int splits, int compute_units,
                                                      int rows_per_group, int rank) {
     DecodeLayout layout;
-    const long long head_groups = (heads + rows_per_group - 1) / rows_per_group;
-    const long long by_workspace = (long long)batch * (splits - 1) - 1;
-    const long long cutting = by_workspace < compute_units ? by_workspace : compute_units;
-    layout.whole_sequences = cutting < 2 ? 1 : 0;
+    layout.head_groups = (heads + rows_per_group - 1) / rows_per_group;
+    const long long padded_rows = (long long)((heads + 31) / 32) * 32;
+    layout.slot_floats = padded_rows * (rank / 2 + 2);
+    const long long workspace = (long long)batch * heads * splits * (rank + 2);
+    // (W + batch) * slot_floats + plan_elements(batch, W, groups) <= workspace, W <= compute_units
+    const long long fixed = (long long)batch * layout.slot_floats + plan_elements(batch, 0, layout.head_groups);
+    long long cutting = workspace >= fixed ? (workspace - fixed) / (layout.slot_floats + 1) : 0;
+    if (cutting > compute_units) cutting = compute_units;
+    layout.whole_sequences = (splits <= 1 || cutting < 2) ? 1 : 0;
     if (layout.whole_sequences) {
         layout.workgroups = batch;
         layout.slots = 0;
@@ -242,8 +271,8 @@ DSCUDA_HOST_DEVICE inline DecodeLayout decode_layout(int batch, int heads, int s
         layout.workgroups = (int)cutting;
         layout.slots = (long long)layout.workgroups + batch;
     }
-    layout.flag_offset = layout.slots * heads * (rank + 2);
-    layout.flag_words = head_groups * layout.workgroups;
+    layout.plan_offset = layout.slots * layout.slot_floats;
+    layout.plan_ints = plan_elements(batch, layout.workgroups, layout.head_groups);
     return layout;
 }
 

@@ -36,18 +36,24 @@
 // Scheduling (decode)
 //   The tiles of all sequences form one list that is cut into equal ranges,
 //   one per workgroup (one workgroup per CU), so uneven lengths balance to
-//   within a tile.  A range may start or end inside a sequence; such a segment
-//   leaves (max, sum, unnormalised O) in the caller's workspace at slot
-//   workgroup + sequence -- unique because ranges and sequences both advance
-//   monotonically -- and a second kernel merges the slots of a sequence.
-//   Sequences that fall inside one range are finished in place.  Lengths live
-//   on the device; the cut is computed in-kernel from a block scan, so the
-//   call stays capturable.
+//   within a tile.  The cut is a small table (the plan) that a one-workgroup
+//   kernel derives from the lengths on the device, so the call stays
+//   capturable; a caller that decodes several layers over the same lengths
+//   builds it once and passes it in.  A range may start or end inside a
+//   sequence; such a segment leaves (exponent reference, sum, unnormalised O
+//   as bf16) in the caller's workspace at slot workgroup + sequence -- unique
+//   because ranges and sequences both advance monotonically -- and a second
+//   kernel, spread over the whole chip, merges the slots of a sequence.
+//   (Merging inside the first kernel, by the workgroup that delivers the last
+//   part of a sequence, was measured: the 64 mergers run alone at the end with
+//   one compute unit each, which cost 110 us against 6 for the second kernel.)
+//   Sequences that fall inside one range are finished in place.
 #include "attn_kernels.h"
 #include "hip_common.h"
 #include "index_math.h"
 
 #include <algorithm>
+#include <cstdint>
 #include <stdexcept>
 #include <string>
 
@@ -66,7 +72,6 @@ constexpr int STAGE_BYTES = BN * ROW_BYTES; // 73728
 constexpr int LOADS_PER_THREAD = BN * CHUNKS / THREADS;  // 18
 constexpr int KSTEPS = WIDTH / 16;          // 36
 constexpr int DBLOCKS = RANK / 32;          // 16
-constexpr int MAX_SEQUENCES = 3072;         // prefix table that fits beside the two stages
 constexpr int EPILOGUE_PITCH = 1024 + 16;   // bytes per staged output row
 
 typedef const __attribute__((address_space(1))) void* global_pointer;
@@ -438,37 +443,22 @@ __device__ __forceinline__ void store_final(const RowState& state, float inverse
     }
 }
 
-// Unnormalised fp32 rows -> partial_row(row) .. +512 floats, in two halves of 256 columns.
-template <typename RowPointer>
-__device__ __forceinline__ void store_partial(const RowState& state, unsigned char* wave_lds, int lane,
-                                              RowPointer partial_row) {
-    const int lq = lane % 32;
-    const int g = lane / 32;
+// A wave's unnormalised accumulators as bf16 in the registers' own order: 16-byte piece
+// j of a lane holds registers 8*(j%2) .. 8*(j%2)+7 of column block j/2, and a wave
+// instruction covers 1 KB of consecutive memory (32 KB per wave).  Nothing crosses
+// lanes; the merge kernel reads the pieces back with the same lane numbering.
+constexpr int PARTIAL_PIECES = 2 * DBLOCKS;
+constexpr int PARTIAL_WAVE_BYTES = PARTIAL_PIECES * 64 * 16;
+
+__device__ __forceinline__ void store_partial(const RowState& state, unsigned char* wave_block, int lane) {
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
+    for (int j = 0; j < PARTIAL_PIECES; ++j) {
+        const int d = j / 2;
+        const int base = 8 * (j % 2);
+        u32x4 packed;
 #pragma unroll
-        for (int dd = 0; dd < DBLOCKS / 2; ++dd) {
-            const int d = half * (DBLOCKS / 2) + dd;
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const f32x4 values = {state.o[d][4 * i4 + 0], state.o[d][4 * i4 + 1], state.o[d][4 * i4 + 2],
-                                      state.o[d][4 * i4 + 3]};
-                const int column = output_column(d, i4, g) - 256 * half;
-                *reinterpret_cast<f32x4*>(wave_lds + lq * EPILOGUE_PITCH + 4 * column) = values;
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll 4
-        for (int row = 0; row < 32; ++row) {
-            float* destination = partial_row(row);
-            if (destination != nullptr) {
-                const f32x4 values = *reinterpret_cast<const f32x4*>(wave_lds + row * EPILOGUE_PITCH + 16 * lane);
-                *reinterpret_cast<f32x4*>(destination + 256 * half + 4 * lane) = values;
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_wave_barrier();
+        for (int k = 0; k < 4; ++k) packed[k] = pack_bf16(state.o[d][base + 2 * k], state.o[d][base + 2 * k + 1]);
+        *reinterpret_cast<u32x4*>(wave_block + (j * 64 + lane) * 16) = packed;
     }
 }
 
@@ -526,15 +516,13 @@ __device__ __forceinline__ bool walk_tiles(RowState& state, const bf16x8 (&qf)[K
     reset(state);
     bool risk = false;
     const int last_token = tokens - 1;
-    // Drain the query loads here: a wait for them inside the loop would also
-    // wait for the tile prefetch that is kept in flight there.
-    wait_vector_memory<0>();
-    issue_tile(locate_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, last_token, wave, true), keys,
-               wave);
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         unsigned char* stage = lds + (tile & 1) * STAGE_BYTES;
-        wait_vector_memory<0>();   // this tile was requested while the previous one was consumed
-        workgroup_barrier();
+        // This tile was requested while the previous one was consumed (the first one by
+        // walk_rows, ahead of the query loads, which this wait drains as well: a wait
+        // for them further down would also wait for the prefetch kept in flight there).
+        wait_vector_memory<0>();
+        workgroup_barrier();   // everybody's share has landed, everybody has left the previous tile
         const int key0 = tile * BN;
         if (key0 + BN > tokens) {
             zero_tail_rows(stage, tokens - key0, tid);
@@ -546,8 +534,8 @@ __device__ __forceinline__ bool walk_tiles(RowState& state, const bf16x8 (&qf)[K
         if (!next_tile.contiguous) issue_tile(next_tile, keys, wave);
         process_tile<SAFE>(state, risk, qf, stage, key0, limit, wave_min_limit, tile == tile_begin, c, lane, next_tile,
                            wave);
-        workgroup_barrier();
     }
+    workgroup_barrier();   // the stages are free: the caller stages its results through them
     return risk;
 }
 
@@ -559,6 +547,9 @@ __device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_l
                                           const bf16_t* query_rope_row, bool valid, unsigned char* lds,
                                           const KeyStream& keys, int tile_begin, int tile_end, int tokens, int limit,
                                           float c, int tid) {
+    // the first tile goes on its way before the query rows: both latencies overlap
+    issue_tile(locate_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, tokens - 1,
+                           __builtin_amdgcn_readfirstlane(tid / 64), true), keys, __builtin_amdgcn_readfirstlane(tid / 64));
     bf16x8 qf[KSTEPS];
     load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
     const bool risk = walk_tiles<SAFE>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
@@ -570,26 +561,47 @@ __device__ __forceinline__ int tiles_of(int length) {
     return (max(length, 0) + BN - 1) / BN;
 }
 
-// Inclusive prefix of tiles per sequence into prefix[0..B]; returns the total.
-__device__ __forceinline__ int scan_tiles(int* prefix, int* scratch, const int* lengths, int batch_size, int tid) {
+// ----------------------------------------------------------------------------
+// decode
+// ----------------------------------------------------------------------------
+
+using index_math::PLAN_HEADER;
+using index_math::PLAN_PER_RANGE;
+using index_math::PLAN_TOTAL;
+using index_math::PLAN_WHOLE;
+using index_math::PLAN_WORKGROUPS;
+
+// One workgroup turns the lengths into the plan (index_math.h): the tile prefix, the
+// cut into `workgroups` equal ranges, the first sequence of each range, and cleared
+// flags.  Any batch size: the scan carries over chunks of THREADS lengths.
+__global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restrict__ plan,
+                                                                  const int* __restrict__ cache_lengths, int batch_size,
+                                                                  int workgroups, int whole_sequences,
+                                                                  int head_groups) {
+    __shared__ int wave_totals[THREADS / 64];
+    const int tid = threadIdx.x;
     const int lane = tid % 64;
     const int wave = tid / 64;
+    int* prefix = plan + index_math::plan_prefix_at();
+    int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
+    int* flags = plan + index_math::plan_flags_at(batch_size, workgroups);
+
     int carry = 0;
     if (tid == 0) prefix[0] = 0;
     for (int base = 0; base < batch_size; base += THREADS) {
         const int index = base + tid;
-        int value = index < batch_size ? tiles_of(lengths[index]) : 0;
+        int value = index < batch_size ? tiles_of(cache_lengths[index]) : 0;
 #pragma unroll
         for (int offset = 1; offset < 64; offset <<= 1) {
             const int other = __shfl_up(value, offset);
             if (lane >= offset) value += other;
         }
-        if (lane == 63) scratch[wave] = value;
+        if (lane == 63) wave_totals[wave] = value;
         __syncthreads();
         int before = 0, total = 0;
 #pragma unroll
         for (int w = 0; w < THREADS / 64; ++w) {
-            const int t = scratch[w];
+            const int t = wave_totals[w];
             if (w < wave) before += t;
             total += t;
         }
@@ -597,34 +609,51 @@ __device__ __forceinline__ int scan_tiles(int* prefix, int* scratch, const int* 
         carry += total;
         __syncthreads();
     }
-    return carry;
+    const int total = carry;
+    const int per = index_math::tiles_per_range(total, workgroups);
+    if (tid == 0) {
+        plan[PLAN_TOTAL] = total;
+        plan[PLAN_WORKGROUPS] = workgroups;
+        plan[PLAN_PER_RANGE] = per;
+        plan[PLAN_WHOLE] = whole_sequences;
+    }
+    for (int index = tid; index < head_groups * batch_size; index += THREADS) flags[index] = 0;
+    __syncthreads();   // the prefix written above is read back below
+    for (int w = tid; w < workgroups; w += THREADS) {
+        int sequence = w;
+        if (!whole_sequences) {
+            const int begin = index_math::range_begin_of(total, workgroups, w);
+            // first sequence whose tiles reach past `begin`
+            int low = 0, high = batch_size;
+            while (low < high) {
+                const int mid = (low + high) / 2;
+                if (prefix[mid + 1] <= begin) low = mid + 1; else high = mid;
+            }
+            sequence = low;
+        }
+        first_sequence[w] = sequence;
+    }
 }
 
-// ----------------------------------------------------------------------------
-// decode
-// ----------------------------------------------------------------------------
-
-struct DecodeSlots {
-    float* partial_output;   // [slots][H][512]
-    float* partial_stats;    // [slots][H][2]  (max in log2 units, sum)
-};
-
-// SAFE == false is the kernel that does the work.  A workgroup in which some
-// row outran the fixed softmax reference (see process_tile) raises its flag
-// word instead of trusting its results; the SAFE == true instantiation,
-// launched right after, repeats exactly the flagged workgroups with the
-// rescaling variant and returns at once everywhere else.  Two kernels rather
-// than two paths in one keep the register allocation of the hot loop free of
-// the slow path's pressure.
+// SAFE == false is the kernel that does the work.  A segment in which some row outran
+// the fixed softmax reference (see process_tile) raises its sequence's flag instead of
+// trusting its results; the SAFE == true instantiation, launched right after, repeats
+// every segment of the flagged sequences with the rescaling variant and returns at once
+// everywhere else.  Two kernels rather than two paths in one keep the register
+// allocation of the hot loop free of the slow path's pressure.  The flags are cleared
+// by whoever reads them last: the merge kernel, or this kernel's rescaling pass when
+// sequences are not cut (then nothing is merged).
+//
+// Workspace: slot workgroup + sequence holds, for a segment that is only part of its
+// sequence, the bf16 accumulators of every wave (store_partial order, 32 KB per wave,
+// waves numbered over all head groups) followed by (reference, sum) per head.
 template <bool SAFE>
 __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query,
     const bf16_t* __restrict__ paged_kv_cache, const int* __restrict__ block_table,
-    const int* __restrict__ cache_lengths, float* __restrict__ workspace, int batch_size, int heads, int page_size,
-    int pages_per_sequence, int workgroups, int whole_sequences, float scale) {
+    const int* __restrict__ cache_lengths, float* __restrict__ workspace, int* __restrict__ plan, int batch_size,
+    int heads, int page_size, int pages_per_sequence, long long slot_floats, int padded_rows, float scale) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    int* prefix = reinterpret_cast<int*>(lds + 2 * STAGE_BYTES);
-    int* scratch = prefix + MAX_SEQUENCES + 1;
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -632,60 +661,54 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     const int lq = lane % 32;
     const int g = lane / 32;
     const int workgroup = blockIdx.x;
-    const int head0 = blockIdx.y * ROWS;
+    const int head_group = blockIdx.y;
+    const int head0 = head_group * ROWS;
     const float c = uniform(scale * LOG2E);
 
-    // one flag word per workgroup, behind the partial-result slots (or at the start of
-    // the workspace when sequences are not cut and no slot is used)
-    const size_t slots = whole_sequences ? 0 : (size_t)workgroups + batch_size;
-    int* flag = reinterpret_cast<int*>(workspace + slots * heads * (RANK + 2)) + blockIdx.y * gridDim.x + workgroup;
-    if (SAFE && *flag == 0) return;
+    const int total = plan[PLAN_TOTAL];
+    const int workgroups = plan[PLAN_WORKGROUPS];
+    const bool whole_sequences = plan[PLAN_WHOLE] != 0;
+    const int* prefix = plan + index_math::plan_prefix_at();
+    const int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
+    int* flags = plan + index_math::plan_flags_at(batch_size, workgroups) + (size_t)head_group * batch_size;
 
-    const int total = scan_tiles(prefix, scratch, cache_lengths, batch_size, tid);
-    int range_begin, range_end, sequence;
+    int range_begin, range_end;
     if (whole_sequences) {
-        sequence = workgroup;
-        range_begin = prefix[sequence];
-        range_end = prefix[sequence + 1];
+        range_begin = prefix[workgroup];
+        range_end = prefix[workgroup + 1];
     } else {
         range_begin = index_math::range_begin_of(total, workgroups, workgroup);
         range_end = index_math::range_end_of(total, workgroups, range_begin);
-        // first sequence whose tiles reach past range_begin
-        int low = 0, high = batch_size;
-        while (low < high) {
-            const int mid = (low + high) / 2;
-            if (prefix[mid + 1] <= range_begin) low = mid + 1; else high = mid;
-        }
-        sequence = low;
     }
-    if (range_begin >= range_end) {
-        if (!SAFE && tid == 0) *flag = 0;
-        return;
-    }
-
-    float* partial_output = workspace;
-    float* partial_stats = workspace + slots * heads * RANK;
+    if (range_begin >= range_end) return;
+    int sequence = first_sequence[workgroup];
 
     const int head = head0 + 32 * wave + lq;
     const bool valid = head < heads;
     const bool wave_active = head0 + 32 * wave < heads;
+    const int row = valid ? head : 0;
     unsigned char* wave_lds = lds + wave * 32 * EPILOGUE_PITCH;
+    const size_t partial_wave_offset = (size_t)(head_group * (ROWS / 32) + wave) * PARTIAL_WAVE_BYTES;
+    const size_t stats_offset = (size_t)padded_rows * (RANK / 2);   // in floats, behind the bf16 rows of a slot
 
     RowState state;
-    bool any_risk = false;
     int position = range_begin;
     while (position < range_end) {
         const int sequence_begin = prefix[sequence];
         const int sequence_end = prefix[sequence + 1];
         const int segment_end = min(range_end, sequence_end);
-        const int tokens = cache_lengths[sequence];
-        const bool whole = position == sequence_begin && segment_end == sequence_end;
         if (segment_end <= position) {  // a sequence without tiles (length < 1) owns nothing
             ++sequence;
             continue;
         }
-
-        const bf16_t* query_row = query + ((size_t)sequence * heads + (valid ? head : 0)) * WIDTH;
+        if (SAFE && flags[sequence] == 0) {   // finished by the fast kernel
+            position = segment_end;
+            ++sequence;
+            continue;
+        }
+        const int tokens = cache_lengths[sequence];
+        const bool whole = position == sequence_begin && segment_end == sequence_end;
+        const bf16_t* query_row = query + ((size_t)sequence * heads + row) * WIDTH;
 
         KeyStream keys;
         keys.latent = paged_kv_cache;
@@ -694,101 +717,136 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.rope_stride = WIDTH;
         keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
         keys.page_size = page_size;
-        if (walk_rows<SAFE>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
-                            segment_end - sequence_begin, tokens, tokens, c, tid)) {
-            any_risk = true;
-        }
-
+        const bool risk = walk_rows<SAFE>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
+                                          segment_end - sequence_begin, tokens, tokens, c, tid);
         const float total_sum = half_wave_sum(state.row_sum);
-        if (wave_active) {
-            if (whole) {
-                const float inverse = 1.0f / total_sum;
+
+        if (!SAFE && risk) {
+            if (tid == 0) flags[sequence] = 1;   // several workgroups may say so: they all write the same value
+        } else if (whole) {
+            if (wave_active) {
                 if (valid && g == 0) {
                     logsumexp[(size_t)sequence * heads + head] = (state.reference + __builtin_amdgcn_logf(total_sum)) * LN2;
                 }
-                store_final(state, inverse, wave_lds, lane, [&](int row) -> bf16_t* {
-                    const int h = head0 + 32 * wave + row;
+                store_final(state, 1.0f / total_sum, wave_lds, lane, [&](int r) -> bf16_t* {
+                    const int h = head0 + 32 * wave + r;
                     return h < heads ? output + ((size_t)sequence * heads + h) * RANK : nullptr;
                 });
-            } else {
-                const size_t slot = (size_t)workgroup + sequence;
-                if (valid && g == 0) {
-                    float* stats = partial_stats + (slot * heads + head) * 2;
-                    stats[0] = state.reference;
-                    stats[1] = total_sum;
-                }
-                store_partial(state, wave_lds, lane, [&](int row) -> float* {
-                    const int h = head0 + 32 * wave + row;
-                    return h < heads ? partial_output + (slot * heads + h) * RANK : nullptr;
-                });
             }
+            if (SAFE && whole_sequences && tid == 0) flags[sequence] = 0;   // nobody else reads it (see above)
+        } else if (wave_active) {
+            float* slot = workspace + ((size_t)workgroup + sequence) * slot_floats;
+            if (valid && g == 0) {
+                slot[stats_offset + 2 * head] = state.reference;
+                slot[stats_offset + 2 * head + 1] = total_sum;
+            }
+            store_partial(state, reinterpret_cast<unsigned char*>(slot) + partial_wave_offset, lane);
         }
         __syncthreads();  // the staging region is about to be overwritten by the next segment's tiles
         position = segment_end;
         ++sequence;
     }
-    if (!SAFE && tid == 0) *flag = any_risk ? 1 : 0;
 }
 
-// Merge the partial results of every sequence that was cut by a range boundary.
-__global__ __launch_bounds__(128) void mla_decode_combine_kernel(
-    bf16_t* __restrict__ output, float* __restrict__ logsumexp, const int* __restrict__ cache_lengths,
-    const float* __restrict__ workspace, int batch_size, int heads, int workgroups) {
-    __shared__ int sums[2][2];
-    const int tid = threadIdx.x;
+// Merge the parts of every sequence that was cut by a range boundary.  One wave per
+// (sequence, wave of 32 heads, quarter of the 512 columns): it reads its share of every
+// part in the order the registers of the split kernel held it (same lane numbering),
+// so lane l ends up with head l % 32 and, per column block d, the columns
+// output_column(d, i4, l / 32) + 0..3; the results go through LDS to leave as 16-byte
+// pieces of output rows.
+constexpr int MERGE_QUARTERS = 4;
+constexpr int MERGE_PIECES = PARTIAL_PIECES / MERGE_QUARTERS;       // 8 pieces of 16 bytes per lane and part
+constexpr int MERGE_COLUMNS = RANK / MERGE_QUARTERS;                // 128
+constexpr int MERGE_PITCH = MERGE_COLUMNS * 2 + 16;                  // bytes per staged row
+
+__global__ __launch_bounds__(64) void mla_decode_merge_kernel(bf16_t* __restrict__ output, float* __restrict__ logsumexp,
+                                                              const float* __restrict__ workspace, int* __restrict__ plan,
+                                                              int batch_size, int heads, long long slot_floats,
+                                                              int padded_rows) {
+    __shared__ __attribute__((aligned(16))) unsigned char staging[32 * MERGE_PITCH];
+    const int lane = threadIdx.x;
+    const int lq = lane % 32;
+    const int g = lane / 32;
+    const int quarter = blockIdx.x % MERGE_QUARTERS;
+    const int wave_block = blockIdx.x / MERGE_QUARTERS;   // 32 heads, numbered over all head groups
     const int sequence = blockIdx.y;
-    const int head = blockIdx.x;
 
-    // tiles before this sequence and in total
-    int before = 0, total = 0;
-    for (int index = tid; index < batch_size; index += 128) {
-        const int t = tiles_of(cache_lengths[index]);
-        total += t;
-        if (index < sequence) before += t;
+    const int workgroups = plan[PLAN_WORKGROUPS];
+    const int per = plan[PLAN_PER_RANGE];
+    const int* prefix = plan + index_math::plan_prefix_at();
+    if (quarter == 0 && wave_block % (ROWS / 32) == 0 && lane == 0) {
+        // this sequence's flag of the head group has been read by everybody who needed it
+        plan[index_math::plan_flags_at(batch_size, workgroups) + (size_t)(wave_block / (ROWS / 32)) * batch_size + sequence] = 0;
     }
-#pragma unroll
-    for (int offset = 1; offset < 64; offset <<= 1) {
-        before += __shfl_xor(before, offset);
-        total += __shfl_xor(total, offset);
-    }
-    if (tid % 64 == 0) {
-        sums[tid / 64][0] = before;
-        sums[tid / 64][1] = total;
-    }
-    __syncthreads();
-    before = sums[0][0] + sums[1][0];
-    total = sums[0][1] + sums[1][1];
-    const int own = tiles_of(cache_lengths[sequence]);
-    if (own == 0) return;
-    int first, last;
-    index_math::ranges_of_sequence(total, workgroups, before, own, first, last);
-    if (first == last) return;  // finished in place by the split kernel
+    const int sequence_begin = prefix[sequence];
+    const int sequence_end = prefix[sequence + 1];
+    if (sequence_end <= sequence_begin) return;   // no tiles: nothing was computed for it
+    const int first = sequence_begin / per;
+    const int last = (sequence_end - 1) / per;
+    if (first == last) return;                    // finished in place by the split kernel
 
-    const size_t slots = (size_t)workgroups + batch_size;
-    const float* partial_output = workspace;
-    const float* partial_stats = workspace + slots * heads * RANK;
+    const int head = 32 * wave_block + lq;
+    const bool valid = head < heads;
+    const size_t stats_offset = (size_t)padded_rows * (RANK / 2);
+    const size_t pieces_offset = (size_t)wave_block * PARTIAL_WAVE_BYTES + (size_t)(quarter * MERGE_PIECES * 64 + lane) * 16;
 
     float reference = -INFINITY;
     for (int w = first; w <= last; ++w) {
-        reference = fmaxf(reference, partial_stats[(((size_t)w + sequence) * heads + head) * 2]);
+        const float* part = workspace + ((size_t)w + sequence) * slot_floats;
+        if (valid) reference = fmaxf(reference, part[stats_offset + 2 * head]);
     }
     float normaliser = 0.f;
-    f32x4 accumulator = {0.f, 0.f, 0.f, 0.f};
-    for (int w = first; w <= last; ++w) {
-        const size_t row = ((size_t)w + sequence) * heads + head;
-        const float weight = __builtin_amdgcn_exp2f(partial_stats[row * 2] - reference);
-        normaliser += weight * partial_stats[row * 2 + 1];
-        const f32x4 values = *reinterpret_cast<const f32x4*>(partial_output + row * RANK + 4 * tid);
-        accumulator += values * weight;
+    float sums[MERGE_PIECES][8];
+#pragma unroll
+    for (int j = 0; j < MERGE_PIECES; ++j) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sums[j][k] = 0.f;
     }
-    const float inverse = 1.0f / normaliser;
-    u32x2 packed;
-    packed.x = pack_bf16(accumulator[0] * inverse, accumulator[1] * inverse);
-    packed.y = pack_bf16(accumulator[2] * inverse, accumulator[3] * inverse);
-    const size_t out_row = (size_t)sequence * heads + head;
-    *reinterpret_cast<u32x2*>(output + out_row * RANK + 4 * tid) = packed;
-    if (tid == 0) {
-        logsumexp[out_row] = (reference + __builtin_amdgcn_logf(normaliser)) * LN2;
+    for (int w = first; w <= last; ++w) {
+        const float* part = workspace + ((size_t)w + sequence) * slot_floats;
+        float weight = 0.f;
+        if (valid) {
+            weight = __builtin_amdgcn_exp2f(part[stats_offset + 2 * head] - reference);
+            normaliser = fmaf(weight, part[stats_offset + 2 * head + 1], normaliser);
+        }
+        const unsigned char* pieces = reinterpret_cast<const unsigned char*>(part) + pieces_offset;
+#pragma unroll
+        for (int j = 0; j < MERGE_PIECES; ++j) {
+            const u32x4 bits = *reinterpret_cast<const u32x4*>(pieces + j * 1024);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                sums[j][2 * k] = fmaf(weight, __uint_as_float(bits[k] << 16), sums[j][2 * k]);
+                sums[j][2 * k + 1] = fmaf(weight, __uint_as_float(bits[k] & 0xffff0000u), sums[j][2 * k + 1]);
+            }
+        }
+    }
+    const float inverse = valid ? 1.0f / normaliser : 0.f;
+    // piece j of the quarter is registers 8*(j%2) .. +7 of column block d = 4*quarter + j/2: two runs of
+    // four columns, output_column(d, 2*(j%2), g) and output_column(d, 2*(j%2) + 1, g)
+#pragma unroll
+    for (int j = 0; j < MERGE_PIECES; ++j) {
+#pragma unroll
+        for (int run = 0; run < 2; ++run) {
+            u32x2 packed;
+            packed.x = pack_bf16(sums[j][4 * run] * inverse, sums[j][4 * run + 1] * inverse);
+            packed.y = pack_bf16(sums[j][4 * run + 2] * inverse, sums[j][4 * run + 3] * inverse);
+            const int column = output_column(j / 2, 2 * (j % 2) + run, g);   // within the quarter's 128 columns
+            *reinterpret_cast<u32x2*>(staging + lq * MERGE_PITCH + 2 * column) = packed;
+        }
+    }
+    __syncthreads();
+    // 32 rows x 256 bytes: 16 lanes per row, four rows per pass
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+        const int r = 4 * pass + lane / 16;
+        const int h = 32 * wave_block + r;
+        if (h < heads) {
+            const u32x4 bits = *reinterpret_cast<const u32x4*>(staging + r * MERGE_PITCH + 16 * (lane % 16));
+            *reinterpret_cast<u32x4*>(output + ((size_t)sequence * heads + h) * RANK + quarter * MERGE_COLUMNS + 8 * (lane % 16)) = bits;
+        }
+    }
+    if (quarter == 0 && valid && g == 0) {
+        logsumexp[(size_t)sequence * heads + head] = (reference + __builtin_amdgcn_logf(normaliser)) * LN2;
     }
 }
 
@@ -849,7 +907,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
     });
 }
 
-constexpr int LDS_BYTES = 2 * STAGE_BYTES + (MAX_SEQUENCES + 1 + 8) * 4;
+constexpr int LDS_BYTES = 2 * STAGE_BYTES;
 
 template <typename Kernel>
 void allow_large_lds(Kernel kernel) {
@@ -869,13 +927,25 @@ int compute_units() {
 
 }  // namespace
 
+std::size_t mla_decode_plan_elements(int batch_size, int heads, int splits) {
+    const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
+    return static_cast<std::size_t>(layout.plan_ints);
+}
+
+void mla_decode_plan_dispatch(int* plan, const int* cache_lengths, int batch_size, int heads, int splits,
+                              hipStream_t stream) {
+    const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
+    hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
+                       layout.workgroups, layout.whole_sequences, layout.head_groups);
+    HIP_CHECK(hipGetLastError());
+}
+
 void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, const bf16_t* paged_kv_cache,
-                         const int* block_table, const int* cache_lengths, float* workspace, int batch_size,
-                         int heads, int page_size, int pages_per_sequence, int splits, float scale,
+                         const int* block_table, const int* cache_lengths, float* workspace, int* plan,
+                         int batch_size, int heads, int page_size, int pages_per_sequence, int splits, float scale,
                          hipStream_t stream) {
-    if (batch_size > MAX_SEQUENCES) {
-        throw std::invalid_argument("MLA decode supports at most " + std::to_string(MAX_SEQUENCES) +
-                                    " sequences per call");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) {
+        throw std::invalid_argument("MLA decode requires a workspace aligned to 16 bytes");
     }
     static thread_local bool prepared = false;
     if (!prepared) {
@@ -885,21 +955,27 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
     }
     // How the caller's B*H*splits*(C+2) floats are used: index_math::decode_layout.
     const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
-    const int whole_sequences = layout.whole_sequences;
-    const int workgroups = layout.workgroups;
-    const int head_groups = (heads + ROWS - 1) / ROWS;
-    const dim3 grid(workgroups, head_groups);
+    if (plan == nullptr) {
+        // no plan from the caller: this call's own, behind the partial-result slots
+        plan = reinterpret_cast<int*>(workspace + layout.plan_offset);
+        hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
+                           layout.workgroups, layout.whole_sequences, layout.head_groups);
+        HIP_CHECK(hipGetLastError());
+    }
+    const int padded_rows = (heads + 31) / 32 * 32;
+    const dim3 grid(layout.workgroups, layout.head_groups);
     hipLaunchKernelGGL(mla_decode_split_kernel<false>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
-                       paged_kv_cache, block_table, cache_lengths, workspace, batch_size, heads, page_size,
-                       pages_per_sequence, workgroups, whole_sequences, scale);
+                       paged_kv_cache, block_table, cache_lengths, workspace, plan, batch_size, heads, page_size,
+                       pages_per_sequence, layout.slot_floats, padded_rows, scale);
     HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(mla_decode_split_kernel<true>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
-                       paged_kv_cache, block_table, cache_lengths, workspace, batch_size, heads, page_size,
-                       pages_per_sequence, workgroups, whole_sequences, scale);
+                       paged_kv_cache, block_table, cache_lengths, workspace, plan, batch_size, heads, page_size,
+                       pages_per_sequence, layout.slot_floats, padded_rows, scale);
     HIP_CHECK(hipGetLastError());
-    if (!whole_sequences) {
-        hipLaunchKernelGGL(mla_decode_combine_kernel, dim3(heads, batch_size), dim3(128), 0, stream, output,
-                           logsumexp, cache_lengths, workspace, batch_size, heads, workgroups);
+    if (!layout.whole_sequences) {
+        hipLaunchKernelGGL(mla_decode_merge_kernel, dim3(MERGE_QUARTERS * (padded_rows / 32), batch_size), dim3(64), 0,
+                           stream, output, logsumexp, workspace, plan, batch_size, heads, layout.slot_floats,
+                           padded_rows);
         HIP_CHECK(hipGetLastError());
     }
 }

@@ -32,6 +32,9 @@ class _Mla:
         self.forward = bind(lib, "dscuda_mla_forward", [P] * 6 + [I] * 5 + [F, P])
         self.backward = bind(lib, "dscuda_mla_backward", [P] * 11 + [I] * 5 + [F, P])
         self.decode = bind(lib, "dscuda_mla_decode", [P] * 7 + [I] * 7 + [F, P])
+        self.decode_plan_elements = bind(lib, "dscuda_mla_decode_plan_elements", [I] * 4, ctypes.c_size_t)
+        self.decode_plan = bind(lib, "dscuda_mla_decode_plan", [P] * 2 + [I] * 4 + [P])
+        self.decode_planned = bind(lib, "dscuda_mla_decode_planned", [P] * 8 + [I] * 7 + [F, P])
         self.decode_static = bind(lib, "dscuda_mla_decode_static", [P] * 6 + [I] * 7 + [F, P])
         self.workspace = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
         self.prefill_forward = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
@@ -173,5 +176,33 @@ def mla_decode_static(packed_query, paged_cache, block_table, lengths, scale, sp
     lib = mla_library()
     checked(lib.lib, "mla", lib.decode_static(
         *pointers((out, lse, packed_query, paged_cache, block_table, lengths)),
+        b, h, rank, width - rank, paged_cache.shape[1], block_table.shape[1], splits, scale, stream()))
+    return out, lse
+
+
+def mla_decode_plan(lengths, heads, splits=8, rank=512):
+    """dscuda_mla_decode_plan: the int table a batch of cache lengths needs, built once on the device for any
+    number of mla_decode_planned calls over the same lengths, head count and splits."""
+    _require_cuda(lengths)
+    lib = mla_library()
+    batch = lengths.numel()
+    plan = torch.empty(lib.decode_plan_elements(batch, heads, splits, rank), device=lengths.device, dtype=torch.int32)
+    checked(lib.lib, "mla", lib.decode_plan(plan.data_ptr(), lengths.data_ptr(), batch, heads, rank, splits, stream()))
+    return plan
+
+
+def mla_decode_planned(packed_query, paged_cache, block_table, lengths, plan, scale, splits=8, rank=512,
+                       workspace=None, out=None, lse=None):
+    """dscuda_mla_decode_planned: mla_decode with the plan of mla_decode_plan."""
+    _require_cuda(packed_query, paged_cache, block_table, lengths, plan)
+    b, _, h, width = packed_query.shape
+    device = packed_query.device
+    if workspace is None:
+        workspace = mla_decode_workspace(b, h, splits, rank, device)
+    out = torch.empty(b, 1, h, rank, device=device, dtype=torch.bfloat16) if out is None else out
+    lse = torch.empty(b, h, 1, device=device, dtype=torch.float32) if lse is None else lse
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.decode_planned(
+        *pointers((out, lse, packed_query, paged_cache, block_table, lengths, workspace, plan)),
         b, h, rank, width - rank, paged_cache.shape[1], block_table.shape[1], splits, scale, stream()))
     return out, lse

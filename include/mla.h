@@ -84,7 +84,8 @@ std::size_t mla_decode_workspace_elements(
 // [blocks,page,1,C+R] with block table [B,pages_per_sequence] and per-sequence
 // lengths (>= 1).  Replaces reference include/mla.h:63-81.  `splits` bounds
 // how finely a sequence may be partitioned (and with it the workspace); the
-// result does not depend on it.
+// result does not depend on it.  The workspace (mla_decode_workspace_elements
+// floats, 16-byte aligned) needs no initialisation.  Any batch size.
 void mla_decode_forward_cuda(
     __hip_bfloat16* output,
     float* logsumexp,
@@ -93,6 +94,55 @@ void mla_decode_forward_cuda(
     const int* block_table,
     const int* cache_lengths,
     float* workspace,
+    int batch_size,
+    int heads,
+    int kv_rank,
+    int rope_size,
+    int page_size,
+    int pages_per_sequence,
+    int splits,
+    float scale,
+    hipStream_t stream = nullptr);
+
+// ---- additive: a decode plan that outlives one call (no counterpart in the reference's
+// kernels; the pattern of FlashMLA's get_mla_metadata, reference/python/flashmla.py:41-63) --
+//
+// Every decode call first turns the cache lengths into a small table: the tile
+// prefix of the batch, its cut into one range per workgroup and the per-sequence
+// tickets the ranges merge by.  mla_decode_forward_cuda builds that table inside
+// its workspace on every call.  A caller that decodes several layers (or steps)
+// over the same lengths builds it once:
+//     plan = device buffer of mla_decode_plan_elements(B, H, splits, C) ints
+//     mla_decode_plan_cuda(plan, lengths, B, H, C, splits, stream)
+//     for each layer: mla_decode_forward_planned_cuda(..., workspace, plan, ...)
+// The plan depends on the lengths, B, H and splits (all must be the same in the
+// calls that use it) and on nothing else.  The calls keep per-sequence counters
+// inside the plan and return them to zero, so calls that share a plan must be
+// ordered (one stream, or events): two of them in flight at once race.
+std::size_t mla_decode_plan_elements(
+    int batch_size,
+    int heads,
+    int splits,
+    int kv_rank);
+
+void mla_decode_plan_cuda(
+    int* plan,
+    const int* cache_lengths,
+    int batch_size,
+    int heads,
+    int kv_rank,
+    int splits,
+    hipStream_t stream = nullptr);
+
+void mla_decode_forward_planned_cuda(
+    __hip_bfloat16* output,
+    float* logsumexp,
+    const __hip_bfloat16* query,
+    const __hip_bfloat16* paged_kv_cache,
+    const int* block_table,
+    const int* cache_lengths,
+    float* workspace,
+    int* plan,
     int batch_size,
     int heads,
     int kv_rank,
@@ -224,6 +274,19 @@ int dscuda_mla_decode(  // mla_bridge.cu:58-73
     __hip_bfloat16* output, float* lse,
     const __hip_bfloat16* query, const __hip_bfloat16* paged_cache,
     const int* block_table, const int* lengths, float* workspace,
+    int batch, int heads, int rank, int rope, int page_size, int pages, int splits,
+    float scale, hipStream_t stream);
+
+// additive: the reusable decode plan (see dscuda::mla_decode_plan_cuda above)
+std::size_t dscuda_mla_decode_plan_elements(int batch, int heads, int splits, int rank);
+
+int dscuda_mla_decode_plan(
+    int* plan, const int* lengths, int batch, int heads, int rank, int splits, hipStream_t stream);
+
+int dscuda_mla_decode_planned(
+    __hip_bfloat16* output, float* lse,
+    const __hip_bfloat16* query, const __hip_bfloat16* paged_cache,
+    const int* block_table, const int* lengths, float* workspace, int* plan,
     int batch, int heads, int rank, int rope, int page_size, int pages, int splits,
     float scale, hipStream_t stream);
 

@@ -229,27 +229,32 @@ void check_forward_items() {
     }
 }
 
-// ---- decode tile loads: the two-candidate-row form equals the general form for every wave, load, lane and limit
+// ---- decode tile loads: the two-candidate-row form equals the general form for every wave, load, lane and limit,
+// for the 64-key tile (16 rows per wave, 18 loads) and the 32-key unit (8 rows per wave, 9 loads)
+template <int ROWS_PER_WAVE>
 void check_decode_loads() {
-    constexpr int ROW_BYTES = 1152, CHUNKS = ROW_BYTES / 16, LOADS = 18;
-    for (int row_limit : {0, 1, 15, 16, 17, 31, 40, 62, 63, 64, 1000}) {
-        std::vector<int> fetched(64 * CHUNKS, 0);
+    constexpr int ROW_BYTES = 1152, CHUNKS = ROW_BYTES / 16, LOADS = ROWS_PER_WAVE * CHUNKS / 64, ROWS = 4 * ROWS_PER_WAVE;
+    for (int row_limit : {0, 1, 7, 8, 15, 16, 17, 31, 40, 62, 63, 64, 1000}) {
+        std::vector<int> fetched(ROWS * CHUNKS, 0);
         for (int wave = 0; wave < 4; ++wave) {
             for (int i = 0; i < LOADS; ++i) {
                 for (int lane = 0; lane < 64; ++lane) {
-                    const int slot = 64 * i + lane;                  // of the wave's 18 KB
+                    const int slot = 64 * i + lane;                  // of the wave's share
                     const int local_row = slot / CHUNKS, position = slot % CHUNKS;
-                    const int row = 16 * wave + local_row;
+                    const int row = ROWS_PER_WAVE * wave + local_row;
                     const int chunk = position ^ tile_swizzle<ROW_BYTES>(row);
                     const unsigned general = (unsigned)std::min(row, row_limit) * ROW_BYTES + 16u * chunk;
-                    const unsigned fast = contiguous_load_offset<ROW_BYTES>(wave, i, lane, row_limit);
-                    EXPECT(fast == general, "row_limit %d wave %d load %d lane %d: %u vs %u", row_limit, wave, i, lane, fast, general);
-                    if (row_limit >= 63) ++fetched[row * CHUNKS + chunk];
+                    const unsigned fast = contiguous_load_offset<ROW_BYTES, ROWS_PER_WAVE>(wave, i, lane, row_limit);
+                    EXPECT(fast == general, "rows/wave %d row_limit %d wave %d load %d lane %d: %u vs %u", ROWS_PER_WAVE, row_limit, wave, i,
+                           lane, fast, general);
+                    // nothing past the limit row is read
+                    EXPECT(fast < (unsigned)std::min(row_limit, ROWS - 1) * ROW_BYTES + ROW_BYTES, "row_limit %d offset %u", row_limit, fast);
+                    if (row_limit >= ROWS - 1) ++fetched[row * CHUNKS + chunk];
                 }
             }
         }
-        if (row_limit >= 63) {
-            for (int index = 0; index < 64 * CHUNKS; ++index) EXPECT(fetched[index] == 1, "chunk %d fetched %d times", index, fetched[index]);
+        if (row_limit >= ROWS - 1) {
+            for (int index = 0; index < ROWS * CHUNKS; ++index) EXPECT(fetched[index] == 1, "chunk %d fetched %d times", index, fetched[index]);
         }
     }
 }
@@ -293,33 +298,54 @@ void check_decode_ranges() {
     }
 }
 
-// ---- decode workspace: slots and flag words stay inside the batch * heads * splits * (rank + 2) floats the caller
-// provides, for every batch size, head count and split count
+// ---- decode workspace: partial-result slots and the call's own plan stay inside the batch * heads * splits *
+// (rank + 2) floats the caller provides, for every batch size, head count and split count; the plan's parts do not
+// overlap
 void check_decode_layout() {
     constexpr int RANK = 512, ROWS = 128;
     for (int compute_units : {1, 8, 256, 304}) {
         for (int batch = 1; batch <= 80; ++batch) {
-            for (int heads : {1, 2, 16, 127, 128, 129, 160, 256}) {
+            for (int heads : {1, 2, 16, 31, 32, 33, 127, 128, 129, 160, 256}) {
                 for (int splits = 1; splits <= 34; ++splits) {
                     const DecodeLayout layout = decode_layout(batch, heads, splits, compute_units, ROWS, RANK);
                     const long long workspace = (long long)batch * heads * splits * (RANK + 2);
+                    const int groups = (heads + ROWS - 1) / ROWS;
+                    EXPECT(layout.head_groups == groups, "B %d H %d: %d head groups", batch, heads, layout.head_groups);
                     EXPECT(layout.workgroups >= 1 && layout.workgroups <= std::max(batch, compute_units), "B %d H %d splits %d: %d workgroups",
                            batch, heads, splits, layout.workgroups);
-                    EXPECT(layout.flag_offset + layout.flag_words <= workspace, "B %d H %d splits %d CUs %d: flags end at %lld of %lld floats",
-                           batch, heads, splits, compute_units, layout.flag_offset + layout.flag_words, workspace);
+                    EXPECT(layout.plan_offset + layout.plan_ints <= workspace, "B %d H %d splits %d CUs %d: plan ends at %lld of %lld floats",
+                           batch, heads, splits, compute_units, layout.plan_offset + layout.plan_ints, workspace);
+                    EXPECT(layout.plan_ints == plan_elements(batch, layout.workgroups, groups), "B %d H %d splits %d", batch, heads, splits);
+                    // a slot holds 32 KB of bf16 accumulators per wave of 32 heads and two floats per head
+                    const long long waves = (heads + 31) / 32;
+                    EXPECT(layout.slot_floats * 4 == waves * 32768 + waves * 32 * 8, "H %d slot of %lld floats", heads, layout.slot_floats);
+                    EXPECT(layout.slot_floats * 4 % 16 == 0, "H %d: slots must keep 16-byte alignment", heads);
                     if (layout.whole_sequences) {
-                        EXPECT(layout.workgroups == batch && layout.slots == 0 && layout.flag_offset == 0, "B %d splits %d", batch, splits);
+                        EXPECT(layout.workgroups == batch && layout.slots == 0 && layout.plan_offset == 0, "B %d splits %d", batch, splits);
                     } else {
                         EXPECT(layout.workgroups >= 2 && layout.slots == layout.workgroups + batch, "B %d splits %d", batch, splits);
-                        EXPECT(layout.flag_offset == layout.slots * heads * (RANK + 2), "B %d splits %d", batch, splits);
+                        EXPECT(layout.plan_offset == layout.slots * layout.slot_floats, "B %d splits %d", batch, splits);
+                        // as many workgroups as fit: one more would not
+                        if (layout.workgroups < compute_units) {
+                            const long long more = (layout.slots + 1) * layout.slot_floats + plan_elements(batch, layout.workgroups + 1, groups);
+                            EXPECT(more > workspace, "B %d H %d splits %d: %d workgroups but %d would fit", batch, heads, splits,
+                                   layout.workgroups, layout.workgroups + 1);
+                        }
                     }
+                    // plan: header, prefix, first sequences, flags follow one another
+                    EXPECT(plan_prefix_at() == PLAN_HEADER && plan_first_sequence_at(batch) == PLAN_HEADER + batch + 1 &&
+                               plan_flags_at(batch, layout.workgroups) == plan_first_sequence_at(batch) + layout.workgroups &&
+                               plan_elements(batch, layout.workgroups, groups) == plan_flags_at(batch, layout.workgroups) + (long long)groups * batch,
+                           "plan parts B %d", batch);
                 }
             }
         }
     }
-    // the case that used to put its flag word one float past the end
-    const DecodeLayout single = decode_layout(1, 128, 2, 256, ROWS, RANK);
-    EXPECT(single.whole_sequences == 1 && single.flag_offset == 0, "B 1 splits 2 must not cut the sequence");
+    // the headline decode shape uses every compute unit
+    const DecodeLayout headline = decode_layout(64, 128, 8, 256, ROWS, RANK);
+    EXPECT(!headline.whole_sequences && headline.workgroups == 256, "B 64 H 128 splits 8: %d workgroups", headline.workgroups);
+    // splits = 1 never cuts
+    EXPECT(decode_layout(5, 128, 1, 256, ROWS, RANK).whole_sequences == 1, "splits 1 must not cut");
 }
 
 int main() {
@@ -338,7 +364,8 @@ int main() {
     check_fragment_reads<384>();
     check_ds_blocks();
     check_forward_items();
-    check_decode_loads();
+    check_decode_loads<16>();
+    check_decode_loads<8>();
     check_decode_ranges();
     check_decode_layout();
     if (failures) {

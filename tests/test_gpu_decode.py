@@ -94,9 +94,9 @@ def test_decode_many_heads(cuda):
 def test_decode_large_scores_take_the_rescaling_path(cuda, splits, tokens, lengths, hot):
     """Scores that outgrow the first tile's maximum by far more than the fast
     path's head room: late keys are aligned with the query, early ones are not.
-    In the second case 13 workgroups share the 44 tiles of the two sequences, four to
-    a range: the ranges that meet the hot keys after an ordinary first tile repeat
-    with the rescaling variant and rewrite partial results that are then merged."""
+    In the second case five workgroups share the 44 tiles of the two sequences, nine to
+    a range: the ranges that meet the hot keys after an ordinary first tile flag their
+    sequence, and the rescaling pass redoes every part of it and merges them again."""
     batch, heads = 2, 8
     g = torch.Generator().manual_seed(12)
     query = (torch.randn(batch, 1, heads, 576, generator=g)).bfloat16()
@@ -110,9 +110,97 @@ def test_decode_large_scores_take_the_rescaling_path(cuda, splits, tokens, lengt
     torch.cuda.synchronize()
     expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths, scale)
     assert expected_lse.max() > 500  # really is far outside the fast path's range
-    assert_close_bf16("O", out, expected, max_abs=6e-2, mean_abs=6e-3)  # values are O(4): bf16 spacing 3e-2
+    # outputs reach |O| ~ 15 here, where bf16 is spaced 0.06 apart: the reference harness's own relative bar
+    # (benchmarks/mla.py:103-105) instead of the absolute one
+    torch.testing.assert_close(out.cpu().float(), expected, atol=8e-3, rtol=8e-3)
+    assert_close_bf16("O", out, expected, max_abs=1.5e-1, mean_abs=6e-3)
     worst = ((lse.cpu() - expected_lse).abs() / expected_lse.abs().clamp_min(1)).max().item()
     assert worst <= 1e-5
+
+
+def test_decode_with_a_reused_plan_equals_the_plain_call(cuda):
+    """One plan, several calls (the layers of a model share the cache lengths): bit-equal to the call that
+    builds its own plan, also after a call over other data in between and with the workspace overwritten."""
+    data = configs.mla_decode_inputs(batch=9, heads=128, low=40, high=2600, seed=41)
+    on_gpu = [data[k].to(cuda) for k in ("query", "paged", "table", "lengths")]
+    announce("mla_decode planned", dict(lengths=data["lengths"].tolist()))
+    for splits in (8, 1):
+        expected, expected_lse = ops.mla_decode(*on_gpu, data["scale"], splits=splits)
+        plan = ops.mla_decode_plan(on_gpu[3], 128, splits)
+        workspace = ops.mla_decode_workspace(9, 128, splits, 512, cuda)
+        other_query = (on_gpu[0].float() * -0.5).bfloat16()
+        for layer in range(3):
+            workspace.fill_(float("nan"))
+            query = on_gpu[0] if layer != 1 else other_query
+            out, lse = ops.mla_decode_planned(query, on_gpu[1], on_gpu[2], on_gpu[3], plan, data["scale"], splits=splits,
+                                              workspace=workspace)
+            torch.cuda.synchronize()
+            if layer != 1:
+                assert torch.equal(out, expected) and torch.equal(lse, expected_lse)
+    oracle_out, oracle_lse = oracle.mla_decode_unrounded(data["query"], data["cache"], data["lengths"], data["scale"])
+    assert_close_bf16("O", expected, oracle_out)
+    assert_close_lse("LSE", expected_lse, oracle_lse)
+
+
+def test_decode_plan_after_a_rescaled_call_is_clean(cuda):
+    """A call that needed the rescaling pass leaves the plan's tickets and flags at zero: the next call over the
+    same plan with ordinary data gives the ordinary result."""
+    batch, tokens, heads = 2, 1500, 8
+    g = torch.Generator().manual_seed(43)
+    query = torch.randn(batch, 1, heads, 576, generator=g).bfloat16()
+    cache = (torch.randn(batch, tokens, 576, generator=g) * 0.05).bfloat16()
+    hot = cache.clone()
+    hot[:, 1000:1100] = (query[:, 0, :1].float() * 4.0).bfloat16()
+    lengths = torch.tensor([1500, 1250], dtype=torch.int32)
+    paged, table = configs.pack_cache(cache, 64)
+    hot_paged, _ = configs.pack_cache(hot, 64)
+    plan = ops.mla_decode_plan(lengths.to(cuda), heads, 8)
+    announce("mla_decode plan reuse after rescaling")
+    ops.mla_decode_planned(query.to(cuda), hot_paged.to(cuda), table.to(cuda), lengths.to(cuda), plan, 1.0, splits=8)
+    out, lse = ops.mla_decode_planned(query.to(cuda), paged.to(cuda), table.to(cuda), lengths.to(cuda), plan, 1.0, splits=8)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths, 1.0)
+    assert_close_bf16("O", out, expected)
+    assert_close_lse("LSE", lse, expected_lse)
+
+
+def test_decode_repeated_calls_never_see_stale_parts(cuda):
+    """Parts of a sequence pass from workgroup to workgroup through the workspace inside one launch.  Sixty calls
+    that alternate between two data sets over one workspace must each reproduce their own first result bit for
+    bit: a part or a statistic left over from the other data set would show."""
+    first = configs.mla_decode_inputs(batch=24, heads=128, low=300, high=5000, seed=51)
+    second = configs.mla_decode_inputs(batch=24, heads=128, low=300, high=5000, seed=52)
+    pages = max(first["table"].shape[1], second["table"].shape[1])
+    workspace = ops.mla_decode_workspace(24, 128, 8, 512, cuda)
+    sets = []
+    for data in (first, second):
+        table = torch.zeros(24, pages, dtype=torch.int32)
+        table[:, :data["table"].shape[1]] = data["table"]
+        sets.append([data["query"].to(cuda), data["paged"].to(cuda), table.to(cuda), data["lengths"].to(cuda)])
+    announce("mla_decode repeated calls")
+    expected = []
+    for tensors, data in zip(sets, (first, second)):
+        out, lse = ops.mla_decode(*tensors, data["scale"], splits=8, workspace=workspace)
+        torch.cuda.synchronize()
+        oracle_out, oracle_lse = oracle.mla_decode_unrounded(data["query"], data["cache"], data["lengths"], data["scale"])
+        assert_close_bf16("O", out, oracle_out)
+        assert_close_lse("LSE", lse, oracle_lse)
+        expected.append((out.clone(), lse.clone()))
+    results = []
+    for call in range(60):
+        which = call % 2
+        out, lse = ops.mla_decode(*sets[which], first["scale"], splits=8, workspace=workspace)
+        results.append((which, out, lse))
+    torch.cuda.synchronize()
+    for call, (which, out, lse) in enumerate(results):
+        assert torch.equal(out, expected[which][0]) and torch.equal(lse, expected[which][1]), f"call {call}"
+
+
+def test_decode_large_batch(cuda):
+    """More sequences than any table a workgroup could hold in LDS: the plan lives in memory."""
+    batch, tokens, heads = 3500, 70, 4
+    lengths = [1 + (7 * b) % tokens for b in range(batch)]
+    _decode_case(cuda, batch, tokens, heads, lengths, splits=2, seed=44)
 
 
 def test_decode_closed_form_constant_fill(cuda):
