@@ -557,6 +557,334 @@ __device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_l
     return __syncthreads_or(risk) != 0;
 }
 
+// ----------------------------------------------------------------------------
+// The decode walk of the fast path (SAFE == false): 32-key units, one matrix stream
+// ----------------------------------------------------------------------------
+//
+// With one wave per SIMD nothing hides the vector arithmetic of the softmax unless the
+// wave's own instruction stream does: the tile loop above computes scores, then
+// probabilities, then the output update, and the matrix pipeline idles through the
+// middle third.  Here the key stream is consumed in units of 32 keys and the work of
+// consecutive units is overlapped by hand:
+//
+//     step u:   S(u+1) = K(u+1) Q^T   36 MFMAs, with the softmax of S(u) -> P(u)
+//                                     (exp2, sums, bf16 packing) and the requests for
+//                                     unit u+3 issued between them
+//               O^T  += V(u)^T P(u)   32 MFMAs
+//
+// one stream of 68 MFMAs per unit, each fed by one LDS fragment read through a small
+// register ring that runs a few MFMAs ahead.  The scores of two units are live at a
+// time (one being accumulated, one being turned into probabilities), so the steps
+// alternate between two register sets.
+//
+// Units sit in a ring of four LDS slots (the same 144 KB as the two tile stages).
+// Unit u+3 is requested during step u into the slot that unit u-1 left at the end of
+// step u-1; unit u+1, requested two steps earlier, must have landed when step u
+// starts: the wave waits for all but its youngest nine loads (its share of unit
+// u+2) and the workgroup meets at one barrier per step.  Rows of a unit past the end
+// of the sequence repeat the last valid row and their scores are masked, so nothing
+// has to be cleared.
+
+constexpr int UNIT = 32;
+constexpr int UNIT_BYTES = UNIT * ROW_BYTES;              // 36 KB
+constexpr int UNIT_SLOTS = 4;
+constexpr int UNIT_LOADS = UNIT * CHUNKS / THREADS;       // 9 wave instructions of 1 KB per wave and unit
+constexpr int STREAM_RING = 6;                            // fragments read ahead of the MFMA that takes them
+static_assert(UNIT_SLOTS * UNIT_BYTES == 2 * STAGE_BYTES, "the unit ring occupies the two tile stages");
+static_assert(UNIT_LOADS * THREADS == UNIT * CHUNKS, "unit loads must divide evenly");
+
+struct UnitSource {
+    const bf16_t* base;      // first row of the unit (contiguous form only)
+    unsigned lds_base;       // LDS byte offset of this wave's 9 KB of the unit's slot
+    int key0;
+    int row_limit;           // rows above it repeat it (>= 0: the unit holds a visible token)
+    bool contiguous;         // the unit is one run of rows: no paging, or pages that hold whole units
+    bool enabled;
+};
+
+// The decode cache is packed (576-wide rows), so only paging decides the form.
+__device__ __forceinline__ UnitSource locate_unit(unsigned char* lds, const KeyStream& keys, int unit, int last_token,
+                                                  int wave, bool enabled) {
+    UnitSource source;
+    const bool paged = keys.block_table != nullptr;
+    source.contiguous = !paged || (keys.page_size % UNIT == 0);
+    source.enabled = enabled;
+    source.key0 = unit * UNIT;
+    source.row_limit = last_token - source.key0;
+    source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(lds) + (unit % UNIT_SLOTS) * UNIT_BYTES +
+                                                     wave * (UNIT_LOADS * 1024));
+    source.base = keys.latent;
+    if (enabled && source.contiguous) {
+        long long physical = source.key0;
+        if (paged) {
+            const int page = keys.block_table[source.key0 / keys.page_size];
+            physical = (long long)page * keys.page_size + source.key0 % keys.page_size;
+        }
+        source.base = keys.latent + physical * WIDTH;
+    }
+    return source;
+}
+
+// Load number i (0..8) of a contiguous unit; i is a constant after unrolling.
+__device__ __forceinline__ void issue_unit_load(const UnitSource& source, int wave, int i, int lane) {
+    direct_load_16_offset(source.base, index_math::contiguous_load_offset<ROW_BYTES, UNIT / 4>(wave, i, lane, source.row_limit),
+                          source.lds_base + i * 1024);
+}
+
+// All nine loads of a unit at once: the first units of a walk, and every unit of the
+// general form (per-lane page lookup).
+__device__ __forceinline__ void issue_unit(const UnitSource& source, const KeyStream& keys, int wave) {
+    if (!source.enabled) return;
+    const int lane = fresh_lane_id();
+    if (source.contiguous) {
+#pragma unroll
+        for (int i = 0; i < UNIT_LOADS; ++i) issue_unit_load(source, wave, i, lane);
+        return;
+    }
+#pragma unroll 1
+    for (int i = 0; i < UNIT_LOADS; ++i) {
+        const int slot = 64 * i + lane;
+        const int row = (UNIT / 4) * wave + slot / CHUNKS;
+        const int chunk = (slot % CHUNKS) ^ swizzle_of_row(row);
+        const int token = source.key0 + min(row, source.row_limit);
+        const int page = keys.block_table[token / keys.page_size];
+        const long long physical = (long long)page * keys.page_size + token % keys.page_size;
+        direct_load_16(keys.latent + physical * WIDTH + 8 * chunk, source.lds_base + i * 1024);
+    }
+}
+
+// Per-lane byte offsets of the fragment reads inside a unit (rows 0..31 of 1152 bytes).
+// K operand: row lane%32, 16-byte chunk 2*ks + g at position (2*ks + g) ^ f(row); the XOR
+// only mixes the low three bits, so four offsets plus (ks/4)*128 reach every k-step.
+// V^T operand through transposing reads: in a block of 16 lanes, lane s points at row
+// 4*g + s/4 (+8 for the second read), columns 4*(s%4)..+3 of the 16-column group
+// 16*(block%2); bit 2 of f moves a row's data by one 64-byte column block, which two
+// offsets per read (even / odd column block) turn back into immediates.
+struct UnitReads {
+    unsigned k[4];
+    unsigned v_first[2];
+    unsigned v_second[2];
+
+    __device__ __forceinline__ void init(int lane) {
+        const int lq = lane % 32;
+        const int g = lane / 32;
+        const int swz = swizzle_of_row(lq);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) k[j] = lq * ROW_BYTES + ((2 * j + g) ^ swz) * 16;
+        const int s16 = lane % 16;
+        const int block = lane / 16;
+        const int row1 = 4 * g + s16 / 4;
+        const int f1 = swizzle_of_row(row1);
+        const int chunk_low = (2 * (block % 2) + (s16 % 4) / 2) ^ (f1 & 3);
+        const int flip = 64 * ((row1 >> 1) & 1);
+        const int lane1 = row1 * ROW_BYTES + chunk_low * 16 + 8 * (s16 & 1);
+        const int lane2 = (row1 + 8) * ROW_BYTES + (chunk_low ^ 1) * 16 + 8 * (s16 & 1);
+        v_first[0] = lane1 + flip;
+        v_first[1] = lane1 - flip;
+        v_second[0] = lane2 + flip;
+        v_second[1] = lane2 - flip;
+    }
+};
+
+typedef short unit_s16x4 __attribute__((ext_vector_type(4)));
+typedef short unit_s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) unit_s16x4* unit_tr_pointer;
+
+template <int KS>
+__device__ __forceinline__ bf16x8 unit_key_fragment(const unsigned char* unit, const UnitReads& reads) {
+    return *reinterpret_cast<const bf16x8*>(unit + reads.k[KS % 4] + (KS / 4) * 128);
+}
+
+// 16-key step N (0, 1) of the unit, column block D (0..15)
+template <int N, int D>
+__device__ __forceinline__ bf16x8 unit_value_fragment(const unsigned char* unit, const UnitReads& reads) {
+    constexpr int CONSTANT = N * 16 * ROW_BYTES + D * 64;
+    const unit_s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((unit_tr_pointer)(unit + reads.v_first[D % 2] + CONSTANT));
+    const unit_s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((unit_tr_pointer)(unit + reads.v_second[D % 2] + CONSTANT));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// Scores of the unit at `unit` into `scores`, nothing overlapped (the first unit of a walk).
+__device__ __forceinline__ void unit_scores(f32x16& scores, const bf16x8 (&qf)[KSTEPS], const unsigned char* unit,
+                                            const UnitReads& reads) {
+    bf16x8 ring[STREAM_RING];
+    unrolled<0, STREAM_RING>([&](auto tag) { ring[decltype(tag)::value] = unit_key_fragment<decltype(tag)::value>(unit, reads); });
+    unrolled<0, KSTEPS>([&](auto tag) {
+        constexpr int I = decltype(tag)::value;
+        if constexpr (I == 0) {
+            score_mfma_first(scores, ring[0], qf[0]);
+        } else {
+            score_mfma(scores, ring[I % STREAM_RING], qf[I]);
+        }
+        if constexpr (I + STREAM_RING < KSTEPS) ring[I % STREAM_RING] = unit_key_fragment<I + STREAM_RING>(unit, reads);
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+__device__ __forceinline__ void mask_unit_scores(f32x16& scores, int key0, int tokens, int g) {
+    if (key0 + UNIT > tokens) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int k = key0 + 8 * (i / 4) + 4 * g + (i % 4);
+            if (k >= tokens) scores[i] = -INFINITY;
+        }
+    }
+}
+
+// One step of the stream: the probabilities of the unit at `current` (its scores are in
+// `scores`), the scores of the unit at `next` into `next_scores` if HAS_NEXT, the output
+// update with `current`, and the requests for `request`.
+template <bool HAS_NEXT>
+__device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& scores, f32x16& next_scores,
+                                          const bf16x8 (&qf)[KSTEPS], const UnitReads& reads,
+                                          const unsigned char* current, const unsigned char* next, int key0, int tokens,
+                                          float c, const UnitSource& request, const KeyStream& keys, int wave) {
+    constexpr int SCORE_MFMAS = HAS_NEXT ? KSTEPS : 0;
+    constexpr int COUNT = SCORE_MFMAS + 2 * DBLOCKS;
+    const int lane = fresh_lane_id();
+
+    // fragment I of the stream: the K fragments of the next unit, then the V fragments of this one
+    auto fragment = [&](auto tag) -> bf16x8 {
+        constexpr int I = decltype(tag)::value;
+        if constexpr (I < SCORE_MFMAS) {
+            return unit_key_fragment<I>(next, reads);
+        } else {
+            return unit_value_fragment<(I - SCORE_MFMAS) / DBLOCKS, (I - SCORE_MFMAS) % DBLOCKS>(current, reads);
+        }
+    };
+    bf16x8 ring[STREAM_RING];
+    unrolled<0, STREAM_RING>([&](auto tag) { ring[decltype(tag)::value] = fragment(tag); });
+
+    // The scores were left by hand-issued MFMAs: spend the wait states a vector-ALU reader needs.
+    score_mfma_drain(scores);
+    mask_unit_scores(scores, key0, tokens, lane / 32);
+
+    float unit_max;
+    u32x4 probabilities[2];
+    const float offset = state.reference;
+    // The softmax in 33 pieces of one to three instructions, spread over the score MFMAs.  Plain
+    // arithmetic has no place of its own in the instruction order (the compiler would gather all of
+    // it next to its last use, behind the score MFMAs); passing a piece's inputs and results through
+    // empty volatile asm statements ties it to the spot between the two hand-issued MFMAs around it.
+    auto here = [](float& value) { asm volatile("" : "+v"(value)); };
+    float exponentials[16];
+    auto softmax_piece = [&](auto tag) {
+        constexpr int I = decltype(tag)::value;
+        if constexpr (I < 8) {
+            float first = scores[2 * I];
+            here(first);
+            unit_max = I == 0 ? fmaxf(first, scores[1]) : fmaxf(unit_max, fmaxf(first, scores[2 * I + 1]));
+            here(unit_max);
+        } else if constexpr (I == 8) {
+            unit_max = half_wave_max(unit_max) * c;
+            risk = risk || (unit_max - offset > FAST_LIMIT);
+        } else if constexpr (I < 25) {
+            constexpr int E = I - 9;
+            float score = scores[E];
+            here(score);
+            float p = __builtin_amdgcn_exp2f(fmaf(score, c, -offset));
+            here(p);
+            state.row_sum += p;
+            exponentials[E] = p;
+        } else if constexpr (I < 33) {
+            constexpr int K = I - 25;
+            float low = exponentials[2 * K];
+            here(low);
+            float packed = __uint_as_float(pack_bf16(low, exponentials[2 * K + 1]));
+            here(packed);
+            probabilities[K / 4][K % 4] = __float_as_uint(packed);
+        }
+    };
+    if constexpr (!HAS_NEXT) {
+        unrolled<0, 33>(softmax_piece);   // the last unit: no score products to hide it behind
+    }
+    if (request.enabled && !request.contiguous) issue_unit(request, keys, wave);
+
+    unrolled<0, COUNT>([&](auto tag) {
+        constexpr int I = decltype(tag)::value;
+        if constexpr (I < SCORE_MFMAS) {
+            if constexpr (I == 0) {
+                score_mfma_first(next_scores, ring[0], qf[0]);
+            } else {
+                score_mfma(next_scores, ring[I % STREAM_RING], qf[I]);
+            }
+        } else {
+            constexpr int J = I - SCORE_MFMAS;
+            state.o[J % DBLOCKS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                ring[I % STREAM_RING], __builtin_bit_cast(bf16x8, probabilities[J / DBLOCKS]), state.o[J % DBLOCKS], 0, 0, 0);
+        }
+        if constexpr (I + STREAM_RING < COUNT) ring[I % STREAM_RING] = fragment(std::integral_constant<int, I + STREAM_RING>{});
+        if constexpr (HAS_NEXT && I < 33) softmax_piece(tag);
+        if constexpr (HAS_NEXT && I % 4 == 0 && I / 4 < UNIT_LOADS) {
+            if (request.enabled && request.contiguous) issue_unit_load(request, wave, I / 4, lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+// Walk tiles [tile_begin, tile_end) of one sequence of the decode cache for the 128 heads of
+// this workgroup with the unit stream, from cleared accumulators.  Every lane's row sees all
+// `tokens` keys.  Returns whether any row of the workgroup came too close to the limit of the
+// fixed softmax reference (workgroup-uniform): the caller then discards the result.
+__device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_row, bool valid, unsigned char* lds,
+                                           const KeyStream& keys, int tile_begin, int tile_end, int tokens, float c,
+                                           int tid) {
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int last_token = tokens - 1;
+    const int unit_begin = (BN / UNIT) * tile_begin;
+    const int unit_end = min((BN / UNIT) * tile_end, (tokens + UNIT - 1) / UNIT);   // > unit_begin
+
+    // The first three units go on their way around the query rows: all latencies overlap.
+    issue_unit(locate_unit(lds, keys, unit_begin, last_token, wave, true), keys, wave);
+    issue_unit(locate_unit(lds, keys, unit_begin + 1, last_token, wave, unit_begin + 1 < unit_end), keys, wave);
+    bf16x8 qf[KSTEPS];
+    load_query(qf, query_row, query_row + RANK, valid, (tid % 64) / 32);
+    issue_unit(locate_unit(lds, keys, unit_begin + 2, last_token, wave, unit_begin + 2 < unit_end), keys, wave);
+    reset(state);
+    bool risk = false;
+    UnitReads reads;
+    reads.init(fresh_lane_id());
+    auto slot_of = [&](int unit) { return lds + (unit % UNIT_SLOTS) * UNIT_BYTES; };
+
+    wait_vector_memory<0>();
+    workgroup_barrier();
+    // scores of the first unit, and the reference every exponential of this walk is taken against
+    f32x16 scores_a, scores_b;
+    unit_scores(scores_a, qf, slot_of(unit_begin), reads);
+    {
+        score_mfma_drain(scores_a);
+        mask_unit_scores(scores_a, unit_begin * UNIT, tokens, fresh_lane_id() / 32);
+        float first_max = scores_a[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) first_max = fmaxf(first_max, scores_a[i]);
+        state.reference = half_wave_max(first_max) * c + FAST_HEADROOM;
+    }
+
+    auto synchronise = [&](int at) {
+        // unit at + 1 (requested during step at - 2, or before the loop) has landed; only this wave's share of
+        // unit at + 2, requested later, may still be in flight
+        if (at + 2 < unit_end) {
+            wait_vector_memory<UNIT_LOADS>();
+        } else {
+            wait_vector_memory<0>();
+        }
+        workgroup_barrier();   // ... and everybody's share; every wave has left step at - 1
+    };
+    int unit = unit_begin;
+    for (; unit + 1 < unit_end; ++unit) {
+        synchronise(unit);
+        unit_step<true>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
+                        locate_unit(lds, keys, unit + 3, last_token, wave, unit + 3 < unit_end), keys, wave);
+        // the next unit's scores take the place of this unit's (sixteen moves against a stream of 68 MFMAs)
+        score_mfma_drain(scores_b);
+        scores_a = scores_b;
+    }
+    unit_step<false>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c,
+                     locate_unit(lds, keys, unit, last_token, wave, false), keys, wave);
+    workgroup_barrier();   // the slots are free: the caller stages its results through them
+    return __syncthreads_or(risk) != 0;
+}
+
 __device__ __forceinline__ int tiles_of(int length) {
     return (max(length, 0) + BN - 1) / BN;
 }
@@ -717,8 +1045,14 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.rope_stride = WIDTH;
         keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
         keys.page_size = page_size;
-        const bool risk = walk_rows<SAFE>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
-                                          segment_end - sequence_begin, tokens, tokens, c, tid);
+        bool risk;
+        if constexpr (SAFE) {
+            risk = walk_rows<true>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
+                                   segment_end - sequence_begin, tokens, tokens, c, tid);
+        } else {
+            risk = walk_units(state, query_row, valid, lds, keys, position - sequence_begin, segment_end - sequence_begin,
+                              tokens, c, tid);
+        }
         const float total_sum = half_wave_sum(state.row_sum);
 
         if (!SAFE && risk) {
