@@ -178,21 +178,48 @@ __device__ __forceinline__ void issue_tile(const TileSource& source, const KeySt
 // Score-chain MFMAs with the accumulator held in ordinary vector registers.
 // The compiler's own MFMAs take accumulator-file destinations in a kernel this
 // large, and that file is fully occupied by the output accumulators.  Issued
-// as asm, the hazard bookkeeping is done here: the first MFMA starts from the
-// inline constant 0 (no producer to wait for), dependent MFMAs accumulating
-// into the very registers they read are interlocked by hardware, and
-// score_mfma_drain spends the wait states a vector-ALU reader of the result
-// needs after the last 8-pass MFMA before the value is handed back.
+// as asm, the hazard bookkeeping is done here.  The first MFMA of a chain starts
+// from the inline constant 0 (its destination may not share registers with its
+// operands); a dependent MFMA that accumulates into the registers it reads is
+// interlocked by hardware; the last MFMA of a chain carries, inside the same
+// asm statement, the wait states a vector-ALU reader of the result needs after
+// an 8-pass MFMA.
+//
+// What the hardware does not interlock is a vector-ALU access to the
+// accumulator between two MFMAs of a chain, and to the compiler the accumulator
+// is an ordinary value after every statement: nothing in the language stops it
+// from moving the value to other registers right there (it has done so, to
+// place the tail of a chain where a later copy wanted it -- the moves read a
+// result the matrix pipeline had not written yet).  Two things keep that from
+// happening unnoticed: the code below never copies a chain's accumulator in
+// C++ (move_scores is asm as well), and tests/test_decode_isa.py reads the
+// generated ISA of every kernel in this file and fails if any instruction
+// other than the chain's own MFMAs touches an accumulator's registers before
+// the wait states have passed.
 __device__ __forceinline__ void score_mfma_first(f32x16& accumulator, const bf16x8& a, const bf16x8& b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(accumulator) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(accumulator) : "v"(a), "v"(b));
 }
 
 __device__ __forceinline__ void score_mfma(f32x16& accumulator, const bf16x8& a, const bf16x8& b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(accumulator) : "v"(a), "v"(b));
 }
 
-__device__ __forceinline__ void score_mfma_drain(f32x16& accumulator) {
-    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(accumulator));
+__device__ __forceinline__ void score_mfma_last(f32x16& accumulator, const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(accumulator) : "v"(a), "v"(b));
+}
+
+// target = source, as one opaque statement: the compiler can neither fold it into the
+// chain that produced `source` nor start it early.
+__device__ __forceinline__ void move_scores(f32x16& target, const f32x16& source) {
+    typedef unsigned long long u64x8 __attribute__((ext_vector_type(8)));
+    const u64x8 in = __builtin_bit_cast(u64x8, source);
+    unsigned long long o0, o1, o2, o3, o4, o5, o6, o7;
+    asm volatile("v_mov_b64 %0, %8\n\tv_mov_b64 %1, %9\n\tv_mov_b64 %2, %10\n\tv_mov_b64 %3, %11\n\t"
+                 "v_mov_b64 %4, %12\n\tv_mov_b64 %5, %13\n\tv_mov_b64 %6, %14\n\tv_mov_b64 %7, %15"
+                 : "=&v"(o0), "=&v"(o1), "=&v"(o2), "=&v"(o3), "=&v"(o4), "=&v"(o5), "=&v"(o6), "=&v"(o7)
+                 : "v"(in[0]), "v"(in[1]), "v"(in[2]), "v"(in[3]), "v"(in[4]), "v"(in[5]), "v"(in[6]), "v"(in[7]));
+    const u64x8 out = {o0, o1, o2, o3, o4, o5, o6, o7};
+    target = __builtin_bit_cast(f32x16, out);
 }
 
 struct RowState {
@@ -301,6 +328,8 @@ __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const 
                     f32x16& chain = (ks % 2 == 0) ? s_acc : s_odd;
                     if (ks < 2) {
                         score_mfma_first(chain, current[j], qf[ks]);
+                    } else if (ks >= KSTEPS - 2) {
+                        score_mfma_last(chain, current[j], qf[ks]);
                     } else {
                         score_mfma(chain, current[j], qf[ks]);
                     }
@@ -311,8 +340,6 @@ __device__ __forceinline__ void process_tile(RowState& state, bool& risk, const 
 #pragma unroll
                 for (int j = 0; j < WIDTH_K; ++j) current[j] = next[j];
             }
-            score_mfma_drain(s_acc);
-            score_mfma_drain(s_odd);
 #pragma unroll
             for (int i = 0; i < 16; ++i) s_acc[i] += s_odd[i];
         }
@@ -568,9 +595,8 @@ __device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_l
 // consecutive units is overlapped by hand:
 //
 //     step u:   S(u+1) = K(u+1) Q^T   36 MFMAs, with the softmax of S(u) -> P(u)
-//                                     (exp2, sums, bf16 packing) and the requests for
-//                                     unit u+3 issued between them
-//               O^T  += V(u)^T P(u)   32 MFMAs
+//                                     (exp2, sums, bf16 packing) issued between them
+//               O^T  += V(u)^T P(u)   32 MFMAs, with the requests for unit u+3 between them
 //
 // one stream of 68 MFMAs per unit, each fed by one LDS fragment read through a small
 // register ring that runs a few MFMAs ahead.  The scores of two units are live at a
@@ -713,6 +739,8 @@ __device__ __forceinline__ void unit_scores(f32x16& scores, const bf16x8 (&qf)[K
         constexpr int I = decltype(tag)::value;
         if constexpr (I == 0) {
             score_mfma_first(scores, ring[0], qf[0]);
+        } else if constexpr (I == KSTEPS - 1) {
+            score_mfma_last(scores, ring[I % STREAM_RING], qf[I]);
         } else {
             score_mfma(scores, ring[I % STREAM_RING], qf[I]);
         }
@@ -755,8 +783,6 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
     bf16x8 ring[STREAM_RING];
     unrolled<0, STREAM_RING>([&](auto tag) { ring[decltype(tag)::value] = fragment(tag); });
 
-    // The scores were left by hand-issued MFMAs: spend the wait states a vector-ALU reader needs.
-    score_mfma_drain(scores);
     mask_unit_scores(scores, key0, tokens, lane / 32);
 
     float unit_max;
@@ -782,9 +808,12 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
             constexpr int E = I - 9;
             float score = scores[E];
             here(score);
-            float p = __builtin_amdgcn_exp2f(fmaf(score, c, -offset));
-            here(p);
+            const float p = __builtin_amdgcn_exp2f(fmaf(score, c, -offset));
             state.row_sum += p;
+            // The sum is what gets tied down, never the exponential itself: an asm statement that
+            // takes the result of v_exp hides from the compiler that its next reader follows a
+            // transcendental, and the wait state that pairing needs would go missing.
+            here(state.row_sum);
             exponentials[E] = p;
         } else if constexpr (I < 33) {
             constexpr int K = I - 25;
@@ -805,6 +834,8 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
         if constexpr (I < SCORE_MFMAS) {
             if constexpr (I == 0) {
                 score_mfma_first(next_scores, ring[0], qf[0]);
+            } else if constexpr (I == KSTEPS - 1) {
+                score_mfma_last(next_scores, ring[I % STREAM_RING], qf[I]);   // its wait states pass while it executes
             } else {
                 score_mfma(next_scores, ring[I % STREAM_RING], qf[I]);
             }
@@ -815,8 +846,9 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
         }
         if constexpr (I + STREAM_RING < COUNT) ring[I % STREAM_RING] = fragment(std::integral_constant<int, I + STREAM_RING>{});
         if constexpr (HAS_NEXT && I < 33) softmax_piece(tag);
-        if constexpr (HAS_NEXT && I % 4 == 0 && I / 4 < UNIT_LOADS) {
-            if (request.enabled && request.contiguous) issue_unit_load(request, wave, I / 4, lane);
+        // the requests go between the output MFMAs, which leave more issue slots free than the score MFMAs
+        if constexpr (HAS_NEXT && I >= SCORE_MFMAS && (I - SCORE_MFMAS) % 3 == 1 && (I - SCORE_MFMAS) / 3 < UNIT_LOADS) {
+            if (request.enabled && request.contiguous) issue_unit_load(request, wave, (I - SCORE_MFMAS) / 3, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
     });
@@ -852,7 +884,6 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
     f32x16 scores_a, scores_b;
     unit_scores(scores_a, qf, slot_of(unit_begin), reads);
     {
-        score_mfma_drain(scores_a);
         mask_unit_scores(scores_a, unit_begin * UNIT, tokens, fresh_lane_id() / 32);
         float first_max = scores_a[0];
 #pragma unroll
@@ -875,9 +906,8 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
         synchronise(unit);
         unit_step<true>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
                         locate_unit(lds, keys, unit + 3, last_token, wave, unit + 3 < unit_end), keys, wave);
-        // the next unit's scores take the place of this unit's (sixteen moves against a stream of 68 MFMAs)
-        score_mfma_drain(scores_b);
-        scores_a = scores_b;
+        // the next unit's scores take the place of this unit's (eight moves against a stream of 68 MFMAs)
+        move_scores(scores_a, scores_b);
     }
     unit_step<false>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c,
                      locate_unit(lds, keys, unit, last_token, wave, false), keys, wave);
