@@ -625,46 +625,108 @@ struct UnitSource {
     int key0;
     int row_limit;           // rows above it repeat it (>= 0: the unit holds a visible token)
     bool contiguous;         // the unit is one run of rows: no paging, or pages that hold whole units
+    bool full;               // all 32 rows are visible tokens: the per-lane offsets are the same for every such unit
     bool enabled;
 };
 
-// The decode cache is packed (576-wide rows), so only paging decides the form.
-__device__ __forceinline__ UnitSource locate_unit(unsigned char* lds, const KeyStream& keys, int unit, int last_token,
-                                                  int wave, bool enabled) {
-    UnitSource source;
-    const bool paged = keys.block_table != nullptr;
-    source.contiguous = !paged || (keys.page_size % UNIT == 0);
-    source.enabled = enabled;
-    source.key0 = unit * UNIT;
-    source.row_limit = last_token - source.key0;
-    source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(lds) + (unit % UNIT_SLOTS) * UNIT_BYTES +
-                                                     wave * (UNIT_LOADS * 1024));
-    source.base = keys.latent;
-    if (enabled && source.contiguous) {
-        long long physical = source.key0;
-        if (paged) {
-            const int page = keys.block_table[source.key0 / keys.page_size];
-            physical = (long long)page * keys.page_size + source.key0 % keys.page_size;
-        }
-        source.base = keys.latent + physical * WIDTH;
+// Hands out the sources of consecutive units of one sequence.  The decode cache is packed
+// (576-wide rows), so only paging decides the form.  When pages hold whole units, the ids of
+// 64 consecutive pages of the sequence sit in one register (lane l: page first_page + l) and a
+// unit finds its page with one lane read: a scalar load per unit would have its wait drain the
+// LDS queue as well, in the middle of the fragment stream.
+struct UnitCursor {
+    int unit;                // the unit handed out next
+    int page;                // its page (index into the sequence's block table) ...
+    int within;              // ... and its place inside that page, in units
+    int units_per_page;
+    int first_page;          // page whose id lane 0 of `ids` holds
+    int last_page;           // last page of the sequence with a visible token: no entry past it is read
+    int ids;
+    bool paged;
+    bool contiguous;
+
+    // Waits for the ids on the spot (the empty asm statement is their first use): a wait left to the
+    // first lane read would sit on the path of every step and wait for the unit requests as well.
+    __device__ __forceinline__ void load_ids(const KeyStream& keys, int from) {
+        first_page = from;
+        ids = keys.block_table[min(from + fresh_lane_id(), last_page)];
+        asm volatile("" : "+v"(ids));
     }
-    return source;
-}
+
+    __device__ __forceinline__ void init(const KeyStream& keys, int first_unit, int last_token) {
+        paged = keys.block_table != nullptr;
+        contiguous = !paged || (keys.page_size % UNIT == 0);
+        unit = __builtin_amdgcn_readfirstlane(first_unit);
+        page = within = units_per_page = first_page = last_page = ids = 0;
+        if (paged && contiguous) {
+            units_per_page = __builtin_amdgcn_readfirstlane(keys.page_size / UNIT);
+            page = __builtin_amdgcn_readfirstlane(first_unit / units_per_page);
+            within = __builtin_amdgcn_readfirstlane(first_unit - page * units_per_page);
+            last_page = __builtin_amdgcn_readfirstlane(last_token / keys.page_size);
+            load_ids(keys, page);
+        }
+    }
+
+    __device__ __forceinline__ UnitSource next(unsigned char* lds, const KeyStream& keys, int last_token, int wave,
+                                               int unit_end) {
+        UnitSource source;
+        source.contiguous = contiguous;
+        source.enabled = unit < unit_end;
+        source.key0 = unit * UNIT;
+        source.row_limit = last_token - source.key0;
+        source.full = source.row_limit >= UNIT - 1;
+        source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(lds) + ((unsigned)unit % UNIT_SLOTS) * UNIT_BYTES +
+                                                         wave * (UNIT_LOADS * 1024));
+        source.base = keys.latent;
+        if (source.enabled && contiguous) {
+            long long physical = source.key0;
+            if (paged) {
+                // enabled: the unit holds a visible token, so page <= last_page
+                if (page - first_page >= 64) load_ids(keys, page);
+                const int id = __builtin_amdgcn_readlane(ids, page - first_page);
+                physical = (long long)id * keys.page_size + within * UNIT;
+            }
+            source.base = keys.latent + physical * WIDTH;
+        }
+        ++unit;
+        if (paged && contiguous && ++within == units_per_page) {
+            within = 0;
+            ++page;
+        }
+        return source;
+    }
+};
+
+// Per-lane offsets of the nine loads of a full unit (no row past the end of the sequence).
+struct FullUnitOffsets {
+    unsigned of[UNIT_LOADS];
+
+    __device__ __forceinline__ void init(int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < UNIT_LOADS; ++i) {
+            of[i] = index_math::contiguous_load_offset<ROW_BYTES, UNIT / 4>(wave, i, lane, UNIT - 1);
+        }
+    }
+};
 
 // Load number i (0..8) of a contiguous unit; i is a constant after unrolling.
-__device__ __forceinline__ void issue_unit_load(const UnitSource& source, int wave, int i, int lane) {
-    direct_load_16_offset(source.base, index_math::contiguous_load_offset<ROW_BYTES, UNIT / 4>(wave, i, lane, source.row_limit),
-                          source.lds_base + i * 1024);
+__device__ __forceinline__ void issue_unit_load(const UnitSource& source, const FullUnitOffsets& offsets, int wave, int i,
+                                                int lane) {
+    const unsigned offset = source.full
+        ? offsets.of[i]
+        : index_math::contiguous_load_offset<ROW_BYTES, UNIT / 4>(wave, i, lane, source.row_limit);
+    direct_load_16_offset(source.base, offset, source.lds_base + i * 1024);
 }
 
 // All nine loads of a unit at once: the first units of a walk, and every unit of the
 // general form (per-lane page lookup).
-__device__ __forceinline__ void issue_unit(const UnitSource& source, const KeyStream& keys, int wave) {
+__device__ __forceinline__ void issue_unit(const UnitSource& source, const FullUnitOffsets& offsets, const KeyStream& keys,
+                                           int wave) {
     if (!source.enabled) return;
     const int lane = fresh_lane_id();
     if (source.contiguous) {
 #pragma unroll
-        for (int i = 0; i < UNIT_LOADS; ++i) issue_unit_load(source, wave, i, lane);
+        for (int i = 0; i < UNIT_LOADS; ++i) issue_unit_load(source, offsets, wave, i, lane);
         return;
     }
 #pragma unroll 1
@@ -766,7 +828,8 @@ template <bool HAS_NEXT>
 __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& scores, f32x16& next_scores,
                                           const bf16x8 (&qf)[KSTEPS], const UnitReads& reads,
                                           const unsigned char* current, const unsigned char* next, int key0, int tokens,
-                                          float c, const UnitSource& request, const KeyStream& keys, int wave) {
+                                          float c, const UnitSource& request, const FullUnitOffsets& offsets,
+                                          const KeyStream& keys, int wave) {
     constexpr int SCORE_MFMAS = HAS_NEXT ? KSTEPS : 0;
     constexpr int COUNT = SCORE_MFMAS + 2 * DBLOCKS;
     const int lane = fresh_lane_id();
@@ -827,7 +890,7 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
     if constexpr (!HAS_NEXT) {
         unrolled<0, 33>(softmax_piece);   // the last unit: no score products to hide it behind
     }
-    if (request.enabled && !request.contiguous) issue_unit(request, keys, wave);
+    if (request.enabled && !request.contiguous) issue_unit(request, offsets, keys, wave);
 
     unrolled<0, COUNT>([&](auto tag) {
         constexpr int I = decltype(tag)::value;
@@ -848,7 +911,7 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
         if constexpr (HAS_NEXT && I < 33) softmax_piece(tag);
         // the requests go between the output MFMAs, which leave more issue slots free than the score MFMAs
         if constexpr (HAS_NEXT && I >= SCORE_MFMAS && (I - SCORE_MFMAS) % 3 == 1 && (I - SCORE_MFMAS) / 3 < UNIT_LOADS) {
-            if (request.enabled && request.contiguous) issue_unit_load(request, wave, (I - SCORE_MFMAS) / 3, lane);
+            if (request.enabled && request.contiguous) issue_unit_load(request, offsets, wave, (I - SCORE_MFMAS) / 3, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
     });
@@ -867,16 +930,20 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
     const int unit_end = min((BN / UNIT) * tile_end, (tokens + UNIT - 1) / UNIT);   // > unit_begin
 
     // The first three units go on their way around the query rows: all latencies overlap.
-    issue_unit(locate_unit(lds, keys, unit_begin, last_token, wave, true), keys, wave);
-    issue_unit(locate_unit(lds, keys, unit_begin + 1, last_token, wave, unit_begin + 1 < unit_end), keys, wave);
+    UnitCursor cursor;
+    cursor.init(keys, unit_begin, last_token);
+    FullUnitOffsets offsets;
+    offsets.init(wave, fresh_lane_id());
+    issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
+    issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
     bf16x8 qf[KSTEPS];
     load_query(qf, query_row, query_row + RANK, valid, (tid % 64) / 32);
-    issue_unit(locate_unit(lds, keys, unit_begin + 2, last_token, wave, unit_begin + 2 < unit_end), keys, wave);
+    issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
     reset(state);
     bool risk = false;
     UnitReads reads;
     reads.init(fresh_lane_id());
-    auto slot_of = [&](int unit) { return lds + (unit % UNIT_SLOTS) * UNIT_BYTES; };
+    auto slot_of = [&](int unit) { return lds + ((unsigned)unit % UNIT_SLOTS) * UNIT_BYTES; };
 
     wait_vector_memory<0>();
     workgroup_barrier();
@@ -905,12 +972,13 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
     for (; unit + 1 < unit_end; ++unit) {
         synchronise(unit);
         unit_step<true>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
-                        locate_unit(lds, keys, unit + 3, last_token, wave, unit + 3 < unit_end), keys, wave);
+                        cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
         // the next unit's scores take the place of this unit's (eight moves against a stream of 68 MFMAs)
         move_scores(scores_a, scores_b);
     }
-    unit_step<false>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c,
-                     locate_unit(lds, keys, unit, last_token, wave, false), keys, wave);
+    UnitSource nothing = {};
+    unit_step<false>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c, nothing,
+                     offsets, keys, wave);
     workgroup_barrier();   // the slots are free: the caller stages its results through them
     return __syncthreads_or(risk) != 0;
 }

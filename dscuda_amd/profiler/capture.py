@@ -58,7 +58,10 @@ PASSES = {
              "SQ_LDS_BANK_CONFLICT", "SQ_INSTS_VALU", "GRBM_GUI_ACTIVE"],
     "waits": ["--pmc", "SQ_WAIT_ANY", "SQ_WAIT_INST_ANY", "SQ_WAIT_INST_LDS", "SQ_ACTIVE_INST_ANY",
               "SQ_ACTIVE_INST_VALU", "SQ_ACTIVE_INST_LDS", "SQ_WAVE_CYCLES", "SQ_INSTS_VMEM"],
+    "lds": ["--pmc", "SQ_INSTS_LDS_LOAD", "SQ_INSTS_LDS_LOAD_BANDWIDTH", "SQ_LDS_IDX_ACTIVE", "SQ_LDS_DATA_FIFO_FULL",
+            "SQ_LDS_CMD_FIFO_FULL", "SQ_INST_LEVEL_LDS", "SQ_INSTS_MFMA", "SQ_BUSY_CYCLES"],
 }
+EXTRA_PASSES = ("waits", "lds")   # reported counter by counter below the table
 DEFAULT_PASSES = ("time", "fetch", "write", "mfma")
 
 Case = collections.namedtuple("Case", "stem label command counter_command kernels")
@@ -241,6 +244,11 @@ def extract_case(case, out, factors):
                     row["mfma_pct"] = 100.0 * settled(counters["SQ_VALU_MFMA_BUSY_CYCLES"]) / (cycles * SIMDS)
             if "SQ_LDS_BANK_CONFLICT" in counters:
                 row["bank_conflict"] = settled(counters["SQ_LDS_BANK_CONFLICT"])
+        row["more"] = collections.OrderedDict()
+        for pass_name in EXTRA_PASSES:
+            table, _ = read_counters(directory / pass_name, case.kernels)
+            for counter, values in table.get(kernel, {}).items():
+                row["more"][f"{pass_name}:{counter}"] = settled(values)
         rows.append(row)
     return rows
 
@@ -293,6 +301,12 @@ def write_case(case, rows, out, profiles, factors):
     lines += ["", f"Counter calibration from the 1 GiB copy: FETCH_SIZE x {factors[0]:.3f}, WRITE_SIZE x {factors[1]:.3f}.",
               "Durations are the mean of the second half of the launches of the timing pass.", ""]
     lines += markdown_table(rows)
+    if any(row.get("more") for row in rows):
+        lines += ["", "Further counters, mean per launch over the second half of the launches (summed over the chip as "
+                      "rocprofv3 reports them):", ""]
+        for row in rows:
+            for name, value in row.get("more", {}).items():
+                lines.append(f"    {row['kernel']} :: {name} = {value:.0f}")
     lines += ["", "Machine-readable (bytes per launch from the two traffic columns, microseconds from the settled column):", ""]
     for row in rows:
         total = (row["read_mb"] + row["write_mb"]) * 1e6

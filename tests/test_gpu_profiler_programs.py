@@ -1,7 +1,5 @@
 """GPU run of the standalone profiler programs: each checks its own results against the closed form of its
-inputs and exits non-zero on a mismatch.  Not collected by pytest under this name: the programs have been
-compiled and their host paths tested, but not yet executed on a GPU; run it by naming the file, and rename
-it to test_*.py once it has passed there."""
+inputs and exits non-zero on a mismatch."""
 
 import json
 import subprocess
@@ -20,6 +18,7 @@ CASES = [
     ("benchmark_mla_prefill", (1, 1024, 8, 192, 128, "--operation", "both")),
     ("benchmark_flash_attention", (2, 256, 8, 128)),
     ("benchmark_flash_attention", (1, 512, 8, 64)),
+    ("hbm_read_probe", (64, 3)),
 ]
 
 
