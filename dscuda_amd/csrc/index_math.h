@@ -183,47 +183,65 @@ DSCUDA_HOST_DEVICE inline unsigned contiguous_load_offset(int wave, int i, int l
     return offset;
 }
 
-// ---- decode: cutting the tile list -------------------------------------------
-// The 64-token tiles of all sequences form one list (sequence after sequence),
-// cut into `workgroups` equal ranges.  A range that holds only part of a
-// sequence leaves a partial result in slot workgroup + sequence: ranges and
-// sequences both advance monotonically, so no two (range, sequence) pairs that
+// ---- decode: cutting the work list ---------------------------------------------
+// Every sequence with tokens contributes `overhead` + tiles positions to one list
+// (sequence after sequence): its 64-token tiles, preceded by positions that stand for
+// what a workgroup spends on a segment besides its tiles (query rows, the first
+// requests, filling and draining the pipeline, storing the result), so that ranges of
+// equal length take about equal time.  The list is cut into W = min(workgroups, total)
+// ranges, none empty, whose lengths differ by at most one: range w is
+// [w * total / W, (w + 1) * total / W).  A
+// range computes the tiles whose positions it holds; a range that holds only part of
+// the tiles of a sequence leaves a partial result in slot workgroup + sequence: ranges
+// and sequences both advance monotonically, so no two (range, sequence) pairs that
 // intersect share a slot, and every slot is below workgroups + sequences.
-DSCUDA_HOST_DEVICE inline int tiles_per_range(int total_tiles, int workgroups) {
-    return (total_tiles + workgroups - 1) / workgroups;
+constexpr int SEGMENT_OVERHEAD = 6;   // in tiles: what a segment costs before, between and after its tiles
+
+DSCUDA_HOST_DEVICE inline int positions_of(int tiles, int overhead) { return tiles > 0 ? tiles + overhead : 0; }
+
+DSCUDA_HOST_DEVICE inline int ranges_of(int total, int workgroups) { return total < workgroups ? total : workgroups; }
+
+// First position of range `range` (0 .. ranges: the last one is the end of the list).
+DSCUDA_HOST_DEVICE inline int range_begin_of(int total, int ranges, int range) {
+    return (int)((long long)range * total / ranges);
 }
 
-DSCUDA_HOST_DEVICE inline int range_begin_of(int total_tiles, int workgroups, int workgroup) {
-    const int first = workgroup * tiles_per_range(total_tiles, workgroups);
-    return first < total_tiles ? first : total_tiles;
+// The range that holds position `position` (0 <= position < total).
+DSCUDA_HOST_DEVICE inline int range_of_position(int total, int ranges, int position) {
+    return (int)((((long long)position + 1) * ranges - 1) / total);
 }
 
-DSCUDA_HOST_DEVICE inline int range_end_of(int total_tiles, int workgroups, int begin) {
-    const int last = begin + tiles_per_range(total_tiles, workgroups);
-    return last < total_tiles ? last : total_tiles;
+// Tiles [first, last) that the positions [begin, end) hold of a sequence whose positions
+// start at `before`; last <= first when they hold none.
+DSCUDA_HOST_DEVICE inline void tiles_in_positions(int begin, int end, int before, int overhead, int& first, int& last) {
+    const int low = begin - before - overhead;
+    const int high = end - before - overhead;
+    first = low > 0 ? low : 0;
+    last = high > 0 ? high : 0;
 }
 
-// First and last range that hold tiles of a sequence of `own` > 0 tiles that starts at tile `before`.
-DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total_tiles, int workgroups, int before, int own, int& first,
-                                                  int& last) {
-    const int per = tiles_per_range(total_tiles, workgroups);
-    first = before / per;
-    last = (before + own - 1) / per;
+// First and last range that hold tiles of a sequence of `positions` > 0 positions that starts at `before`.
+DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total, int ranges, int before, int positions, int overhead,
+                                                  int& first, int& last) {
+    first = range_of_position(total, ranges, before + overhead);
+    last = range_of_position(total, ranges, before + positions - 1);
 }
 
 // ---- decode: the plan and how a call uses the caller's workspace ---------------
 // The plan is what a decode call needs to know about the lengths of its batch
 // before any workgroup starts: an int table
-//     [0] total tiles   [1] workgroups   [2] tiles per range   [3] 1 = sequences are not cut
-//     [4 .. 4+B]        inclusive prefix of tiles per sequence (B + 1 entries)
-//     [.. + W]          first sequence whose tiles reach past the start of each range
+//     [0] total positions   [1] workgroups   [2] overhead positions per sequence   [3] 1 = sequences are not cut
+//     [4] ranges the list is cut into (<= workgroups)
+//     [5 .. 5+B]        inclusive prefix of positions per sequence (B + 1 entries)
+//     [.. + W]          first sequence whose positions reach past the start of each range
 //     [.. + G*B]        one flag per (head group, sequence): some part needs the rescaling pass
 // with G = head groups of 128 heads.  The flags are zero between calls.
 constexpr int PLAN_TOTAL = 0;
 constexpr int PLAN_WORKGROUPS = 1;
-constexpr int PLAN_PER_RANGE = 2;
+constexpr int PLAN_OVERHEAD = 2;
 constexpr int PLAN_WHOLE = 3;
-constexpr int PLAN_HEADER = 4;
+constexpr int PLAN_RANGES = 4;
+constexpr int PLAN_HEADER = 5;
 
 DSCUDA_HOST_DEVICE inline long long plan_prefix_at() { return PLAN_HEADER; }
 DSCUDA_HOST_DEVICE inline long long plan_first_sequence_at(int batch) { return PLAN_HEADER + (long long)batch + 1; }

@@ -923,22 +923,26 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
 // fixed softmax reference (workgroup-uniform): the caller then discards the result.
 __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_row, bool valid, unsigned char* lds,
                                            const KeyStream& keys, int tile_begin, int tile_end, int tokens, float c,
-                                           int tid) {
+                                           int tid, bool cold) {
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int last_token = tokens - 1;
     const int unit_begin = (BN / UNIT) * tile_begin;
     const int unit_end = min((BN / UNIT) * tile_end, (tokens + UNIT - 1) / UNIT);   // > unit_begin
 
-    // The first three units go on their way around the query rows: all latencies overlap.
+    // The first three units and the query rows.  In the middle of a kernel one round trip brings them all.  At the
+    // start of the kernel (`cold`) every workgroup asks at once and the answers come at the rate of the memory, not
+    // of its latency: then only what the first scores need is asked for first, the rest once that has arrived.
     UnitCursor cursor;
     cursor.init(keys, unit_begin, last_token);
     FullUnitOffsets offsets;
     offsets.init(wave, fresh_lane_id());
     issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
-    issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
+    const UnitSource second = cursor.next(lds, keys, last_token, wave, unit_end);
+    const UnitSource third = cursor.next(lds, keys, last_token, wave, unit_end);
+    if (!cold) issue_unit(second, offsets, keys, wave);
     bf16x8 qf[KSTEPS];
     load_query(qf, query_row, query_row + RANK, valid, (tid % 64) / 32);
-    issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
+    if (!cold) issue_unit(third, offsets, keys, wave);
     reset(state);
     bool risk = false;
     UnitReads reads;
@@ -947,6 +951,10 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
 
     wait_vector_memory<0>();
     workgroup_barrier();
+    if (cold) {
+        issue_unit(second, offsets, keys, wave);
+        issue_unit(third, offsets, keys, wave);
+    }
     // scores of the first unit, and the reference every exponential of this walk is taken against
     f32x16 scores_a, scores_b;
     unit_scores(scores_a, qf, slot_of(unit_begin), reads);
@@ -992,14 +1000,16 @@ __device__ __forceinline__ int tiles_of(int length) {
 // ----------------------------------------------------------------------------
 
 using index_math::PLAN_HEADER;
-using index_math::PLAN_PER_RANGE;
+using index_math::PLAN_OVERHEAD;
+using index_math::PLAN_RANGES;
 using index_math::PLAN_TOTAL;
 using index_math::PLAN_WHOLE;
 using index_math::PLAN_WORKGROUPS;
 
-// One workgroup turns the lengths into the plan (index_math.h): the tile prefix, the
-// cut into `workgroups` equal ranges, the first sequence of each range, and cleared
-// flags.  Any batch size: the scan carries over chunks of THREADS lengths.
+// One workgroup turns the lengths into the plan (index_math.h): the prefix of positions
+// (tiles plus the per-sequence overhead when sequences are cut), the first sequence of
+// each of the `workgroups` ranges, and cleared flags.  Any batch size: the scan carries
+// over chunks of THREADS lengths.
 __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restrict__ plan,
                                                                   const int* __restrict__ cache_lengths, int batch_size,
                                                                   int workgroups, int whole_sequences,
@@ -1012,11 +1022,12 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
     int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
     int* flags = plan + index_math::plan_flags_at(batch_size, workgroups);
 
+    const int overhead = whole_sequences ? 0 : index_math::SEGMENT_OVERHEAD;
     int carry = 0;
     if (tid == 0) prefix[0] = 0;
     for (int base = 0; base < batch_size; base += THREADS) {
         const int index = base + tid;
-        int value = index < batch_size ? tiles_of(cache_lengths[index]) : 0;
+        int value = index < batch_size ? index_math::positions_of(tiles_of(cache_lengths[index]), overhead) : 0;
 #pragma unroll
         for (int offset = 1; offset < 64; offset <<= 1) {
             const int other = __shfl_up(value, offset);
@@ -1036,11 +1047,12 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
         __syncthreads();
     }
     const int total = carry;
-    const int per = index_math::tiles_per_range(total, workgroups);
+    const int ranges = index_math::ranges_of(total, workgroups);
     if (tid == 0) {
         plan[PLAN_TOTAL] = total;
         plan[PLAN_WORKGROUPS] = workgroups;
-        plan[PLAN_PER_RANGE] = per;
+        plan[PLAN_OVERHEAD] = overhead;
+        plan[PLAN_RANGES] = ranges;
         plan[PLAN_WHOLE] = whole_sequences;
     }
     for (int index = tid; index < head_groups * batch_size; index += THREADS) flags[index] = 0;
@@ -1048,8 +1060,12 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
     for (int w = tid; w < workgroups; w += THREADS) {
         int sequence = w;
         if (!whole_sequences) {
-            const int begin = index_math::range_begin_of(total, workgroups, w);
-            // first sequence whose tiles reach past `begin`
+            if (w >= ranges) {
+                first_sequence[w] = batch_size;
+                continue;
+            }
+            const int begin = index_math::range_begin_of(total, ranges, w);
+            // first sequence whose positions reach past `begin`
             int low = 0, high = batch_size;
             while (low < high) {
                 const int mid = (low + high) / 2;
@@ -1086,13 +1102,17 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     const int wave = tid / 64;
     const int lq = lane % 32;
     const int g = lane / 32;
-    const int workgroup = blockIdx.x;
+    // Workgroups go to the eight XCDs round-robin by linear id.  Neighbouring ranges are mostly parts of the same
+    // sequence and fetch the same query rows, so each XCD takes a run of consecutive ranges and its L2 serves all but
+    // the first of those fetches.
+    const int workgroup = gridDim.x % 8 == 0 ? (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
     const int head_group = blockIdx.y;
     const int head0 = head_group * ROWS;
     const float c = uniform(scale * LOG2E);
 
     const int total = plan[PLAN_TOTAL];
     const int workgroups = plan[PLAN_WORKGROUPS];
+    const int overhead = plan[PLAN_OVERHEAD];
     const bool whole_sequences = plan[PLAN_WHOLE] != 0;
     const int* prefix = plan + index_math::plan_prefix_at();
     const int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
@@ -1103,8 +1123,10 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         range_begin = prefix[workgroup];
         range_end = prefix[workgroup + 1];
     } else {
-        range_begin = index_math::range_begin_of(total, workgroups, workgroup);
-        range_end = index_math::range_end_of(total, workgroups, range_begin);
+        const int ranges = plan[PLAN_RANGES];
+        if (workgroup >= ranges) return;
+        range_begin = index_math::range_begin_of(total, ranges, workgroup);
+        range_end = index_math::range_begin_of(total, ranges, workgroup + 1);
     }
     if (range_begin >= range_end) return;
     int sequence = first_sequence[workgroup];
@@ -1127,13 +1149,16 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
             ++sequence;
             continue;
         }
-        if (SAFE && flags[sequence] == 0) {   // finished by the fast kernel
+        int tile_begin, tile_end;
+        index_math::tiles_in_positions(position, segment_end, sequence_begin, overhead, tile_begin, tile_end);
+        // no tiles: the range ends among the positions that stand for the sequence's overhead
+        if (tile_end <= tile_begin || (SAFE && flags[sequence] == 0)) {   // ... or finished by the fast kernel
             position = segment_end;
             ++sequence;
             continue;
         }
         const int tokens = cache_lengths[sequence];
-        const bool whole = position == sequence_begin && segment_end == sequence_end;
+        const bool whole = tile_begin == 0 && tile_end == sequence_end - sequence_begin - overhead;
         const bf16_t* query_row = query + ((size_t)sequence * heads + row) * WIDTH;
 
         KeyStream keys;
@@ -1145,11 +1170,10 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.page_size = page_size;
         bool risk;
         if constexpr (SAFE) {
-            risk = walk_rows<true>(state, query_row, query_row + RANK, valid, lds, keys, position - sequence_begin,
-                                   segment_end - sequence_begin, tokens, tokens, c, tid);
+            risk = walk_rows<true>(state, query_row, query_row + RANK, valid, lds, keys, tile_begin, tile_end, tokens, tokens,
+                                   c, tid);
         } else {
-            risk = walk_units(state, query_row, valid, lds, keys, position - sequence_begin, segment_end - sequence_begin,
-                              tokens, c, tid);
+            risk = walk_units(state, query_row, valid, lds, keys, tile_begin, tile_end, tokens, c, tid, position == range_begin);
         }
         const float total_sum = half_wave_sum(state.row_sum);
 
@@ -1203,8 +1227,9 @@ __global__ __launch_bounds__(64) void mla_decode_merge_kernel(bf16_t* __restrict
     const int wave_block = blockIdx.x / MERGE_QUARTERS;   // 32 heads, numbered over all head groups
     const int sequence = blockIdx.y;
 
+    const int total = plan[PLAN_TOTAL];
     const int workgroups = plan[PLAN_WORKGROUPS];
-    const int per = plan[PLAN_PER_RANGE];
+    const int overhead = plan[PLAN_OVERHEAD];
     const int* prefix = plan + index_math::plan_prefix_at();
     if (quarter == 0 && wave_block % (ROWS / 32) == 0 && lane == 0) {
         // this sequence's flag of the head group has been read by everybody who needed it
@@ -1213,8 +1238,8 @@ __global__ __launch_bounds__(64) void mla_decode_merge_kernel(bf16_t* __restrict
     const int sequence_begin = prefix[sequence];
     const int sequence_end = prefix[sequence + 1];
     if (sequence_end <= sequence_begin) return;   // no tiles: nothing was computed for it
-    const int first = sequence_begin / per;
-    const int last = (sequence_end - 1) / per;
+    int first, last;
+    index_math::ranges_of_sequence(total, plan[PLAN_RANGES], sequence_begin, sequence_end - sequence_begin, overhead, first, last);
     if (first == last) return;                    // finished in place by the split kernel
 
     const int head = 32 * wave_block + lq;

@@ -6,7 +6,8 @@
 //               fetches in flight per lane) and XORs them together;
 //   lds         the decode kernel's own instruction: each wave streams 1 KB per instruction
 //               straight into LDS (global_load_lds_dwordx4), 36 KB units through a ring of four
-//               slots with three units in flight per workgroup, one workgroup per compute unit.
+//               slots with one, two or three units in flight per workgroup, one workgroup per
+//               compute unit.
 //
 // Usage: hbm_read_probe [MiB = 1024] [iterations = 20]
 // Prints one line per form and launch shape, and "HBM_READ_PROBE best_GBps=..." at the end.
@@ -57,6 +58,8 @@ constexpr int SLOTS = 4;
 constexpr int WAVE_LOADS = 9;       // 9 KB per wave and unit
 
 // Units blockIdx.x, blockIdx.x + gridDim.x, ... of the buffer; `units` whole units lie inside it.
+// IN_FLIGHT units of a workgroup are on their way at a time (the youngest IN_FLIGHT - 1 are not waited for).
+template <int IN_FLIGHT>
 __global__ __launch_bounds__(256) void read_into_lds(const unsigned char* data, int units, unsigned* sink) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -68,7 +71,7 @@ __global__ __launch_bounds__(256) void read_into_lds(const unsigned char* data, 
         const unsigned target = lds_base + (issued % SLOTS) * UNIT_BYTES + wave * (WAVE_LOADS * 1024);
 #pragma unroll
         for (int i = 0; i < WAVE_LOADS; ++i) dscuda::direct_load_16_offset(source, i * 1024 + lane * 16, target + i * 1024);
-        dscuda::wait_vector_memory<2 * WAVE_LOADS>();   // two younger units may still be on their way
+        dscuda::wait_vector_memory<(IN_FLIGHT - 1) * WAVE_LOADS>();
     }
     dscuda::wait_vector_memory<0>();
     dscuda::workgroup_barrier();
@@ -91,8 +94,10 @@ int main(int argc, char** argv) {
         PROFILER_HIP_CHECK(hipGetLastError());
         unsigned expected = 0;   // XOR of every word of the buffer
         for (size_t i = 0; i < bytes / 4; ++i) expected ^= (unsigned)i * 2654435761u;
-        PROFILER_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(read_into_lds),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, SLOTS * UNIT_BYTES));
+        for (const void* kernel : {reinterpret_cast<const void*>(read_into_lds<1>), reinterpret_cast<const void*>(read_into_lds<2>),
+                                   reinterpret_cast<const void*>(read_into_lds<3>)}) {
+            PROFILER_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SLOTS * UNIT_BYTES));
+        }
         hipEvent_t start, stop;
         PROFILER_HIP_CHECK(hipEventCreate(&start));
         PROFILER_HIP_CHECK(hipEventCreate(&stop));
@@ -122,9 +127,13 @@ int main(int argc, char** argv) {
             if (folded != expected) throw std::runtime_error("register form: XOR of the buffer differs from its closed form");
         }
         const int units = (int)std::min<size_t>(bytes / UNIT_BYTES, 1u << 30);
-        timed("lds", 256, (double)units * UNIT_BYTES, [&] {
-            read_into_lds<<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, reinterpret_cast<unsigned*>(sink.get()));
-        });
+        unsigned* words = reinterpret_cast<unsigned*>(sink.get());
+        timed("lds x1", 256, (double)units * UNIT_BYTES,
+              [&] { read_into_lds<1><<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, words); });
+        timed("lds x2", 256, (double)units * UNIT_BYTES,
+              [&] { read_into_lds<2><<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, words); });
+        timed("lds x3", 256, (double)units * UNIT_BYTES,
+              [&] { read_into_lds<3><<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, words); });
         std::printf("check passed\nHBM_READ_PROBE bytes=%zu best_GBps=%.1f\n", bytes, best);
         PROFILER_HIP_CHECK(hipEventDestroy(start));
         PROFILER_HIP_CHECK(hipEventDestroy(stop));

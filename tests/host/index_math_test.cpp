@@ -259,31 +259,50 @@ void check_decode_loads() {
     }
 }
 
-// ---- decode: the ranges partition the tile list; (range, sequence) pairs that intersect own distinct slots
+// ---- decode: the ranges partition the list of positions, their lengths differ by at most one, every tile of every
+// sequence is computed by exactly one range, and (range, sequence) pairs that hold part of a sequence own distinct slots
 void check_decode_ranges() {
     unsigned state = 12345;
     auto random = [&](int low, int high) { state = state * 1664525u + 1013904223u; return low + (int)((state >> 8) % (unsigned)(high - low + 1)); };
-    for (int trial = 0; trial < 400; ++trial) {
+    for (int trial = 0; trial < 600; ++trial) {
         const int sequences = random(1, 70);
-        const int workgroups = random(1, 300);
-        std::vector<int> prefix(sequences + 1, 0);
-        for (int s = 0; s < sequences; ++s) prefix[s + 1] = prefix[s] + random(trial % 3 == 0 ? 0 : 1, trial % 2 ? 130 : 5);
+        int workgroups = random(1, 300);
+        const int overhead = trial % 4 == 0 ? 0 : (trial % 4 == 1 ? SEGMENT_OVERHEAD : random(1, 9));
+        std::vector<int> tiles(sequences), prefix(sequences + 1, 0);
+        for (int s = 0; s < sequences; ++s) {
+            tiles[s] = random(trial % 3 == 0 ? 0 : 1, trial % 2 ? 130 : 5);
+            prefix[s + 1] = prefix[s] + positions_of(tiles[s], overhead);
+        }
         const int total = prefix[sequences];
         if (total == 0) continue;
-        int expected_begin = 0;
+        const int launched = workgroups;
+        workgroups = ranges_of(total, launched);   // the ranges the list is cut into
+        EXPECT(workgroups >= 1 && workgroups <= launched && workgroups <= total, "%d ranges for %d positions, %d workgroups", workgroups, total, launched);
         std::set<int> slots;
-        std::vector<int> covered(total, 0);
+        std::vector<std::vector<int>> covered(sequences);
+        for (int s = 0; s < sequences; ++s) covered[s].assign(tiles[s], 0);
+        EXPECT(range_begin_of(total, workgroups, 0) == 0 && range_begin_of(total, workgroups, workgroups) == total, "ends of the list");
+        int shortest = total, longest = 0;
         for (int w = 0; w < workgroups; ++w) {
-            const int begin = range_begin_of(total, workgroups, w), end = range_end_of(total, workgroups, begin);
-            EXPECT(begin == std::min(expected_begin, total) && end >= begin && end <= total, "workgroup %d range %d..%d", w, begin, end);
-            expected_begin = end;
+            const int begin = range_begin_of(total, workgroups, w), end = range_begin_of(total, workgroups, w + 1);
+            EXPECT(end > begin, "workgroup %d range %d..%d", w, begin, end);
+            shortest = std::min(shortest, end - begin);
+            longest = std::max(longest, end - begin);
+            for (int position = begin; position < end; ++position) {
+                EXPECT(range_of_position(total, workgroups, position) == w, "position %d of %d, %d workgroups: owner %d, in range %d", position,
+                       total, workgroups, range_of_position(total, workgroups, position), w);
+            }
             for (int s = 0; s < sequences; ++s) {
                 const int low = std::max(begin, prefix[s]), high = std::min(end, prefix[s + 1]);
                 if (low >= high) continue;
-                for (int tile = low; tile < high; ++tile) ++covered[tile];
-                const bool whole = low == prefix[s] && high == prefix[s + 1];
+                int first_tile, last_tile;
+                tiles_in_positions(low, high, prefix[s], overhead, first_tile, last_tile);
+                if (last_tile <= first_tile) continue;   // only positions of the sequence's overhead
+                EXPECT(first_tile >= 0 && last_tile <= tiles[s], "sequence %d tiles %d..%d of %d", s, first_tile, last_tile, tiles[s]);
+                for (int tile = first_tile; tile < last_tile; ++tile) ++covered[s][tile];
+                const bool whole = first_tile == 0 && last_tile == tiles[s];
                 int first, last;
-                ranges_of_sequence(total, workgroups, prefix[s], prefix[s + 1] - prefix[s], first, last);
+                ranges_of_sequence(total, workgroups, prefix[s], prefix[s + 1] - prefix[s], overhead, first, last);
                 EXPECT(first <= w && w <= last, "sequence %d is in range %d but its ranges are %d..%d", s, w, first, last);
                 EXPECT(whole == (first == last), "sequence %d whole %d first %d last %d", s, (int)whole, first, last);
                 if (!whole) {
@@ -293,8 +312,20 @@ void check_decode_ranges() {
                 }
             }
         }
-        EXPECT(expected_begin == total, "ranges end at %d of %d", expected_begin, total);
-        for (int tile = 0; tile < total; ++tile) EXPECT(covered[tile] == 1, "tile %d covered %d times", tile, covered[tile]);
+        EXPECT(longest - shortest <= 1, "range lengths %d..%d", shortest, longest);
+        for (int s = 0; s < sequences; ++s) {
+            for (int tile = 0; tile < tiles[s]; ++tile) EXPECT(covered[s][tile] == 1, "sequence %d tile %d covered %d times", s, tile, covered[s][tile]);
+            if (tiles[s] == 0) continue;
+            // every range between the first and the last of a sequence holds some of its tiles (the merge reads them all)
+            int first, last;
+            ranges_of_sequence(total, workgroups, prefix[s], prefix[s + 1] - prefix[s], overhead, first, last);
+            for (int w = first; w <= last; ++w) {
+                const int begin = range_begin_of(total, workgroups, w), end = range_begin_of(total, workgroups, w + 1);
+                int first_tile, last_tile;
+                tiles_in_positions(std::max(begin, prefix[s]), std::min(end, prefix[s + 1]), prefix[s], overhead, first_tile, last_tile);
+                EXPECT(last_tile > first_tile, "sequence %d: range %d of %d..%d holds none of its tiles", s, w, first, last);
+            }
+        }
     }
 }
 
