@@ -282,7 +282,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     bf16_t* __restrict__ key_gradient, bf16_t* __restrict__ value_gradient, unsigned char* __restrict__ ds_blocks,
     const float* __restrict__ statistics, const bf16_t* __restrict__ output_gradient,
     const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
-    int sequence_length, int heads, int key_blocks, int query_tiles, float scale) {
+    int sequence_length, int heads, int key_blocks, int query_tiles, int first_pair, float scale) {
     using C = KeyValueGradConfig<DQK, DV>;
     constexpr int QK_STEPS = DQK / 16;
     constexpr int V_STEPS = DV / 16;
@@ -321,6 +321,10 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             kb = blockIdx.x % key_blocks;
         }
     }
+    // the launch covers the (batch, head) pairs first_pair .. first_pair + gridDim.x / key_blocks - 1; the dS blocks
+    // of pair first_pair + i sit at position i of the workspace
+    const int local_pair = bh;
+    bh += first_pair;
     const int b = bh / heads;
     const int h = bh % heads;
     const int k0 = kb * KBLOCK;
@@ -536,7 +540,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         f32x16 dk_acc[DK_BLOCKS];
 #pragma unroll
         for (int d = 0; d < DK_BLOCKS; ++d) clear(dk_acc[d]);
-        unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+        unsigned char* ds_head = ds_blocks + (size_t)local_pair * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
         constexpr int DK_MFMAS = 4 * DK_BLOCKS;
         constexpr int DP_MFMAS = 2 * V_STEPS;
         static_assert(RING <= DK_MFMAS && RING <= DP_MFMAS, "a ring of fragments must fit each product");
@@ -683,7 +687,7 @@ constexpr int DQ_THREADS = 512;
 template <int DQK>
 __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
     bf16_t* __restrict__ query_gradient, const unsigned char* __restrict__ ds_blocks, const bf16_t* __restrict__ key,
-    int sequence_length, int heads, int query_blocks, int key_blocks, int query_tiles, float scale) {
+    int sequence_length, int heads, int query_blocks, int key_blocks, int query_tiles, int first_pair, float scale) {
     using C = QueryGradConfig<DQK>;
     constexpr int WAVES = DQ_THREADS / 64;
 
@@ -699,6 +703,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
     int bh, rank;
     xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, rank);
     const int jb = query_blocks - 1 - rank;   // heaviest (last) query blocks first
+    const int local_pair = bh;                // position of this pair's dS blocks in the workspace
+    bh += first_pair;
     const int b = bh / heads;
     const int h = bh % heads;
     const int tile_of_wave = wave % 2;
@@ -707,7 +713,7 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
 
     const unsigned k_stride_bytes = (unsigned)heads * DQK * 2;
     const unsigned char* k_base = reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * heads + h) * DQK);
-    const unsigned char* ds_head = ds_blocks + (size_t)bh * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+    const unsigned char* ds_head = ds_blocks + (size_t)local_pair * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
     const unsigned lds_base = lds_offset_of(lds);
 
     // query tiles of this workgroup (the second may not exist at a ragged end: it
@@ -891,12 +897,31 @@ void raise_lds_limit(Kernel kernel, int bytes) {
     }
 }
 
+// The dS blocks of one (batch, head) pair take about S * S bytes, so a long sequence with many heads would ask for
+// tens of gigabytes if every pair kept its own.  The two gradient passes therefore run over the pairs in chunks that
+// share one set of dS blocks of at most DS_BUDGET_BYTES (the chunk of a launch is a multiple of 8 pairs when it can
+// be: one pair at a time per XCD); the statistics, small, are computed for all pairs at once.
+// DSCUDA_AMD_DS_BUDGET_BYTES in the environment (read once) replaces the budget: for tests of the chunked path at
+// small sizes, and for callers who would rather trade launches for memory.
+constexpr long long DS_BUDGET_BYTES = 3LL << 30;
+
+long long ds_budget_bytes() {
+    static const long long budget = [] {
+        const char* text = std::getenv("DSCUDA_AMD_DS_BUDGET_BYTES");
+        const long long value = text ? std::strtoll(text, nullptr, 10) : 0;
+        return value > 0 ? value : DS_BUDGET_BYTES;
+    }();
+    return budget;
+}
+
 struct BackwardShape {
     int key_blocks;
     int query_tiles;
     int query_blocks;
-    long long statistics_floats;   // per launch
-    long long ds_floats;
+    long long pairs;               // batch * heads
+    long long pairs_per_launch;
+    long long statistics_floats;   // all pairs
+    long long ds_floats;           // one chunk of pairs
 };
 
 BackwardShape backward_shape(int batch_size, int sequence_length, int heads) {
@@ -904,9 +929,14 @@ BackwardShape backward_shape(int batch_size, int sequence_length, int heads) {
     shape.key_blocks = (sequence_length + KBLOCK - 1) / KBLOCK;
     shape.query_tiles = (sequence_length + QTILE - 1) / QTILE;
     shape.query_blocks = shape.key_blocks;   // 128 queries per workgroup of the dQ pass
-    const long long groups = (long long)batch_size * heads;
-    shape.statistics_floats = groups * shape.query_tiles * STAT_FLOATS;
-    shape.ds_floats = groups * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_FLOATS;
+    shape.pairs = (long long)batch_size * heads;
+    shape.statistics_floats = shape.pairs * shape.query_tiles * STAT_FLOATS;
+    const long long pair_bytes = (long long)ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_BYTES;
+    long long chunk = pair_bytes > 0 ? ds_budget_bytes() / pair_bytes : shape.pairs;
+    if (chunk >= 8) chunk -= chunk % 8;
+    if (chunk < 1) chunk = 1;
+    shape.pairs_per_launch = chunk < shape.pairs ? chunk : shape.pairs;
+    shape.ds_floats = shape.pairs_per_launch * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_FLOATS;
     return shape;
 }
 
@@ -939,15 +969,19 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
                        0, stream, statistics, output_gradient, output, logsumexp, batch_size, sequence_length, heads,
                        shape.query_tiles);
     HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL((attention_key_value_gradient_kernel<DQK, DV>), dim3((unsigned)(groups * shape.key_blocks)),
-                       dim3(KV_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
-                       output_gradient, query, key, value, sequence_length, heads, shape.key_blocks,
-                       shape.query_tiles, scale);
-    HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>), dim3((unsigned)(groups * shape.query_blocks)),
-                       dim3(DQ_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
-                       heads, shape.query_blocks, shape.key_blocks, shape.query_tiles, scale);
-    HIP_CHECK(hipGetLastError());
+    for (long long first = 0; first < shape.pairs; first += shape.pairs_per_launch) {
+        const long long count = std::min(shape.pairs_per_launch, shape.pairs - first);
+        hipLaunchKernelGGL((attention_key_value_gradient_kernel<DQK, DV>), dim3((unsigned)(count * shape.key_blocks)),
+                           dim3(KV_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
+                           output_gradient, query, key, value, sequence_length, heads, shape.key_blocks,
+                           shape.query_tiles, (int)first, scale);
+        HIP_CHECK(hipGetLastError());
+        // the next chunk's first pass overwrites the dS blocks: it follows this pass in the stream
+        hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>), dim3((unsigned)(count * shape.query_blocks)),
+                           dim3(DQ_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
+                           heads, shape.query_blocks, shape.key_blocks, shape.query_tiles, (int)first, scale);
+        HIP_CHECK(hipGetLastError());
+    }
 }
 
 }  // namespace

@@ -93,10 +93,15 @@ def mla_prefill_forward(query, key, value, scale, out=None, lse=None):
     return out, lse
 
 
+def mla_prefill_backward_workspace_elements(batch, seq, heads, dqk, dv):
+    """fp32 elements of the per-head backward's workspace (dscuda_mla_prefill_backward_workspace_elements)."""
+    return mla_library().prefill_workspace(batch, seq, heads, dqk, dv)
+
+
 def mla_prefill_backward_workspace(batch, seq, heads, dqk, dv, device="cuda"):
-    """fp32 workspace of the per-head backward: row statistics plus the bf16 dS blocks
-    that the dK/dV kernel hands to the dQ pass (about S^2 bytes per head)."""
-    elements = mla_library().prefill_workspace(batch, seq, heads, dqk, dv)
+    """fp32 workspace of the per-head backward: row statistics plus the bf16 dS blocks that the dK/dV kernel hands
+    to the dQ pass (about S^2 bytes per (batch, head) pair, for as many pairs as one pass covers)."""
+    elements = mla_prefill_backward_workspace_elements(batch, seq, heads, dqk, dv)
     return torch.empty(elements, device=device, dtype=torch.float32)
 
 

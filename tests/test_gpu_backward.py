@@ -4,6 +4,11 @@ C-ABI.  As in the reference harness (benchmarks/mla.py:68,113-117) the
 backward is fed the oracle's own bf16-rounded O and fp32 LSE, so forward and
 backward are tested independently."""
 
+import os
+import subprocess
+import sys
+from pathlib import Path
+
 import pytest
 import torch
 
@@ -125,3 +130,30 @@ def test_absorbed_backward_closed_form_constant_fill(cuda):
     before = torch.cat([torch.zeros(1, dtype=torch.float64), harmonic[:-1]])
     expected = (heads * 0.015625 * (harmonic[-1] - before)).float()
     assert (dlat - expected[None, :, None]).abs().max() <= 4e-3  # bf16 rounding of values up to 0.32
+
+
+@pytest.mark.parametrize("batch,seq,heads,budget_pairs,expected_chunk", [
+    (2, 640, 12, 9.5, 8),     # 24 pairs in chunks of 8 (a multiple of 8 when the budget allows one)
+    (1, 640, 7, 2.5, 2),      # 7 pairs in chunks of 2, 2, 2, 1
+    (1, 300, 3, 0.5, 1),      # a budget below one pair still runs, one pair at a time
+])
+def test_backward_in_chunks_of_pairs(cuda, batch, seq, heads, budget_pairs, expected_chunk):
+    """The dS workspace is bounded: with a budget that holds only some (batch, head) pairs the two gradient passes run
+    chunk after chunk over one set of dS blocks, and the workspace the library asks for shrinks accordingly."""
+    key_blocks, tiles = (seq + 127) // 128, (seq + 63) // 64
+    pair_bytes = sum(tiles - 2 * kb for kb in range(key_blocks)) * 16384
+    environment = dict(os.environ, DSCUDA_AMD_DS_BUDGET_BYTES=str(int(budget_pairs * pair_bytes)))
+    root = Path(__file__).resolve().parents[1]
+    result = subprocess.run([sys.executable, "-m", "tests.backward_chunk_case", str(batch), str(seq), str(heads),
+                             str(expected_chunk)], cwd=root, env=environment, capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stdout[-2000:] + result.stderr[-4000:]
+    assert "chunked backward ok" in result.stdout
+
+
+def test_backward_workspace_is_bounded(cuda):
+    """Workload 5 (S=16384, H=128) asks for less than 4 GiB; workload 3 still fits one launch."""
+    long_case = ops.mla_prefill_backward_workspace_elements(1, 16384, 128, 192, 128)
+    assert long_case * 4 < 4 << 30, long_case
+    tiles, key_blocks = 64, 32
+    blocks = sum(tiles - 2 * kb for kb in range(key_blocks))
+    assert ops.mla_prefill_backward_workspace_elements(1, 4096, 128, 192, 128) == 128 * tiles * 128 + 128 * blocks * 4096
