@@ -204,6 +204,11 @@ void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* k
                                 scale, stream);
 }
 
+void rope_apply_cuda(__hip_bfloat16* tensor, const int* positions, int batch_size, int sequence_length, int heads,
+                     int width, int rope_offset, int rope_size, float theta, hipStream_t stream) {
+    rope_apply_dispatch(tensor, positions, batch_size, sequence_length, heads, width, rope_offset, rope_size, theta, stream);
+}
+
 }  // namespace dscuda
 
 namespace {
@@ -315,5 +320,12 @@ extern "C" int dscuda_mla_prefill_backward(__hip_bfloat16* dquery, __hip_bfloat1
     return guarded([&] {
         dscuda::mla_prefill_backward_cuda(dquery, dkey, dvalue, dout, output, lse, query, key, value, workspace,
                                           batch, sequence, heads, qk_head_size, v_head_size, scale, stream);
+    });
+}
+
+extern "C" int dscuda_rope_apply(__hip_bfloat16* tensor, const int* positions, int batch, int sequence, int heads,
+                                 int width, int rope_offset, int rope_size, float theta, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::rope_apply_cuda(tensor, positions, batch, sequence, heads, width, rope_offset, rope_size, theta, stream);
     });
 }

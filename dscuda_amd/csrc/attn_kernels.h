@@ -31,6 +31,11 @@ void attention_backward_dispatch(__hip_bfloat16* query_gradient, __hip_bfloat16*
                                  int sequence_length, int heads, int qk_head_size, int v_head_size, float scale,
                                  hipStream_t stream);
 
+// rope.hip -- rotary position embedding, in place, on columns rope_offset .. rope_offset + rope_size - 1 of a
+// [B, S, H, width] bf16 tensor (interleaved pairs; positions: per-sequence start positions or nullptr for 0).
+void rope_apply_dispatch(__hip_bfloat16* tensor, const int* positions, int batch_size, int sequence_length, int heads,
+                         int width, int rope_offset, int rope_size, float theta, hipStream_t stream);
+
 // mla_absorbed.hip -- absorbed (C=512, R=64) causal forward and backward with
 // one shared latent KV head.
 void mla_absorbed_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query_latent,

@@ -37,6 +37,7 @@ class _Mla:
         self.decode_planned = bind(lib, "dscuda_mla_decode_planned", [P] * 8 + [I] * 7 + [F, P])
         self.decode_static = bind(lib, "dscuda_mla_decode_static", [P] * 6 + [I] * 7 + [F, P])
         self.workspace = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
+        self.rope_apply = bind(lib, "dscuda_rope_apply", [P] * 2 + [I] * 6 + [F, P])
         self.prefill_forward = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
         self.prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
         self.prefill_workspace = bind(
@@ -211,3 +212,21 @@ def mla_decode_planned(packed_query, paged_cache, block_table, lengths, plan, sc
         *pointers((out, lse, packed_query, paged_cache, block_table, lengths, workspace, plan)),
         b, h, rank, width - rank, paged_cache.shape[1], block_table.shape[1], splits, scale, stream()))
     return out, lse
+
+
+def rope_apply(tensor, rope_offset=0, rope_size=None, theta=10000.0, positions=None):
+    """Rotary position embedding in place on columns rope_offset .. rope_offset + rope_size - 1 of a contiguous
+    [B,S,H,W] bf16 tensor (dscuda_rope_apply); positions: int32 [B] start positions or None.  Returns the tensor."""
+    _require_cuda(tensor)
+    if tensor.dim() != 4 or not tensor.is_contiguous() or tensor.dtype != torch.bfloat16:
+        raise ValueError("rope_apply: a contiguous bf16 [B,S,H,W] tensor is required")
+    b, s, h, w = tensor.shape
+    rope_size = w - rope_offset if rope_size is None else rope_size
+    if positions is not None:
+        _require_cuda(positions)
+        if positions.dtype != torch.int32 or positions.numel() != b:
+            raise ValueError("rope_apply: positions must be int32 [B]")
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.rope_apply(tensor.data_ptr(), positions.data_ptr() if positions is not None else None,
+                                           b, s, h, w, rope_offset, rope_size, theta, stream()))
+    return tensor

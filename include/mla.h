@@ -240,6 +240,26 @@ void mla_prefill_backward_cuda(
     float scale,
     hipStream_t stream = nullptr);
 
+// Rotary position embedding in place on columns rope_offset .. rope_offset + rope_size - 1 of
+// every row of a [batch, sequence, heads, width] BF16 tensor: within the slice, columns
+// (2i, 2i + 1) are rotated by position * theta^(-2i / rope_size), position = s +
+// positions[b] (positions == nullptr: s).  The step before the attention kernels of an MLA
+// layer -- q_rope [B,S,H,64] and k_rope [B,S,1,64] with rope_offset 0, or the rope columns
+// 128..191 of per-head Q / K [B,S,H,192] -- that the reference leaves to its caller
+// (reference/python/sources.json:2); it has no counterpart there.  rope_size a power of two
+// up to 128; offset and width even.
+void rope_apply_cuda(
+    __hip_bfloat16* tensor,
+    const int* positions,
+    int batch_size,
+    int sequence_length,
+    int heads,
+    int width,
+    int rope_offset,
+    int rope_size,
+    float theta,
+    hipStream_t stream = nullptr);
+
 }  // namespace dscuda
 
 // ---- C ABI (libdscuda_mla_bench.so) ----------------------------------------
@@ -315,6 +335,12 @@ int dscuda_mla_prefill_backward(
     const __hip_bfloat16* query, const __hip_bfloat16* key, const __hip_bfloat16* value,
     float* workspace,
     int batch, int sequence, int heads, int qk_head_size, int v_head_size, float scale,
+    hipStream_t stream);
+
+// additive (no counterpart in the reference): see dscuda::rope_apply_cuda above; errors through dscuda_mla_last_error
+int dscuda_rope_apply(
+    __hip_bfloat16* tensor, const int* positions,
+    int batch, int sequence, int heads, int width, int rope_offset, int rope_size, float theta,
     hipStream_t stream);
 
 }  // extern "C"
