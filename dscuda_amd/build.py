@@ -37,7 +37,7 @@ COMMON_FLAGS = [
 
 LIBRARIES = {
     "libdscuda_mla_bench.so": ["api_mla", "attn_fwd", "attn_bwd", "mla_absorbed", "mla_decode", "rope"],
-    "libdscuda_flash_attention_bench.so": ["api_flash", "attn_fwd"],
+    "libdscuda_flash_attention_bench.so": ["api_flash", "attn_fwd", "attn_bwd"],
 }
 
 

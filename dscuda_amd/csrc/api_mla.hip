@@ -185,7 +185,7 @@ std::size_t mla_prefill_backward_workspace_elements(int batch_size, int sequence
     if (batch_size <= 0 || sequence_length <= 0 || heads <= 0) {
         return 0;
     }
-    return attention_backward_workspace_elements(batch_size, sequence_length, heads);
+    return attention_backward_workspace_elements(batch_size, sequence_length, heads, heads);
 }
 
 void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
@@ -200,8 +200,8 @@ void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* k
         throw std::invalid_argument("MLA prefill backward requires a workspace");
     }
     attention_backward_dispatch(query_gradient, key_gradient, value_gradient, output_gradient, output, logsumexp, query,
-                                key, value, workspace, batch_size, sequence_length, heads, qk_head_size, v_head_size,
-                                scale, stream);
+                                key, value, workspace, batch_size, sequence_length, heads, heads, qk_head_size,
+                                v_head_size, scale, stream);
 }
 
 void rope_apply_cuda(__hip_bfloat16* tensor, const int* positions, int batch_size, int sequence_length, int heads,

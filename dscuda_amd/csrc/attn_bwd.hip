@@ -282,7 +282,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     bf16_t* __restrict__ key_gradient, bf16_t* __restrict__ value_gradient, unsigned char* __restrict__ ds_blocks,
     const float* __restrict__ statistics, const bf16_t* __restrict__ output_gradient,
     const bf16_t* __restrict__ query, const bf16_t* __restrict__ key, const bf16_t* __restrict__ value,
-    int sequence_length, int heads, int key_blocks, int query_tiles, int first_pair, float scale) {
+    int sequence_length, int heads, int kv_heads, int key_blocks, int query_tiles, int first_pair, float scale) {
     using C = KeyValueGradConfig<DQK, DV>;
     constexpr int QK_STEPS = DQK / 16;
     constexpr int V_STEPS = DV / 16;
@@ -321,27 +321,36 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             kb = blockIdx.x % key_blocks;
         }
     }
-    // the launch covers the (batch, head) pairs first_pair .. first_pair + gridDim.x / key_blocks - 1; the dS blocks
-    // of pair first_pair + i sit at position i of the workspace
+    // The launch covers the (batch, key/value head) pairs first_pair .. first_pair + gridDim.x / key_blocks - 1.
+    // `heads` query heads share `kv_heads` key/value heads: query heads h * sharing .. + sharing - 1 read key/value
+    // head h, and this workgroup walks the query tiles of each of them in turn, all into the same dK / dV
+    // accumulators.  The dS blocks of member m of pair first_pair + i sit at position i * sharing + m of the
+    // workspace (query-head order, which is how the query-gradient pass finds them).
+    const int sharing = heads / kv_heads;
     const int local_pair = bh;
     bh += first_pair;
-    const int b = bh / heads;
-    const int h = bh % heads;
+    const int b = bh / kv_heads;
+    const int h = bh % kv_heads;          // key/value head
+    const int first_query_head = h * sharing;
     const int k0 = kb * KBLOCK;
     const int group_k0 = k0 + 32 * group;
     const int key_row = group_k0 + lq;
 
-    const size_t qk_stride = (size_t)heads * DQK;
-    const size_t v_stride = (size_t)heads * DV;
+    const size_t qk_stride = (size_t)kv_heads * DQK;   // rows of K and dK
+    const size_t v_stride = (size_t)kv_heads * DV;     // rows of V and dV
     const unsigned q_stride_bytes = (unsigned)heads * DQK * 2;
     const unsigned o_stride_bytes = (unsigned)heads * DV * 2;
-    const unsigned char* q_base = reinterpret_cast<const unsigned char*>(query + ((size_t)b * S * heads + h) * DQK);
+    // of the first query head of the group; member m follows m head rows further
+    const unsigned char* q_base =
+        reinterpret_cast<const unsigned char*>(query + ((size_t)b * S * heads + first_query_head) * DQK);
     const unsigned char* do_base =
-        reinterpret_cast<const unsigned char*>(output_gradient + ((size_t)b * S * heads + h) * DV);
-    const float* stat_base = statistics + (size_t)bh * query_tiles * STAT_FLOATS;
+        reinterpret_cast<const unsigned char*>(output_gradient + ((size_t)b * S * heads + first_query_head) * DV);
+    const float* stat_base = statistics + ((size_t)b * heads + first_query_head) * query_tiles * STAT_FLOATS;
     const unsigned lds_base = lds_offset_of(lds);
 
-    const int tiles = query_tiles - 2 * kb;   // >= 1; step `index` works on tile query_tiles - 1 - index
+    // Step `index` of the walk works on tile query_tiles - 1 - index % tiles of member index / tiles.
+    const int tiles = query_tiles - 2 * kb;   // >= 1, per member
+    const int steps = tiles * sharing;
 
     // Tiles are requested by the four value waves, each the same number of loads per
     // tile: a value wave then knows that all but its last REQUEST_LOADS loads have
@@ -353,15 +362,18 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     o_requests.init(o_stride_bytes, wave % 4, lane);
     constexpr int REQUEST_LOADS = TileRequests<C::Q_ROW, 4>::LOADS + TileRequests<C::O_ROW, 4>::LOADS + 1;
     auto request_tile = [&](int index) {
-        const int tile = query_tiles - 1 - index;
+        const int member = index / tiles;
+        const int tile = query_tiles - 1 - (index - member * tiles);
         const int row0 = tile * QTILE;
         const int row_limit = S - 1 - row0;
         const unsigned target = lds_base + (index % 3) * C::STAGE_BYTES;
-        q_requests.request(q_base + (size_t)row0 * q_stride_bytes, q_stride_bytes, row_limit, target, wave);
-        o_requests.request(do_base + (size_t)row0 * o_stride_bytes, o_stride_bytes, row_limit, target + C::Q_BYTES, wave);
+        q_requests.request(q_base + (size_t)member * (DQK * 2) + (size_t)row0 * q_stride_bytes, q_stride_bytes, row_limit,
+                           target, wave);
+        o_requests.request(do_base + (size_t)member * (DV * 2) + (size_t)row0 * o_stride_bytes, o_stride_bytes, row_limit,
+                           target + C::Q_BYTES, wave);
         // statistics: 128 floats = two loads; waves 2 and 3 repeat those of waves 0 and 1
         // (same bytes to the same place) so that every value wave issues the same count
-        direct_load_4_offset(stat_base + (size_t)tile * STAT_FLOATS + 64 * (wave % 2), 4u * lane,
+        direct_load_4_offset(stat_base + ((size_t)member * query_tiles + tile) * STAT_FLOATS + 64 * (wave % 2), 4u * lane,
                              target + C::Q_BYTES + C::O_BYTES + 256 * (wave % 2));
     };
 
@@ -378,10 +390,10 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     if (!key_wave) {
         // ================= value wave: S, P, dV =================
         request_tile(0);
-        if (tiles > 1) {
+        if (steps > 1) {
             request_tile(1);
         }
-        const bf16_t* k_base = key + ((size_t)b * S * heads + h) * DQK;
+        const bf16_t* k_base = key + ((size_t)b * S * kv_heads + h) * DQK;
         bf16x8 kf[QK_STEPS];   // B operand: column = key lq
         load_row_fragments<DQK>(kf, k_base, qk_stride, key_row, key_row < S, g);
         f32x16 dv_acc[DV_BLOCKS];
@@ -437,13 +449,13 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         auto value_tile = [&](auto masked_tag, int index) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             workgroup_barrier();   // A: every wave has left tile index - 1
-            if (index + 2 < tiles) {
+            if (index + 2 < steps) {
                 request_tile(index + 2);
             }
             // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
             // local index below `threshold` lies before this lane's key.
             u32x4 pf[2][2];
-            const int threshold = key_row - 4 * g - (query_tiles - 1 - index) * QTILE;
+            const int threshold = key_row - 4 * g - (query_tiles - 1 - index % tiles) * QTILE;
             static_for<0, 2>([&](auto qb_tag) {
                 constexpr int QB = decltype(qb_tag)::value;
                 static_for<0, 4>([&](auto i4_tag) {
@@ -470,7 +482,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             });
             // this wave's share of tile index + 1 has landed (the request of tile index + 2,
             // if there is one, may stay in flight)
-            if (index + 2 < tiles) {
+            if (index + 2 < steps) {
                 wait_vector_memory<REQUEST_LOADS>();
             } else {
                 wait_vector_memory<0>();
@@ -493,7 +505,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
-            if (index + 1 < tiles) {
+            if (index + 1 < steps) {
                 score_stream(index + 1);
             }
         };
@@ -501,12 +513,11 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         wait_vector_memory<0>();
         workgroup_barrier();
         score_stream(0);
-        {
-            int index = 0;
-            for (; index < tiles - 2; ++index) {
+        for (int member = 0, index = 0; member < sharing; ++member) {
+            for (int local = 0; local < tiles - 2; ++local, ++index) {
                 value_tile(std::false_type{}, index);
             }
-            for (; index < tiles; ++index) {
+            for (int local = max(tiles - 2, 0); local < tiles; ++local, ++index) {
                 value_tile(std::true_type{}, index);
             }
         }
@@ -523,7 +534,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             }
         }
         __syncthreads();
-        bf16_t* dv_base = value_gradient + ((size_t)b * S * heads + h) * DV;
+        bf16_t* dv_base = value_gradient + ((size_t)b * S * kv_heads + h) * DV;
         for (int position = lane; position < 32 * (DV / 8); position += 64) {
             const int row = position / (DV / 8);
             const int chunk = position % (DV / 8);
@@ -534,13 +545,14 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         }
     } else {
         // ================= key wave: dP, dS, dK =================
-        const bf16_t* v_base = value + ((size_t)b * S * heads + h) * DV;
+        const bf16_t* v_base = value + ((size_t)b * S * kv_heads + h) * DV;
         bf16x8 vf[V_STEPS];   // B operand: column = key lq
         load_row_fragments<DV>(vf, v_base, v_stride, key_row, key_row < S, g);
         f32x16 dk_acc[DK_BLOCKS];
 #pragma unroll
         for (int d = 0; d < DK_BLOCKS; ++d) clear(dk_acc[d]);
-        unsigned char* ds_head = ds_blocks + (size_t)local_pair * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+        const size_t ds_head_bytes = (size_t)ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
+        unsigned char* ds_group = ds_blocks + (size_t)local_pair * sharing * ds_head_bytes;   // member m: + m * ds_head_bytes
         constexpr int DK_MFMAS = 4 * DK_BLOCKS;
         constexpr int DP_MFMAS = 2 * V_STEPS;
         static_assert(RING <= DK_MFMAS && RING <= DP_MFMAS, "a ring of fragments must fit each product");
@@ -562,7 +574,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         wait_vector_memory<0>();   // the V rows
         workgroup_barrier();       // tile 0 has landed
 
-        for (int index = 0; index < tiles; ++index) {
+        for (int index = 0; index < steps; ++index) {
             workgroup_barrier();   // A: every wave has left tile index - 1 (tile `index` landed a phase ago)
             const unsigned stage = (index % 3) * C::STAGE_BYTES;
             unsigned o_at[TileReads<C::O_ROW>::NAT], q_at[2][TileReads<C::Q_ROW>::TR];
@@ -599,8 +611,9 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 constexpr int PIECE = decltype(piece_tag)::value;
                 packed[PIECE] = *reinterpret_cast<const u32x4*>(lds + handover + PIECE * 1024);
             });
-            unsigned char* block =
-                ds_head + (size_t)ds_block_index(kb, query_tiles - 1 - index, query_tiles) * DS_BLOCK_BYTES;
+            const int member = index / tiles;
+            unsigned char* block = ds_group + member * ds_head_bytes +
+                (size_t)ds_block_index(kb, query_tiles - 1 - (index - member * tiles), query_tiles) * DS_BLOCK_BYTES;
             u32x4 dsf[2][2];
             static_for<0, 4>([&](auto piece_tag) {
                 constexpr int PIECE = decltype(piece_tag)::value;
@@ -647,7 +660,7 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
             }
         }
         __syncthreads();
-        bf16_t* dk_base = key_gradient + ((size_t)b * S * heads + h) * DQK;
+        bf16_t* dk_base = key_gradient + ((size_t)b * S * kv_heads + h) * DQK;
         for (int position = lane; position < 32 * (DQK / 8); position += 64) {
             const int row = position / (DQK / 8);
             const int chunk = position % (DQK / 8);
@@ -687,7 +700,8 @@ constexpr int DQ_THREADS = 512;
 template <int DQK>
 __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
     bf16_t* __restrict__ query_gradient, const unsigned char* __restrict__ ds_blocks, const bf16_t* __restrict__ key,
-    int sequence_length, int heads, int query_blocks, int key_blocks, int query_tiles, int first_pair, float scale) {
+    int sequence_length, int heads, int kv_heads, int query_blocks, int key_blocks, int query_tiles, int first_pair,
+    float scale) {
     using C = QueryGradConfig<DQK>;
     constexpr int WAVES = DQ_THREADS / 64;
 
@@ -711,8 +725,10 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
     const int column_half = (wave / 2) % 2;
     const int key_half = wave / 4;
 
-    const unsigned k_stride_bytes = (unsigned)heads * DQK * 2;
-    const unsigned char* k_base = reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * heads + h) * DQK);
+    // query head h reads key/value head h / (heads / kv_heads)
+    const unsigned k_stride_bytes = (unsigned)kv_heads * DQK * 2;
+    const unsigned char* k_base =
+        reinterpret_cast<const unsigned char*>(key + ((size_t)b * S * kv_heads + h / (heads / kv_heads)) * DQK);
     const unsigned char* ds_head = ds_blocks + (size_t)local_pair * ds_block_count(key_blocks, query_tiles) * DS_BLOCK_BYTES;
     const unsigned lds_base = lds_offset_of(lds);
 
@@ -918,25 +934,27 @@ struct BackwardShape {
     int key_blocks;
     int query_tiles;
     int query_blocks;
-    long long pairs;               // batch * heads
+    int sharing;                   // query heads per key/value head
+    long long pairs;               // batch * key/value heads: what the launches are cut by
     long long pairs_per_launch;
-    long long statistics_floats;   // all pairs
-    long long ds_floats;           // one chunk of pairs
+    long long statistics_floats;   // every (batch, query head)
+    long long ds_floats;           // one chunk of pairs, `sharing` query heads each
 };
 
-BackwardShape backward_shape(int batch_size, int sequence_length, int heads) {
+BackwardShape backward_shape(int batch_size, int sequence_length, int heads, int kv_heads) {
     BackwardShape shape;
     shape.key_blocks = (sequence_length + KBLOCK - 1) / KBLOCK;
     shape.query_tiles = (sequence_length + QTILE - 1) / QTILE;
     shape.query_blocks = shape.key_blocks;   // 128 queries per workgroup of the dQ pass
-    shape.pairs = (long long)batch_size * heads;
-    shape.statistics_floats = shape.pairs * shape.query_tiles * STAT_FLOATS;
-    const long long pair_bytes = (long long)ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_BYTES;
+    shape.sharing = heads / kv_heads;
+    shape.pairs = (long long)batch_size * kv_heads;
+    shape.statistics_floats = (long long)batch_size * heads * shape.query_tiles * STAT_FLOATS;
+    const long long pair_bytes = (long long)shape.sharing * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_BYTES;
     long long chunk = pair_bytes > 0 ? ds_budget_bytes() / pair_bytes : shape.pairs;
     if (chunk >= 8) chunk -= chunk % 8;
     if (chunk < 1) chunk = 1;
     shape.pairs_per_launch = chunk < shape.pairs ? chunk : shape.pairs;
-    shape.ds_floats = shape.pairs_per_launch * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_FLOATS;
+    shape.ds_floats = shape.pairs_per_launch * shape.sharing * ds_block_count(shape.key_blocks, shape.query_tiles) * DS_BLOCK_FLOATS;
     return shape;
 }
 
@@ -944,10 +962,10 @@ template <int DQK, int DV>
 void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value_gradient,
                      const bf16_t* output_gradient, const bf16_t* output, const float* logsumexp,
                      const bf16_t* query, const bf16_t* key, const bf16_t* value, float* workspace, int batch_size,
-                     int sequence_length, int heads, float scale, hipStream_t stream) {
+                     int sequence_length, int heads, int kv_heads, float scale, hipStream_t stream) {
     using KC = KeyValueGradConfig<DQK, DV>;
     using QC = QueryGradConfig<DQK>;
-    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads);
+    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads, kv_heads);
     const long long groups = (long long)batch_size * heads;
     const long long padded_rows = groups * shape.query_tiles * QTILE;
     if ((padded_rows + 15) / 16 > 0x7fffffffLL || groups * shape.key_blocks > 0x7fffffffLL) {
@@ -973,33 +991,42 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
         const long long count = std::min(shape.pairs_per_launch, shape.pairs - first);
         hipLaunchKernelGGL((attention_key_value_gradient_kernel<DQK, DV>), dim3((unsigned)(count * shape.key_blocks)),
                            dim3(KV_THREADS), KC::LDS_BYTES, stream, key_gradient, value_gradient, ds_blocks, statistics,
-                           output_gradient, query, key, value, sequence_length, heads, shape.key_blocks,
+                           output_gradient, query, key, value, sequence_length, heads, kv_heads, shape.key_blocks,
                            shape.query_tiles, (int)first, scale);
         HIP_CHECK(hipGetLastError());
-        // the next chunk's first pass overwrites the dS blocks: it follows this pass in the stream
-        hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>), dim3((unsigned)(count * shape.query_blocks)),
-                           dim3(DQ_THREADS), QC::LDS_BYTES, stream, query_gradient, ds_blocks, key, sequence_length,
-                           heads, shape.query_blocks, shape.key_blocks, shape.query_tiles, (int)first, scale);
+        // the next chunk's first pass overwrites the dS blocks: it follows this pass in the stream.  The query
+        // heads of the chunk's pairs are consecutive: count * sharing of them from first * sharing on.
+        hipLaunchKernelGGL((attention_query_gradient_kernel<DQK>),
+                           dim3((unsigned)(count * shape.sharing * shape.query_blocks)), dim3(DQ_THREADS), QC::LDS_BYTES,
+                           stream, query_gradient, ds_blocks, key, sequence_length, heads, kv_heads, shape.query_blocks,
+                           shape.key_blocks, shape.query_tiles, (int)(first * shape.sharing), scale);
         HIP_CHECK(hipGetLastError());
     }
 }
 
 }  // namespace
 
-std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads) {
-    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads);
+std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads, int kv_heads) {
+    if (kv_heads <= 0 || heads % kv_heads != 0) {
+        throw std::invalid_argument("attention backward: query heads must be a positive multiple of key/value heads");
+    }
+    const BackwardShape shape = backward_shape(batch_size, sequence_length, heads, kv_heads);
     return static_cast<std::size_t>(shape.statistics_floats + shape.ds_floats);
 }
 
 void attention_backward_dispatch(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value_gradient,
                                  const bf16_t* output_gradient, const bf16_t* output, const float* logsumexp,
                                  const bf16_t* query, const bf16_t* key, const bf16_t* value, float* workspace,
-                                 int batch_size, int sequence_length, int heads, int qk_head_size, int v_head_size,
-                                 float scale, hipStream_t stream) {
+                                 int batch_size, int sequence_length, int heads, int kv_heads, int qk_head_size,
+                                 int v_head_size, float scale, hipStream_t stream) {
+    if (kv_heads <= 0 || heads % kv_heads != 0) {
+        throw std::invalid_argument("attention backward: query heads must be a positive multiple of key/value heads");
+    }
 #define DSCUDA_BWD_CASE(DQK, DV)                                                                                   \
     if (qk_head_size == DQK && v_head_size == DV) {                                                                \
         launch_backward<DQK, DV>(query_gradient, key_gradient, value_gradient, output_gradient, output, logsumexp, \
-                                 query, key, value, workspace, batch_size, sequence_length, heads, scale, stream);  \
+                                 query, key, value, workspace, batch_size, sequence_length, heads, kv_heads, scale, \
+                                 stream);                                                                          \
         return;                                                                                                    \
     }
     DSCUDA_BWD_CASE(192, 128)

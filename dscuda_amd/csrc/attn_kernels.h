@@ -22,14 +22,14 @@ void attention_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const 
 // attn_bwd.hip -- recompute backward of the above for Hq == Hkv.  The fp32
 // workspace (attention_backward_workspace_elements floats) holds the per-row
 // statistics and the bf16 dS blocks handed from the dK/dV kernel to the dQ pass.
-std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads);
+std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads, int kv_heads);
 
 void attention_backward_dispatch(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
                                  __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
                                  const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
                                  const __hip_bfloat16* key, const __hip_bfloat16* value, float* workspace, int batch_size,
-                                 int sequence_length, int heads, int qk_head_size, int v_head_size, float scale,
-                                 hipStream_t stream);
+                                 int sequence_length, int heads, int kv_heads, int qk_head_size, int v_head_size,
+                                 float scale, hipStream_t stream);
 
 // rope.hip -- rotary position embedding, in place, on columns rope_offset .. rope_offset + rope_size - 1 of a
 // [B, S, H, width] bf16 tensor (interleaved pairs; positions: per-sequence start positions or nullptr for 0).

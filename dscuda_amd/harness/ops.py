@@ -49,6 +49,8 @@ class _Flash:
         lib = library("flash_attention")
         self.lib = lib
         self.forward = bind(lib, "dscuda_flash_forward", [P] * 5 + [I] * 5 + [F, P])
+        self.backward = bind(lib, "dscuda_flash_backward", [P] * 10 + [I] * 5 + [F, P])
+        self.backward_workspace = bind(lib, "dscuda_flash_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
 
 
 _mla = None
@@ -230,3 +232,24 @@ def rope_apply(tensor, rope_offset=0, rope_size=None, theta=10000.0, positions=N
     checked(lib.lib, "mla", lib.rope_apply(tensor.data_ptr(), positions.data_ptr() if positions is not None else None,
                                            b, s, h, w, rope_offset, rope_size, theta, stream()))
     return tensor
+
+
+def flash_backward_workspace(batch, seq, q_heads, kv_heads, dim, device="cuda"):
+    """fp32 workspace of the flash-attention backward (dscuda_flash_backward_workspace_elements)."""
+    elements = flash_library().backward_workspace(batch, seq, q_heads, kv_heads, dim)
+    return torch.empty(elements, device=device, dtype=torch.float32)
+
+
+def flash_backward(dout, out, lse, query, key, value, scale, workspace=None, grads=None):
+    """Causal (grouped-query) attention backward (dscuda_flash_backward) -> (dQ [B,T,Hq,D], dK, dV [B,T,Hkv,D])."""
+    _require_cuda(dout, out, lse, query, key, value)
+    b, t, hq, d = query.shape
+    hkv = key.shape[2]
+    lib = flash_library()
+    if workspace is None:
+        workspace = flash_backward_workspace(b, t, hq, hkv, d, query.device)
+    if grads is None:
+        grads = (torch.empty_like(query), torch.empty_like(key), torch.empty_like(value))
+    checked(lib.lib, "flash", lib.backward(
+        *pointers((*grads, dout, out, lse, query, key, value, workspace)), b, t, hq, hkv, d, scale, stream()))
+    return grads

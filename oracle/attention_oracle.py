@@ -103,21 +103,28 @@ def attention_backward(dout, out, lse, query, key, value, scale, heads=None):
     Same recompute structure as reference/python/mla.py:42-57 with per-head
     K/V:  P = exp(S - LSE);  dP = dO V^T;  delta = sum_c dO*O;
     dS = P (dP - delta) scale;  dQ = dS K;  dK = dS^T Q;  dV = P^T dO.
-    Only MHA (Hq == Hkv) is needed by this path.  Returns unrounded
-    (dQ, dK, dV) for the selected heads.
+    Grouped-query heads (Hq a multiple of Hkv, query head h reads kv head
+    h // (Hq/Hkv) as in the forward): dK and dV of a kv head are the sums over
+    the query heads of its group; ``heads`` must then be None.  Returns
+    unrounded (dQ [B,S,heads,Dqk], dK [B,S,Hkv or heads,Dqk], dV likewise).
     """
     dout, out, query, key, value = map(_compute, (dout, out, query, key, value))
     lse = _compute(lse)
     batch, seq, q_heads, _ = query.shape
-    assert key.shape[2] == q_heads, "backward oracle covers the MHA form"
+    kv_heads = key.shape[2]
+    assert q_heads % kv_heads == 0, "query heads must be a multiple of key/value heads"
+    group = q_heads // kv_heads
+    assert group == 1 or heads is None, "a head subset is only defined for the MHA form"
     heads = list(range(q_heads)) if heads is None else list(heads)
     mask = torch.ones(seq, seq, dtype=torch.bool).tril()
     dq = torch.empty(batch, seq, len(heads), query.shape[-1], dtype=query.dtype)
-    dk = torch.empty_like(dq)
-    dv = torch.empty(batch, seq, len(heads), value.shape[-1], dtype=query.dtype)
+    kv_count = len(heads) if group == 1 else kv_heads
+    dk = torch.zeros(batch, seq, kv_count, query.shape[-1], dtype=query.dtype)
+    dv = torch.zeros(batch, seq, kv_count, value.shape[-1], dtype=query.dtype)
     for b in range(batch):
         for i, h in enumerate(heads):
-            q, k, v = query[b, :, h], key[b, :, h], value[b, :, h]
+            shared = h // group
+            q, k, v = query[b, :, h], key[b, :, shared], value[b, :, shared]
             do, o = dout[b, :, h], out[b, :, h]
             scores = (q @ k.transpose(0, 1) * scale).masked_fill(~mask, -math.inf)
             prob = (scores - lse[b, h][:, None]).exp()
@@ -125,8 +132,9 @@ def attention_backward(dout, out, lse, query, key, value, scale, heads=None):
             delta = (do * o).sum(-1, keepdim=True)
             dscore = prob * (dprob - delta) * scale
             dq[b, :, i] = dscore @ k
-            dk[b, :, i] = dscore.transpose(0, 1) @ q
-            dv[b, :, i] = prob.transpose(0, 1) @ do
+            target = i if group == 1 else shared
+            dk[b, :, target] += dscore.transpose(0, 1) @ q
+            dv[b, :, target] += prob.transpose(0, 1) @ do
     return dq, dk, dv
 
 

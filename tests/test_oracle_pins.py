@@ -107,6 +107,30 @@ def test_backward_matches_autograd(dqk, dv):
         assert (a - r).abs().max() < 1e-10, name
 
 
+@pytest.mark.parametrize("q_heads,kv_heads", [(4, 2), (8, 1), (6, 3)])
+def test_grouped_query_backward_matches_autograd(q_heads, kv_heads):
+    """dK and dV of a shared key/value head are the sums over the query heads that read it: autograd through an
+    explicit repeat_interleave of K and V (the reference's own GQA formulation, benchmarks/flash_attention.py:72-74)
+    says so, and a wrong head mapping (h % Hkv instead of h // group) or a missing term fails it."""
+    b, s, d = 2, 29, 16
+    q = _rand((b, s, q_heads, d), 50, 0.5, torch.float64).requires_grad_()
+    k = _rand((b, s, kv_heads, d), 51, 0.5, torch.float64).requires_grad_()
+    v = _rand((b, s, kv_heads, d), 52, 0.5, torch.float64).requires_grad_()
+    dout = _rand((b, s, q_heads, d), 53, 1.0, torch.float64)
+    scale = d ** -0.5
+    group = q_heads // kv_heads
+    mask = torch.ones(s, s, dtype=torch.bool).tril()
+    scores = torch.einsum("bqhd,bkhd->bhqk", q, k.repeat_interleave(group, dim=2)) * scale
+    out = torch.einsum("bhqk,bkhd->bqhd", scores.masked_fill(~mask, -math.inf).softmax(-1), v.repeat_interleave(group, dim=2))
+    rq, rk, rv = torch.autograd.grad(out, (q, k, v), dout)
+    saved, lse = oracle.causal_attention_forward(q.detach(), k.detach(), v.detach(), scale)
+    assert (saved - out.detach()).abs().max() < 1e-12
+    dq, dk, dv = oracle.attention_backward(dout, saved, lse, q.detach(), k.detach(), v.detach(), scale)
+    assert dk.shape == k.shape and dv.shape == v.shape
+    for name, a, r in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        assert (a - r).abs().max() < 1e-10, name
+
+
 def test_backward_finite_differences():
     b, s, h, dqk, dv = 1, 7, 1, 4, 3
     q, k, v = (_rand(shape, seed, 1.0, torch.float64) for seed, shape in
