@@ -361,9 +361,9 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
     q_requests.init(q_stride_bytes, wave % 4, lane);
     o_requests.init(o_stride_bytes, wave % 4, lane);
     constexpr int REQUEST_LOADS = TileRequests<C::Q_ROW, 4>::LOADS + TileRequests<C::O_ROW, 4>::LOADS + 1;
-    auto request_tile = [&](int index) {
-        const int member = index / tiles;
-        const int tile = query_tiles - 1 - (index - member * tiles);
+    // step `index` = tile-step `local` of member `member` (the callers keep the three in step: no division here)
+    auto request_tile = [&](int index, int member, int local) {
+        const int tile = query_tiles - 1 - local;
         const int row0 = tile * QTILE;
         const int row_limit = S - 1 - row0;
         const unsigned target = lds_base + (index % 3) * C::STAGE_BYTES;
@@ -389,9 +389,9 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
 
     if (!key_wave) {
         // ================= value wave: S, P, dV =================
-        request_tile(0);
+        request_tile(0, 0, 0);
         if (steps > 1) {
-            request_tile(1);
+            if (tiles > 1) request_tile(1, 0, 1); else request_tile(1, 1, 0);
         }
         const bf16_t* k_base = key + ((size_t)b * S * kv_heads + h) * DQK;
         bf16x8 kf[QK_STEPS];   // B operand: column = key lq
@@ -446,16 +446,21 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         // matrix work.  MASKED applies the causal mask: it can only bite in the two
         // tiles at the diagonal, the last ones of the walk (and all the tiles a ragged
         // last block has).
-        auto value_tile = [&](auto masked_tag, int index) {
+        auto value_tile = [&](auto masked_tag, int index, int member, int local) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             workgroup_barrier();   // A: every wave has left tile index - 1
             if (index + 2 < steps) {
-                request_tile(index + 2);
+                int ahead_member = member, ahead_local = local + 2;
+                while (ahead_local >= tiles) {
+                    ahead_local -= tiles;
+                    ++ahead_member;
+                }
+                request_tile(index + 2, ahead_member, ahead_local);
             }
             // P: lane holds key lq and queries 32*qb + 8*i4 + 4*g + e.  A query with
             // local index below `threshold` lies before this lane's key.
             u32x4 pf[2][2];
-            const int threshold = key_row - 4 * g - (query_tiles - 1 - index % tiles) * QTILE;
+            const int threshold = key_row - 4 * g - (query_tiles - 1 - local) * QTILE;
             static_for<0, 2>([&](auto qb_tag) {
                 constexpr int QB = decltype(qb_tag)::value;
                 static_for<0, 4>([&](auto i4_tag) {
@@ -515,10 +520,10 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         score_stream(0);
         for (int member = 0, index = 0; member < sharing; ++member) {
             for (int local = 0; local < tiles - 2; ++local, ++index) {
-                value_tile(std::false_type{}, index);
+                value_tile(std::false_type{}, index, member, local);
             }
             for (int local = max(tiles - 2, 0); local < tiles; ++local, ++index) {
-                value_tile(std::true_type{}, index);
+                value_tile(std::true_type{}, index, member, local);
             }
         }
 
@@ -574,7 +579,11 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
         wait_vector_memory<0>();   // the V rows
         workgroup_barrier();       // tile 0 has landed
 
-        for (int index = 0; index < steps; ++index) {
+        for (int index = 0, member = 0, local = 0; index < steps; ++index, ++local) {
+            if (local == tiles) {
+                local = 0;
+                ++member;
+            }
             workgroup_barrier();   // A: every wave has left tile index - 1 (tile `index` landed a phase ago)
             const unsigned stage = (index % 3) * C::STAGE_BYTES;
             unsigned o_at[TileReads<C::O_ROW>::NAT], q_at[2][TileReads<C::Q_ROW>::TR];
@@ -611,9 +620,8 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                 constexpr int PIECE = decltype(piece_tag)::value;
                 packed[PIECE] = *reinterpret_cast<const u32x4*>(lds + handover + PIECE * 1024);
             });
-            const int member = index / tiles;
             unsigned char* block = ds_group + member * ds_head_bytes +
-                (size_t)ds_block_index(kb, query_tiles - 1 - (index - member * tiles), query_tiles) * DS_BLOCK_BYTES;
+                (size_t)ds_block_index(kb, query_tiles - 1 - local, query_tiles) * DS_BLOCK_BYTES;
             u32x4 dsf[2][2];
             static_for<0, 4>([&](auto piece_tag) {
                 constexpr int PIECE = decltype(piece_tag)::value;

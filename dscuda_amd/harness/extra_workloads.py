@@ -49,7 +49,8 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
     results["mla_decode_B64_H128"] = {
         "us": ms * 1000.0, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
         "bytes": nbytes, "total_tokens": total, "tflops": configs.decode_flops(total, h) / ms / 1e9,
-        "kernels": "mla_decode_split + mla_decode_combine"}
+        "kernels": "mla_decode_plan + mla_decode_split (fast, then the rescaling pass, which finds nothing to do) + "
+                   "mla_decode_merge"}
     del paged, workspace
 
     # long context: MLA prefill forward + backward, B=1 S=16384 H=128.  Timing does not depend on the
@@ -75,6 +76,32 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
                                            "workspace_gib": workspace.numel() * 4 / 2 ** 30,
                                            "data": "synthetic, GPU generator"}
     del lq, lk, lv, ldo, lout, llse, grads, workspace
+
+    # the reference's own prefill API (absorbed form: 576-wide scores against one shared latent head, 512-wide
+    # output), forward and backward, at the sequence length and head count of the headline workload
+    try:
+        tokens = 4096
+        ql, qr = draw((1, tokens, heads, 512), 0.25), draw((1, tokens, heads, 64), 0.25)
+        latent, kr = draw((1, tokens, 512), 0.25), draw((1, tokens, 64), 0.25)
+        dout_a = draw((1, tokens, heads, 512), 0.2)
+        aout = torch.empty(1, tokens, heads, 512, device=device, dtype=torch.bfloat16)
+        alse = torch.empty(1, heads, tokens, device=device, dtype=torch.float32)
+        ascale = configs.c_float(576 ** -0.5)
+        ms, _ = event_time_ms(lambda: ops.mla_forward(ql, qr, latent, kr, ascale, aout, alse), 10, 3)
+        pairs = heads * tokens * tokens / 2
+        flops = pairs * 2 * (576 + 512)
+        results["mla_absorbed_forward_T4096_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
+                                                      "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,
+                                                      "entry": "dscuda_mla_forward", "data": "synthetic, GPU generator"}
+        agrads = tuple(torch.empty_like(x) for x in (ql, qr, latent, kr))
+        ms, _ = event_time_ms(lambda: ops.mla_backward(dout_a, aout, alse, ql, qr, latent, kr, ascale, agrads), 5, 2)
+        flops = pairs * 2 * (3 * 576 + 2 * 512)   # S, dP, dV (512), dQ and dK (576): the five products
+        results["mla_absorbed_backward_T4096_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
+                                                       "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,
+                                                       "entry": "dscuda_mla_backward", "data": "synthetic, GPU generator"}
+        del ql, qr, latent, kr, dout_a, aout, alse, agrads
+    except Exception as error:
+        results["mla_absorbed_T4096_H128"] = {"error": str(error)}
 
     # for scale only: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this chip with random
     # operands, timed the same way; a plain GEMM is the practical ceiling of any MFMA-bound kernel here

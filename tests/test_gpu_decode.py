@@ -236,7 +236,7 @@ def test_decode_workload_4(cuda):
 
 # ---- absorbed causal prefill forward (dscuda_mla_forward) ----------------------
 
-@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 200, 128)])
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 200, 128), (1, 1024, 16)])
 def test_absorbed_forward(cuda, batch, tokens, heads):
     ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
     announce("mla_forward", dict(B=batch, T=tokens, H=heads))
