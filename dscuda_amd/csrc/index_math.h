@@ -234,8 +234,7 @@ DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total, int ranges, int bef
 //     [4] ranges the list is cut into (<= workgroups)
 //     [5 .. 5+B]        inclusive prefix of positions per sequence (B + 1 entries)
 //     [.. + W]          first sequence whose positions reach past the start of each range
-//     [.. + G*B]        one flag per (head group, sequence): some part needs the rescaling pass
-// with G = head groups of 128 heads.  The flags are zero between calls.
+// It is read-only once built.
 constexpr int PLAN_TOTAL = 0;
 constexpr int PLAN_WORKGROUPS = 1;
 constexpr int PLAN_OVERHEAD = 2;
@@ -245,11 +244,8 @@ constexpr int PLAN_HEADER = 5;
 
 DSCUDA_HOST_DEVICE inline long long plan_prefix_at() { return PLAN_HEADER; }
 DSCUDA_HOST_DEVICE inline long long plan_first_sequence_at(int batch) { return PLAN_HEADER + (long long)batch + 1; }
-DSCUDA_HOST_DEVICE inline long long plan_flags_at(int batch, int workgroups) {
+DSCUDA_HOST_DEVICE inline long long plan_elements(int batch, int workgroups) {
     return plan_first_sequence_at(batch) + workgroups;
-}
-DSCUDA_HOST_DEVICE inline long long plan_elements(int batch, int workgroups, int head_groups) {
-    return plan_flags_at(batch, workgroups) + (long long)head_groups * batch;
 }
 
 // The caller's workspace holds batch * heads * splits * (rank + 2) floats.  A
@@ -277,8 +273,8 @@ DSCUDA_HOST_DEVICE inline DecodeLayout decode_layout(int batch, int heads, int s
     const long long padded_rows = (long long)((heads + 31) / 32) * 32;
     layout.slot_floats = padded_rows * (rank / 2 + 2);
     const long long workspace = (long long)batch * heads * splits * (rank + 2);
-    // (W + batch) * slot_floats + plan_elements(batch, W, groups) <= workspace, W <= compute_units
-    const long long fixed = (long long)batch * layout.slot_floats + plan_elements(batch, 0, layout.head_groups);
+    // (W + batch) * slot_floats + plan_elements(batch, W) <= workspace, W <= compute_units
+    const long long fixed = (long long)batch * layout.slot_floats + plan_elements(batch, 0);
     long long cutting = workspace >= fixed ? (workspace - fixed) / (layout.slot_floats + 1) : 0;
     if (cutting > compute_units) cutting = compute_units;
     layout.whole_sequences = (splits <= 1 || cutting < 2) ? 1 : 0;
@@ -290,7 +286,7 @@ DSCUDA_HOST_DEVICE inline DecodeLayout decode_layout(int batch, int heads, int s
         layout.slots = (long long)layout.workgroups + batch;
     }
     layout.plan_offset = layout.slots * layout.slot_floats;
-    layout.plan_ints = plan_elements(batch, layout.workgroups, layout.head_groups);
+    layout.plan_ints = plan_elements(batch, layout.workgroups);
     return layout;
 }
 

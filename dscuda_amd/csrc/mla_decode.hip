@@ -821,11 +821,39 @@ __device__ __forceinline__ void mask_unit_scores(f32x16& scores, int key0, int t
     }
 }
 
+// A row's scores have outrun its reference by more than FAST_LIMIT: the reference of every such row of the
+// wave moves to FAST_HEADROOM above the row's new maximum, and what the row has accumulated is scaled to
+// match.  Next to never taken; when it is, some wave pays 256 multiplications per lane once.  The
+// accumulators are scaled where they are (accumulation registers, read and written back by one asm
+// statement each): any formulation that lets the compiler see a conditional assignment to them makes it
+// copy all 256 at the join, on the path that never takes the branch as well.  The output MFMAs that wrote
+// them were issued a whole unit ago; the wait states at the top cover the distance all the same.
+__device__ __forceinline__ void raise_reference(RowState& state, float& offset, float unit_max) {
+    const float raised = unit_max - offset > FAST_LIMIT ? unit_max + FAST_HEADROOM : offset;
+    const float factor = __builtin_amdgcn_exp2f(offset - raised);   // 1 for the rows that stay
+    offset = raised;
+    state.reference = raised;
+    state.row_sum *= factor;
+    asm volatile("s_nop 15\n\ts_nop 3");
+#pragma unroll
+    for (int d = 0; d < DBLOCKS; ++d) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float value = state.o[d][i];
+            float moved;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(value), "=&v"(moved)
+                         : "v"(factor));
+            state.o[d][i] = value;
+        }
+    }
+}
+
 // One step of the stream: the probabilities of the unit at `current` (its scores are in
 // `scores`), the scores of the unit at `next` into `next_scores` if HAS_NEXT, the output
 // update with `current`, and the requests for `request`.
 template <bool HAS_NEXT>
-__device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& scores, f32x16& next_scores,
+__device__ __forceinline__ void unit_step(RowState& state, f32x16& scores, f32x16& next_scores,
                                           const bf16x8 (&qf)[KSTEPS], const UnitReads& reads,
                                           const unsigned char* current, const unsigned char* next, int key0, int tokens,
                                           float c, const UnitSource& request, const FullUnitOffsets& offsets,
@@ -850,7 +878,7 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
 
     float unit_max;
     u32x4 probabilities[2];
-    const float offset = state.reference;
+    float offset = state.reference;
     // The softmax in 33 pieces of one to three instructions, spread over the score MFMAs.  Plain
     // arithmetic has no place of its own in the instruction order (the compiler would gather all of
     // it next to its last use, behind the score MFMAs); passing a piece's inputs and results through
@@ -866,7 +894,9 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
             here(unit_max);
         } else if constexpr (I == 8) {
             unit_max = half_wave_max(unit_max) * c;
-            risk = risk || (unit_max - offset > FAST_LIMIT);
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(unit_max - offset > FAST_LIMIT) != 0, 0)) {
+                raise_reference(state, offset, unit_max);
+            }
         } else if constexpr (I < 25) {
             constexpr int E = I - 9;
             float score = scores[E];
@@ -919,9 +949,8 @@ __device__ __forceinline__ void unit_step(RowState& state, bool& risk, f32x16& s
 
 // Walk tiles [tile_begin, tile_end) of one sequence of the decode cache for the 128 heads of
 // this workgroup with the unit stream, from cleared accumulators.  Every lane's row sees all
-// `tokens` keys.  Returns whether any row of the workgroup came too close to the limit of the
-// fixed softmax reference (workgroup-uniform): the caller then discards the result.
-__device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_row, bool valid, unsigned char* lds,
+// `tokens` keys (see raise_reference for what happens when a row outruns its softmax reference).
+__device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_row, bool valid, unsigned char* lds,
                                            const KeyStream& keys, int tile_begin, int tile_end, int tokens, float c,
                                            int tid, bool cold) {
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -944,7 +973,6 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
     load_query(qf, query_row, query_row + RANK, valid, (tid % 64) / 32);
     if (!cold) issue_unit(third, offsets, keys, wave);
     reset(state);
-    bool risk = false;
     UnitReads reads;
     reads.init(fresh_lane_id());
     auto slot_of = [&](int unit) { return lds + ((unsigned)unit % UNIT_SLOTS) * UNIT_BYTES; };
@@ -979,16 +1007,15 @@ __device__ __forceinline__ bool walk_units(RowState& state, const bf16_t* query_
     int unit = unit_begin;
     for (; unit + 1 < unit_end; ++unit) {
         synchronise(unit);
-        unit_step<true>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
+        unit_step<true>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
                         cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
         // the next unit's scores take the place of this unit's (eight moves against a stream of 68 MFMAs)
         move_scores(scores_a, scores_b);
     }
     UnitSource nothing = {};
-    unit_step<false>(state, risk, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c, nothing,
+    unit_step<false>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c, nothing,
                      offsets, keys, wave);
     workgroup_barrier();   // the slots are free: the caller stages its results through them
-    return __syncthreads_or(risk) != 0;
 }
 
 __device__ __forceinline__ int tiles_of(int length) {
@@ -1008,19 +1035,17 @@ using index_math::PLAN_WORKGROUPS;
 
 // One workgroup turns the lengths into the plan (index_math.h): the prefix of positions
 // (tiles plus the per-sequence overhead when sequences are cut), the first sequence of
-// each of the `workgroups` ranges, and cleared flags.  Any batch size: the scan carries
-// over chunks of THREADS lengths.
+// each of the `workgroups` ranges.  Any batch size: the scan carries over chunks of
+// THREADS lengths.
 __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restrict__ plan,
                                                                   const int* __restrict__ cache_lengths, int batch_size,
-                                                                  int workgroups, int whole_sequences,
-                                                                  int head_groups) {
+                                                                  int workgroups, int whole_sequences) {
     __shared__ int wave_totals[THREADS / 64];
     const int tid = threadIdx.x;
     const int lane = tid % 64;
     const int wave = tid / 64;
     int* prefix = plan + index_math::plan_prefix_at();
     int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
-    int* flags = plan + index_math::plan_flags_at(batch_size, workgroups);
 
     const int overhead = whole_sequences ? 0 : index_math::SEGMENT_OVERHEAD;
     int carry = 0;
@@ -1055,7 +1080,6 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
         plan[PLAN_RANGES] = ranges;
         plan[PLAN_WHOLE] = whole_sequences;
     }
-    for (int index = tid; index < head_groups * batch_size; index += THREADS) flags[index] = 0;
     __syncthreads();   // the prefix written above is read back below
     for (int w = tid; w < workgroups; w += THREADS) {
         int sequence = w;
@@ -1077,19 +1101,11 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
     }
 }
 
-// SAFE == false is the kernel that does the work.  A segment in which some row outran
-// the fixed softmax reference (see process_tile) raises its sequence's flag instead of
-// trusting its results; the SAFE == true instantiation, launched right after, repeats
-// every segment of the flagged sequences with the rescaling variant and returns at once
-// everywhere else.  Two kernels rather than two paths in one keep the register
-// allocation of the hot loop free of the slow path's pressure.  The flags are cleared
-// by whoever reads them last: the merge kernel, or this kernel's rescaling pass when
-// sequences are not cut (then nothing is merged).
+// The decode kernel: every workgroup walks its range of the work list (see index_math.h).
 //
 // Workspace: slot workgroup + sequence holds, for a segment that is only part of its
 // sequence, the bf16 accumulators of every wave (store_partial order, 32 KB per wave,
 // waves numbered over all head groups) followed by (reference, sum) per head.
-template <bool SAFE>
 __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query,
     const bf16_t* __restrict__ paged_kv_cache, const int* __restrict__ block_table,
@@ -1116,7 +1132,6 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     const bool whole_sequences = plan[PLAN_WHOLE] != 0;
     const int* prefix = plan + index_math::plan_prefix_at();
     const int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
-    int* flags = plan + index_math::plan_flags_at(batch_size, workgroups) + (size_t)head_group * batch_size;
 
     int range_begin, range_end;
     if (whole_sequences) {
@@ -1152,7 +1167,7 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         int tile_begin, tile_end;
         index_math::tiles_in_positions(position, segment_end, sequence_begin, overhead, tile_begin, tile_end);
         // no tiles: the range ends among the positions that stand for the sequence's overhead
-        if (tile_end <= tile_begin || (SAFE && flags[sequence] == 0)) {   // ... or finished by the fast kernel
+        if (tile_end <= tile_begin) {
             position = segment_end;
             ++sequence;
             continue;
@@ -1168,18 +1183,10 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.rope_stride = WIDTH;
         keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
         keys.page_size = page_size;
-        bool risk;
-        if constexpr (SAFE) {
-            risk = walk_rows<true>(state, query_row, query_row + RANK, valid, lds, keys, tile_begin, tile_end, tokens, tokens,
-                                   c, tid);
-        } else {
-            risk = walk_units(state, query_row, valid, lds, keys, tile_begin, tile_end, tokens, c, tid, position == range_begin);
-        }
+        walk_units(state, query_row, valid, lds, keys, tile_begin, tile_end, tokens, c, tid, position == range_begin);
         const float total_sum = half_wave_sum(state.row_sum);
 
-        if (!SAFE && risk) {
-            if (tid == 0) flags[sequence] = 1;   // several workgroups may say so: they all write the same value
-        } else if (whole) {
+        if (whole) {
             if (wave_active) {
                 if (valid && g == 0) {
                     logsumexp[(size_t)sequence * heads + head] = (state.reference + __builtin_amdgcn_logf(total_sum)) * LN2;
@@ -1189,7 +1196,6 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
                     return h < heads ? output + ((size_t)sequence * heads + h) * RANK : nullptr;
                 });
             }
-            if (SAFE && whole_sequences && tid == 0) flags[sequence] = 0;   // nobody else reads it (see above)
         } else if (wave_active) {
             float* slot = workspace + ((size_t)workgroup + sequence) * slot_floats;
             if (valid && g == 0) {
@@ -1231,10 +1237,6 @@ __global__ __launch_bounds__(64) void mla_decode_merge_kernel(bf16_t* __restrict
     const int workgroups = plan[PLAN_WORKGROUPS];
     const int overhead = plan[PLAN_OVERHEAD];
     const int* prefix = plan + index_math::plan_prefix_at();
-    if (quarter == 0 && wave_block % (ROWS / 32) == 0 && lane == 0) {
-        // this sequence's flag of the head group has been read by everybody who needed it
-        plan[index_math::plan_flags_at(batch_size, workgroups) + (size_t)(wave_block / (ROWS / 32)) * batch_size + sequence] = 0;
-    }
     const int sequence_begin = prefix[sequence];
     const int sequence_end = prefix[sequence + 1];
     if (sequence_end <= sequence_begin) return;   // no tiles: nothing was computed for it
@@ -1393,7 +1395,7 @@ void mla_decode_plan_dispatch(int* plan, const int* cache_lengths, int batch_siz
                               hipStream_t stream) {
     const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
     hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
-                       layout.workgroups, layout.whole_sequences, layout.head_groups);
+                       layout.workgroups, layout.whole_sequences);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -1406,8 +1408,7 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
     }
     static thread_local bool prepared = false;
     if (!prepared) {
-        allow_large_lds(mla_decode_split_kernel<false>);
-        allow_large_lds(mla_decode_split_kernel<true>);
+        allow_large_lds(mla_decode_split_kernel);
         prepared = true;
     }
     // How the caller's B*H*splits*(C+2) floats are used: index_math::decode_layout.
@@ -1416,16 +1417,12 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
         // no plan from the caller: this call's own, behind the partial-result slots
         plan = reinterpret_cast<int*>(workspace + layout.plan_offset);
         hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
-                           layout.workgroups, layout.whole_sequences, layout.head_groups);
+                           layout.workgroups, layout.whole_sequences);
         HIP_CHECK(hipGetLastError());
     }
     const int padded_rows = (heads + 31) / 32 * 32;
     const dim3 grid(layout.workgroups, layout.head_groups);
-    hipLaunchKernelGGL(mla_decode_split_kernel<false>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
-                       paged_kv_cache, block_table, cache_lengths, workspace, plan, batch_size, heads, page_size,
-                       pages_per_sequence, layout.slot_floats, padded_rows, scale);
-    HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(mla_decode_split_kernel<true>, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
+    hipLaunchKernelGGL(mla_decode_split_kernel, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
                        paged_kv_cache, block_table, cache_lengths, workspace, plan, batch_size, heads, page_size,
                        pages_per_sequence, layout.slot_floats, padded_rows, scale);
     HIP_CHECK(hipGetLastError());

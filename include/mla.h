@@ -160,7 +160,7 @@ constexpr std::size_t MLA_DECODE_STATIC_SCRATCH_BYTES = std::size_t(64) << 20;
 // mla_decode_forward_cuda for callers that cannot allocate or pass a workspace
 // (code under HIP graph capture, tight serving loops, harnesses that forbid
 // hipMalloc).  No counterpart in the reference.  Same arguments without the
-// workspace: the partial results and flags live in a fixed array inside the
+// workspace: the partial results and the plan live in a fixed array inside the
 // library, and the call performs no allocation of any kind.  Sizes for which
 // batch*heads*splits*(kv_rank+2) floats exceed MLA_DECODE_STATIC_SCRATCH_BYTES
 // are rejected with std::invalid_argument (lower `splits`: the result does not

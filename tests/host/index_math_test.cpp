@@ -346,7 +346,7 @@ void check_decode_layout() {
                            batch, heads, splits, layout.workgroups);
                     EXPECT(layout.plan_offset + layout.plan_ints <= workspace, "B %d H %d splits %d CUs %d: plan ends at %lld of %lld floats",
                            batch, heads, splits, compute_units, layout.plan_offset + layout.plan_ints, workspace);
-                    EXPECT(layout.plan_ints == plan_elements(batch, layout.workgroups, groups), "B %d H %d splits %d", batch, heads, splits);
+                    EXPECT(layout.plan_ints == plan_elements(batch, layout.workgroups), "B %d H %d splits %d", batch, heads, splits);
                     // a slot holds 32 KB of bf16 accumulators per wave of 32 heads and two floats per head
                     const long long waves = (heads + 31) / 32;
                     EXPECT(layout.slot_floats * 4 == waves * 32768 + waves * 32 * 8, "H %d slot of %lld floats", heads, layout.slot_floats);
@@ -358,15 +358,14 @@ void check_decode_layout() {
                         EXPECT(layout.plan_offset == layout.slots * layout.slot_floats, "B %d splits %d", batch, splits);
                         // as many workgroups as fit: one more would not
                         if (layout.workgroups < compute_units) {
-                            const long long more = (layout.slots + 1) * layout.slot_floats + plan_elements(batch, layout.workgroups + 1, groups);
+                            const long long more = (layout.slots + 1) * layout.slot_floats + plan_elements(batch, layout.workgroups + 1);
                             EXPECT(more > workspace, "B %d H %d splits %d: %d workgroups but %d would fit", batch, heads, splits,
                                    layout.workgroups, layout.workgroups + 1);
                         }
                     }
-                    // plan: header, prefix, first sequences, flags follow one another
+                    // plan: header, prefix, first sequences follow one another
                     EXPECT(plan_prefix_at() == PLAN_HEADER && plan_first_sequence_at(batch) == PLAN_HEADER + batch + 1 &&
-                               plan_flags_at(batch, layout.workgroups) == plan_first_sequence_at(batch) + layout.workgroups &&
-                               plan_elements(batch, layout.workgroups, groups) == plan_flags_at(batch, layout.workgroups) + (long long)groups * batch,
+                               plan_elements(batch, layout.workgroups) == plan_first_sequence_at(batch) + layout.workgroups,
                            "plan parts B %d", batch);
                 }
             }

@@ -89,23 +89,27 @@ def test_decode_many_heads(cuda):
     _decode_case(cuda, 2, 200, 160, [200, 77], seed=10)
 
 
-@pytest.mark.parametrize("splits,tokens,lengths,hot", [(1, 300, [300, 250], (200, 260)),
-                                                       (8, 1500, [1500, 1250], (1000, 1100))])
-def test_decode_large_scores_take_the_rescaling_path(cuda, splits, tokens, lengths, hot):
-    """Scores that outgrow the first tile's maximum by far more than the fast
-    path's head room: late keys are aligned with the query, early ones are not.
-    In the second case five workgroups share the 44 tiles of the two sequences, nine to
-    a range: the ranges that meet the hot keys after an ordinary first tile flag their
-    sequence, and the rescaling pass redoes every part of it and merges them again."""
+@pytest.mark.parametrize("splits,tokens,lengths,hot", [
+    (1, 300, [300, 250], [(200, 260, 4.0)]),
+    (8, 1500, [1500, 1250], [(1000, 1100, 4.0)]),
+    (8, 1500, [1500, 1250], [(600, 650, 1.0), (1000, 1100, 4.0)]),   # the reference is raised twice in one walk
+    (1, 700, [700, 433], [(45, 50, 0.5), (300, 301, 2.0), (690, 700, 8.0)]),   # in the middle of units, thrice
+])
+def test_decode_large_scores_raise_the_reference(cuda, splits, tokens, lengths, hot):
+    """Scores that outgrow the maximum of the first keys by far more than the head room the fixed softmax
+    reference leaves (2^120): late keys are aligned with the query, early ones are not.  The walk that meets
+    them raises the reference of the rows concerned and scales what they had accumulated; in the cut cases
+    several workgroups share the tiles of the two sequences and the parts merge as usual."""
     batch, heads = 2, 8
     g = torch.Generator().manual_seed(12)
     query = (torch.randn(batch, 1, heads, 576, generator=g)).bfloat16()
     cache = (torch.randn(batch, tokens, 576, generator=g) * 0.05).bfloat16()
-    cache[:, hot[0]:hot[1]] = (query[:, 0, :1].float() * 4.0).bfloat16()  # huge positive scores late in the stream
+    for first, last, factor in hot:   # huge positive scores late in the stream
+        cache[:, first:last] = (query[:, 0, :1].float() * factor).bfloat16()
     lengths = torch.tensor(lengths, dtype=torch.int32)
     paged, table = configs.pack_cache(cache, 64)
     scale = 1.0
-    announce("mla_decode rescaling path", dict(splits=splits))
+    announce("mla_decode raised reference", dict(splits=splits, hot=hot))
     out, lse = ops.mla_decode(query.to(cuda), paged.to(cuda), table.to(cuda), lengths.to(cuda), scale, splits=splits)
     torch.cuda.synchronize()
     expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths, scale)
@@ -142,9 +146,9 @@ def test_decode_with_a_reused_plan_equals_the_plain_call(cuda):
     assert_close_lse("LSE", expected_lse, oracle_lse)
 
 
-def test_decode_plan_after_a_rescaled_call_is_clean(cuda):
-    """A call that needed the rescaling pass leaves the plan's tickets and flags at zero: the next call over the
-    same plan with ordinary data gives the ordinary result."""
+def test_decode_plan_is_read_only(cuda):
+    """A plan is not written by the calls that use it, whatever their data (also data that makes rows outrun their
+    softmax reference): the next call over the same plan with ordinary data gives the ordinary result."""
     batch, tokens, heads = 2, 1500, 8
     g = torch.Generator().manual_seed(43)
     query = torch.randn(batch, 1, heads, 576, generator=g).bfloat16()
@@ -155,10 +159,13 @@ def test_decode_plan_after_a_rescaled_call_is_clean(cuda):
     paged, table = configs.pack_cache(cache, 64)
     hot_paged, _ = configs.pack_cache(hot, 64)
     plan = ops.mla_decode_plan(lengths.to(cuda), heads, 8)
-    announce("mla_decode plan reuse after rescaling")
+    torch.cuda.synchronize()
+    before = plan.clone()
+    announce("mla_decode plan reuse")
     ops.mla_decode_planned(query.to(cuda), hot_paged.to(cuda), table.to(cuda), lengths.to(cuda), plan, 1.0, splits=8)
     out, lse = ops.mla_decode_planned(query.to(cuda), paged.to(cuda), table.to(cuda), lengths.to(cuda), plan, 1.0, splits=8)
     torch.cuda.synchronize()
+    assert torch.equal(plan, before)
     expected, expected_lse = oracle.mla_decode_unrounded(query, cache, lengths, 1.0)
     assert_close_bf16("O", out, expected)
     assert_close_lse("LSE", lse, expected_lse)

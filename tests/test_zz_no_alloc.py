@@ -1,6 +1,6 @@
 """The decode entry point that allocates nothing (dscuda_mla_decode_static) against the entry point that
 takes a caller workspace (dscuda_mla_decode), through the C-ABI: two calls in a row on one GPU, the second
-with a smaller input, so the second call finds the first call's partial results and flags in the built-in
+with a smaller input, so the second call finds the first call's partial results and plan in the built-in
 workspace.  Integer/byte-exact bar: both entry points run the same kernels, so outputs must be equal bit
 for bit; the first call is also checked against the fp32 oracle."""
 
@@ -29,7 +29,7 @@ def test_static_workspace_decode_matches_the_workspace_entry_point(cuda):
     scale = configs.c_float(192 ** -0.5)
     first_oracle_done = False
     # a call that cuts sequences over many workgroups, then a smaller one that leaves most of the first
-    # call's slots and flags untouched, then one that does not cut at all
+    # call's slots and plan untouched, then one that does not cut at all
     for batch, tokens, heads, splits, seed in [(12, 3000, 128, 8, 101), (3, 700, 128, 4, 102), (5, 300, 16, 1, 103)]:
         query, cache, paged, table, lengths = _inputs(batch, tokens, heads, seed)
         assert ops.mla_library().workspace(batch, heads, splits, 512) * 4 <= STATIC_BYTES
