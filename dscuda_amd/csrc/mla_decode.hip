@@ -1101,6 +1101,8 @@ __global__ __launch_bounds__(THREADS) void mla_decode_plan_kernel(int* __restric
     }
 }
 
+constexpr int SELF_PLAN_BATCH = THREADS;   // sequences a workgroup turns into a plan by itself
+
 // The decode kernel: every workgroup walks its range of the work list (see index_math.h).
 //
 // Workspace: slot workgroup + sequence holds, for a segment that is only part of its
@@ -1110,8 +1112,11 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     bf16_t* __restrict__ output, float* __restrict__ logsumexp, const bf16_t* __restrict__ query,
     const bf16_t* __restrict__ paged_kv_cache, const int* __restrict__ block_table,
     const int* __restrict__ cache_lengths, float* __restrict__ workspace, int* __restrict__ plan, int batch_size,
-    int heads, int page_size, int pages_per_sequence, long long slot_floats, int padded_rows, float scale) {
+    int heads, int page_size, int pages_per_sequence, long long slot_floats, int padded_rows, float scale,
+    int own_workgroups, int own_whole) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ int own_prefix[SELF_PLAN_BATCH + 1];
+    __shared__ int own_wave_totals[THREADS / 64];
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -1126,25 +1131,78 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     const int head0 = head_group * ROWS;
     const float c = uniform(scale * LOG2E);
 
-    const int total = plan[PLAN_TOTAL];
-    const int workgroups = plan[PLAN_WORKGROUPS];
-    const int overhead = plan[PLAN_OVERHEAD];
-    const bool whole_sequences = plan[PLAN_WHOLE] != 0;
-    const int* prefix = plan + index_math::plan_prefix_at();
-    const int* first_sequence = plan + index_math::plan_first_sequence_at(batch_size);
+    // The plan: read from memory (own_workgroups == 0: the caller's, or one mla_decode_plan_kernel has just built),
+    // or, for a batch that one workgroup scans in one go, worked out here by every workgroup for itself, which
+    // saves the call a kernel launch.  The first workgroup then also leaves what the merge kernel reads of it.
+    int total, overhead, ranges;
+    bool whole_sequences;
+    const int* prefix;
+    if (own_workgroups > 0) {
+        whole_sequences = own_whole != 0;
+        overhead = whole_sequences ? 0 : index_math::SEGMENT_OVERHEAD;
+        int value = tid < batch_size ? index_math::positions_of(tiles_of(cache_lengths[tid]), overhead) : 0;
+#pragma unroll
+        for (int offset = 1; offset < 64; offset <<= 1) {
+            const int other = __shfl_up(value, offset);
+            if (lane >= offset) value += other;
+        }
+        if (lane == 63) own_wave_totals[wave] = value;
+        if (tid == 0) own_prefix[0] = 0;
+        __syncthreads();
+        int before = 0;
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; ++w) {
+            if (w < wave) before += own_wave_totals[w];
+        }
+        if (tid < batch_size) own_prefix[tid + 1] = before + value;
+        __syncthreads();
+        // what comes out of LDS is the same in every lane, which the compiler cannot know: say so, or everything
+        // computed from it (the base addresses of the unit requests among it) ends up in vector registers
+        total = __builtin_amdgcn_readfirstlane(own_prefix[batch_size]);
+        ranges = index_math::ranges_of(total, own_workgroups);
+        prefix = own_prefix;
+        if (blockIdx.x == 0 && blockIdx.y == 0) {
+            if (tid == 0) {
+                plan[PLAN_TOTAL] = total;
+                plan[PLAN_WORKGROUPS] = own_workgroups;
+                plan[PLAN_OVERHEAD] = overhead;
+                plan[PLAN_WHOLE] = own_whole;
+                plan[PLAN_RANGES] = ranges;
+            }
+            if (tid <= batch_size) plan[index_math::plan_prefix_at() + tid] = own_prefix[tid];
+        }
+    } else {
+        total = plan[PLAN_TOTAL];
+        overhead = plan[PLAN_OVERHEAD];
+        whole_sequences = plan[PLAN_WHOLE] != 0;
+        ranges = plan[PLAN_RANGES];
+        prefix = plan + index_math::plan_prefix_at();
+    }
 
     int range_begin, range_end;
     if (whole_sequences) {
-        range_begin = prefix[workgroup];
-        range_end = prefix[workgroup + 1];
+        range_begin = __builtin_amdgcn_readfirstlane(prefix[workgroup]);
+        range_end = __builtin_amdgcn_readfirstlane(prefix[workgroup + 1]);
     } else {
-        const int ranges = plan[PLAN_RANGES];
         if (workgroup >= ranges) return;
         range_begin = index_math::range_begin_of(total, ranges, workgroup);
         range_end = index_math::range_begin_of(total, ranges, workgroup + 1);
     }
     if (range_begin >= range_end) return;
-    int sequence = first_sequence[workgroup];
+    int sequence;
+    if (own_workgroups > 0 && !whole_sequences) {
+        // first sequence whose positions reach past range_begin
+        int low = 0, high = batch_size;
+        while (low < high) {
+            const int mid = (low + high) / 2;
+            if (__builtin_amdgcn_readfirstlane(prefix[mid + 1]) <= range_begin) low = mid + 1; else high = mid;
+        }
+        sequence = low;
+    } else if (own_workgroups > 0) {
+        sequence = workgroup;
+    } else {
+        sequence = plan[index_math::plan_first_sequence_at(batch_size) + workgroup];
+    }
 
     const int head = head0 + 32 * wave + lq;
     const bool valid = head < heads;
@@ -1157,8 +1215,8 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     RowState state;
     int position = range_begin;
     while (position < range_end) {
-        const int sequence_begin = prefix[sequence];
-        const int sequence_end = prefix[sequence + 1];
+        const int sequence_begin = __builtin_amdgcn_readfirstlane(prefix[sequence]);
+        const int sequence_end = __builtin_amdgcn_readfirstlane(prefix[sequence + 1]);
         const int segment_end = min(range_end, sequence_end);
         if (segment_end <= position) {  // a sequence without tiles (length < 1) owns nothing
             ++sequence;
@@ -1413,18 +1471,24 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
     }
     // How the caller's B*H*splits*(C+2) floats are used: index_math::decode_layout.
     const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
+    int own_workgroups = 0;
     if (plan == nullptr) {
-        // no plan from the caller: this call's own, behind the partial-result slots
+        // no plan from the caller: this call's own, behind the partial-result slots -- built by the decode kernel
+        // itself when one workgroup can scan the batch, by the plan kernel otherwise
         plan = reinterpret_cast<int*>(workspace + layout.plan_offset);
-        hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
-                           layout.workgroups, layout.whole_sequences);
-        HIP_CHECK(hipGetLastError());
+        if (batch_size <= SELF_PLAN_BATCH) {
+            own_workgroups = layout.workgroups;
+        } else {
+            hipLaunchKernelGGL(mla_decode_plan_kernel, dim3(1), dim3(THREADS), 0, stream, plan, cache_lengths, batch_size,
+                               layout.workgroups, layout.whole_sequences);
+            HIP_CHECK(hipGetLastError());
+        }
     }
     const int padded_rows = (heads + 31) / 32 * 32;
     const dim3 grid(layout.workgroups, layout.head_groups);
     hipLaunchKernelGGL(mla_decode_split_kernel, grid, dim3(THREADS), LDS_BYTES, stream, output, logsumexp, query,
                        paged_kv_cache, block_table, cache_lengths, workspace, plan, batch_size, heads, page_size,
-                       pages_per_sequence, layout.slot_floats, padded_rows, scale);
+                       pages_per_sequence, layout.slot_floats, padded_rows, scale, own_workgroups, layout.whole_sequences);
     HIP_CHECK(hipGetLastError());
     if (!layout.whole_sequences) {
         hipLaunchKernelGGL(mla_decode_merge_kernel, dim3(MERGE_QUARTERS * (padded_rows / 32), batch_size), dim3(64), 0,
