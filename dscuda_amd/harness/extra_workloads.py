@@ -49,8 +49,7 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
     results["mla_decode_B64_H128"] = {
         "us": ms * 1000.0, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS,
         "bytes": nbytes, "total_tokens": total, "tflops": configs.decode_flops(total, h) / ms / 1e9,
-        "kernels": "mla_decode_plan + mla_decode_split (fast, then the rescaling pass, which finds nothing to do) + "
-                   "mla_decode_merge"}
+        "kernels": "mla_decode_split (plans for itself up to 256 sequences) + mla_decode_merge"}
     del paged, workspace
 
     # long context: MLA prefill forward + backward, B=1 S=16384 H=128.  Timing does not depend on the

@@ -230,7 +230,7 @@ void check_forward_items() {
 }
 
 // ---- decode tile loads: the two-candidate-row form equals the general form for every wave, load, lane and limit,
-// for the 64-key tile (16 rows per wave, 18 loads) and the 32-key unit (8 rows per wave, 9 loads)
+// for the 64-key tile (16 rows per wave, 18 loads), the 32-key unit (8 rows per wave, 9 loads) and 32 rows per wave
 template <int ROWS_PER_WAVE>
 void check_decode_loads() {
     constexpr int ROW_BYTES = 1152, CHUNKS = ROW_BYTES / 16, LOADS = ROWS_PER_WAVE * CHUNKS / 64, ROWS = 4 * ROWS_PER_WAVE;
@@ -396,6 +396,7 @@ int main() {
     check_forward_items();
     check_decode_loads<16>();
     check_decode_loads<8>();
+    check_decode_loads<32>();   // the query rows of a wave (32 rows, 36 loads, wave 0 of the template)
     check_decode_ranges();
     check_decode_layout();
     if (failures) {
