@@ -227,6 +227,68 @@ DSCUDA_HOST_DEVICE inline void ranges_of_sequence(int total, int ranges, int bef
     last = range_of_position(total, ranges, before + positions - 1);
 }
 
+// ---- absorbed backward: the list of (key block, row tile) visits -----------------
+// Rows are the (token, head) pairs of one batch element in memory order, 32 to a row
+// tile (`row_tiles` of them); key block kb (32 keys) is seen by the row tiles from
+// kb * heads (the tile of row 32 * kb * heads, the first row of token 32 * kb) to the
+// last.  The visits of all key blocks of all batch elements, in that order, form one
+// list that the key-gradient kernel cuts into ranges of equal length (+-1); a range
+// that holds only part of a key block's visits leaves an fp32 partial result in slot
+// range + (batch * key_blocks + key block): ranges and key blocks both advance
+// monotonically along the list, so the sums are distinct and below ranges + blocks.
+struct KeyVisits {
+    int key_blocks;
+    int row_tiles;
+    int heads;
+
+    DSCUDA_HOST_DEVICE long long before(int key_block) const {   // visits of key blocks 0 .. key_block-1
+        return (long long)key_block * row_tiles - (long long)heads * key_block * (key_block - 1) / 2;
+    }
+    DSCUDA_HOST_DEVICE long long per_batch() const { return before(key_blocks); }
+    DSCUDA_HOST_DEVICE int first_tile(int key_block) const { return key_block * heads; }
+    // the key block that holds visit `visit` (0 <= visit < per_batch())
+    DSCUDA_HOST_DEVICE int block_of(long long visit) const {
+        int low = 0, high = key_blocks - 1;
+        while (low < high) {
+            const int middle = (low + high + 1) / 2;
+            if (before(middle) <= visit) low = middle; else high = middle - 1;
+        }
+        return low;
+    }
+};
+
+DSCUDA_HOST_DEVICE inline KeyVisits key_visits(int sequence_length, int heads) {
+    KeyVisits visits;
+    visits.key_blocks = (sequence_length + 31) / 32;
+    visits.row_tiles = (int)(((long long)sequence_length * heads + 31) / 32);
+    visits.heads = heads;
+    return visits;
+}
+
+DSCUDA_HOST_DEVICE inline long long wide_range_begin(long long total, long long ranges, long long range) {
+    return range * total / ranges;
+}
+
+DSCUDA_HOST_DEVICE inline long long wide_range_of(long long total, long long ranges, long long position) {
+    return ((position + 1) * ranges - 1) / total;
+}
+
+constexpr long long KEY_PARTIAL_BYTES = 32LL * 576 * 4;   // one slot: [32 keys][576] fp32
+
+// How many ranges the list is cut into when `scratch_bytes` are there for the slots: one per compute unit if the
+// slots allow.  0: every key block is one range and writes its result itself (too few slots for a cut whose
+// longest range is shorter than the longest key block, `row_tiles` visits).
+DSCUDA_HOST_DEVICE inline long long key_gradient_ranges(long long total, long long blocks, int row_tiles,
+                                                        long long scratch_bytes, int compute_units) {
+    const long long slots = scratch_bytes / KEY_PARTIAL_BYTES;
+    long long ranges = slots - blocks;
+    if (ranges > compute_units) ranges = compute_units;
+    if (ranges > total / 2) ranges = total / 2;    // at least two visits per range
+    if (ranges < 2) return 0;
+    const long long longest = (total + ranges - 1) / ranges;
+    return (longest < row_tiles || blocks > compute_units) ? ranges : 0;
+}
+
 // ---- decode: the plan and how a call uses the caller's workspace ---------------
 // The plan is what a decode call needs to know about the lengths of its batch
 // before any workgroup starts: an int table

@@ -2,37 +2,50 @@
 // shared KV head).  Takes the place of the reference's
 // mla_query_backward_kernel and mla_kv_backward_kernel
 // (kernels/attention/mla/sm89.cu:295-411) and keeps their contract: the four
-// gradients are overwritten, each gradient row has exactly one writer (no
-// atomics, deterministic), no workspace.  The mathematics is
-// reference/python/mla.py:42-57:
+// gradients are overwritten, the result does not depend on timing (no atomics:
+// every sum has a fixed order), the caller passes no workspace.  The
+// mathematics is reference/python/mla.py:42-57:
 //     P = exp(S - LSE),  dP = dO latent^T,  delta = sum(dO * O),
 //     dS = P (dP - delta) scale,
 //     dQ = dS [latent|rope],  d[latent|rope] = dS^T [q_lat|q_rope],  dlatent += P^T dO.
 //
 // "Rows" are the (token, head) pairs of one batch element in memory order
 // (row = token*H + head), which makes query / dO / O rows contiguous 512- and
-// 64-wide vectors.  Both kernels run every product on bf16 MFMA 32x32x16 with
-// fp32 accumulation and keep all operands in LDS, 32 rows or keys at a time,
-// each tile stored row-major and (where it is also needed with its row index
-// as the contraction index) transposed, as in the per-head backward.
+// 64-wide vectors.  Every product runs on bf16 MFMA 32x32x16 with fp32
+// accumulation on operands kept in LDS, 32 rows or keys at a time, each tile
+// stored row-major once: where its row index is the contraction index the
+// fragments come through transposing reads.  The next tile is fetched into
+// registers while the current one is multiplied.
 //
-//   query gradients   a workgroup owns 32 rows and walks the keys up to the
-//                     last token of those rows.  Every wave forms the 32x32
-//                     S^T and dP^T of the tile, and accumulates dQ^T for its
-//                     own share of the 18 column blocks.
-//   key gradients     a workgroup owns 32 keys (held in registers) and walks
-//                     the rows from the first token that can see them.  Every
-//                     wave forms S and dP of the tile and accumulates its
-//                     own four latent column blocks (key path and value path
-//                     in the same accumulator) plus a rope column block.
+// Four launches, in this order (the order matters: the first three use the
+// query-gradient buffers, which the last one overwrites, as scratch memory):
+//   row statistics    delta of every row, kept in the first four bytes of the row's
+//                     own 128 bytes of the rope query gradient.
+//   key gradients     one shared KV head means every key is seen by all H heads of
+//                     every later token: T/32 key blocks would be far too few
+//                     workgroups with far too unequal work.  The (key block, row
+//                     tile) visits form one list, cut into equal ranges, one per
+//                     compute unit (index_math.h); a workgroup holds the keys of a
+//                     block in registers, walks its row tiles, forms S and dP of the
+//                     tile in every wave and accumulates its own four latent column
+//                     blocks (key path and value path in the same accumulator) plus
+//                     a rope column block.  A range that holds all visits of a key
+//                     block writes the gradients, otherwise an fp32 partial result
+//                     into the latent query gradient buffer.
+//   reduction         sums the partial results of each cut key block in range order.
+//   query gradients   a workgroup owns 32 rows and walks the keys up to the last
+//                     token of those rows.  Every wave forms the 32x32 S^T and dP^T
+//                     of the tile, and accumulates dQ^T for its own share of the 18
+//                     column blocks.
 //
-// The score products are repeated by the four waves of a workgroup; this entry
-// point is kept for interface parity and correctness at the reference's
-// shapes, the throughput path of this library is the per-head form.
+// The score products are repeated by the four waves of a workgroup.
 #include "attn_kernels.h"
 #include "hip_common.h"
+#include "index_math.h"
 
+#include <cstdint>
 #include <stdexcept>
+#include <type_traits>
 #include <string>
 
 namespace dscuda {
@@ -46,70 +59,76 @@ constexpr int THREADS = 256;
 
 template <int D>
 struct Tile32 {
-    static constexpr int PITCH = 2 * D + 16;                // row-major copy
-    static constexpr int NATURAL_BYTES = TILE * PITCH;
-    static constexpr int T_PITCH = 2 * TILE;                 // transposed copy: 64-byte rows
-    static constexpr int TRANSPOSED_BYTES = D * T_PITCH;
-    static constexpr int UNITS = (TILE / 4) * (D / 4);       // 4 rows x 4 columns
-    static constexpr int PER_THREAD = (UNITS + THREADS - 1) / THREADS;
+    static constexpr int PITCH = 2 * D + 16;                // row-major, rows 16 bytes apart modulo 256
+    static constexpr int BYTES = TILE * PITCH;
 };
 
-// Stage a [32][D] tile whose row `row` starts at row_pointer(row) (nullptr: zero
-// row) into LDS, row-major and/or transposed.  Columns [column0, column0 + D_PART)
-// of the LDS tile come from this call, so a tile can be assembled from two tensors.
-template <int D, int D_PART, bool NATURAL, bool TRANSPOSED, typename RowPointer>
-__device__ __forceinline__ void stage_tile(unsigned char* natural, unsigned char* transposed, int column0,
-                                           RowPointer row_pointer, int tid) {
-    using T = Tile32<D>;
-    constexpr int UNITS = (TILE / 4) * (D_PART / 4);
-    for (int unit = tid; unit < UNITS; unit += THREADS) {
-        const int c4 = unit % (D_PART / 4);
-        const int rg = unit / (D_PART / 4);
-        u32x2 r[4];
+// One thread's share of a [32][D_PART] tile in registers: 16-byte pieces of rows.
+template <int D_PART>
+struct TileShare {
+    static constexpr int PIECES = TILE * D_PART / 8;
+    static constexpr int PER_THREAD = (PIECES + THREADS - 1) / THREADS;
+    u32x4 r[PER_THREAD];
+};
+
+// Fetch a [32][D_PART] tile whose rows lie one behind the other in memory from `first`; rows from `valid_rows`
+// on (possibly <= 0) are zero.
+template <int D_PART>
+__device__ __forceinline__ void fetch_tile(TileShare<D_PART>& share, const bf16_t* first, int valid_rows, int tid) {
+    using S = TileShare<D_PART>;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const bf16_t* source = row_pointer(4 * rg + j);
-            r[j] = u32x2{0, 0};
-            if (source != nullptr) r[j] = *reinterpret_cast<const u32x2*>(source + 4 * c4);
-        }
-        const int column = column0 + 4 * c4;
-        if (NATURAL) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<u32x2*>(natural + (4 * rg + j) * T::PITCH + 2 * column) = r[j];
-            }
-        }
-        if (TRANSPOSED) {
-            // rows 4*rg .. +3 = 16*n + 8*a + 4*g' + (0..3)  ->  position 16*n + 8*g' + 4*a
-            const int n = rg / 4;
-            const int a = (rg % 4) / 2;
-            const int gp = rg % 2;
-            const int chunk = 2 * n + gp;
-            u32x2 t[4];
-            t[0] = u32x2{(r[0].x & 0xffffu) | (r[1].x << 16), (r[2].x & 0xffffu) | (r[3].x << 16)};
-            t[1] = u32x2{(r[0].x >> 16) | (r[1].x & 0xffff0000u), (r[2].x >> 16) | (r[3].x & 0xffff0000u)};
-            t[2] = u32x2{(r[0].y & 0xffffu) | (r[1].y << 16), (r[2].y & 0xffffu) | (r[3].y << 16)};
-            t[3] = u32x2{(r[0].y >> 16) | (r[1].y & 0xffff0000u), (r[2].y >> 16) | (r[3].y & 0xffff0000u)};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int col = column + e;
-                const int swz = chunk ^ ((col >> 2) & 3);
-                *reinterpret_cast<u32x2*>(transposed + col * T::T_PITCH + 16 * swz + 8 * a) = t[e];
-            }
+    for (int p = 0; p < S::PER_THREAD; ++p) {
+        const int piece = tid + p * THREADS;
+        share.r[p] = u32x4{0, 0, 0, 0};
+        if (piece < S::PIECES && piece / (D_PART / 8) < valid_rows) {
+            share.r[p] = *reinterpret_cast<const u32x4*>(first + 8 * piece);
         }
     }
 }
 
-template <int D>
-__device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* natural, int row, int ks, int g) {
-    return *reinterpret_cast<const bf16x8*>(natural + row * Tile32<D>::PITCH + 32 * ks + 16 * g);
+// Place a fetched share into columns [column0, column0 + D_PART) of a [32][D] LDS tile, so that a tile can be
+// assembled from two tensors.
+template <int D, int D_PART>
+__device__ __forceinline__ void place_tile(const TileShare<D_PART>& share, unsigned char* tile, int column0, int tid) {
+    using S = TileShare<D_PART>;
+#pragma unroll
+    for (int p = 0; p < S::PER_THREAD; ++p) {
+        const int piece = tid + p * THREADS;
+        if (piece >= S::PIECES) break;
+        const int row = piece / (D_PART / 8);
+        const int column = column0 + 8 * (piece % (D_PART / 8));
+        *reinterpret_cast<u32x4*>(tile + row * Tile32<D>::PITCH + 2 * column) = share.r[p];
+    }
 }
 
-// column `column`, tile rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}
+// Operand with the tile's column as the contraction index: row lane%32, k-step ks.
 template <int D>
-__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* transposed, int column, int n, int g) {
-    const int swz = (2 * n + g) ^ ((column >> 2) & 3);
-    return *reinterpret_cast<const bf16x8*>(transposed + column * Tile32<D>::T_PITCH + 16 * swz);
+__device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* tile, int row, int ks, int g) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * Tile32<D>::PITCH + 32 * ks + 16 * g);
+}
+
+// Operand with the tile's row as the contraction index, through transposing reads (ds_read_b64_tr_b16): in a
+// block of 16 lanes, lane s points at row 4*g + s/4 (+8 for the second read), columns 4*(s%4)..+3 of the block's
+// 16 columns, and receives the four rows' values of column s.  The lane ends up with column lane%32 of the
+// 32-column block at `column0` and tile rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}, the order in which the
+// accumulators of the score products hold rows.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4* transposing_read_pointer;
+
+template <int D>
+__device__ __forceinline__ int transposed_lane_offset(int lane) {
+    const int g = lane / 32;
+    const int s = lane % 16;
+    const int half = (lane / 16) % 2;
+    return (4 * g + s / 4) * Tile32<D>::PITCH + 32 * half + 8 * (s % 4);
+}
+
+template <int D>
+__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* tile, int lane_offset, int column0, int n) {
+    const unsigned char* at = tile + lane_offset + n * 16 * Tile32<D>::PITCH + 2 * column0;
+    const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)at);
+    const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(at + 8 * Tile32<D>::PITCH));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
 __device__ __forceinline__ void clear(f32x16& value) {
@@ -117,18 +136,46 @@ __device__ __forceinline__ void clear(f32x16& value) {
     for (int i = 0; i < 16; ++i) value[i] = 0.f;
 }
 
-// Per-row statistics of a 32-row tile: lse*log2e, delta = sum(dO*O), token index.
-// Eight threads share a row and 64 columns each.
-__device__ __forceinline__ void stage_row_statistics(float* lse2, float* delta, int* token_of, const bf16_t* dout_rows,
-                                                     const bf16_t* out_rows, const float* lse_batch, long long row0,
-                                                     long long rows, int heads, int sequence_length, int tid) {
-    const int local = tid / 8;
+// f(integral_constant<int, BEGIN>) ... f(integral_constant<int, END - 1>)
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+// COUNT MFMAs, each fed by one LDS fragment read AHEAD steps before its use: with one wave per SIMD nothing
+// else hides the latency of the reads.  `ring` holds fragments 0 .. AHEAD-1 on entry.
+template <int COUNT, int AHEAD, typename Fragment, typename Multiply>
+__device__ __forceinline__ void fragment_stream(bf16x8 (&ring)[AHEAD], Fragment&& fragment, Multiply&& multiply) {
+    static_for<0, COUNT>([&](auto tag) {
+        constexpr int I = decltype(tag)::value;
+        multiply(tag, ring[I % AHEAD]);
+        if constexpr (I + AHEAD < COUNT) ring[I % AHEAD] = fragment(std::integral_constant<int, I + AHEAD>{});
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+template <int AHEAD, typename Fragment>
+__device__ __forceinline__ void fill_ring(bf16x8 (&ring)[AHEAD], Fragment&& fragment) {
+    static_for<0, AHEAD>([&](auto tag) { ring[decltype(tag)::value] = fragment(tag); });
+}
+
+// delta = sum(dO * O) of a row is kept in the first four bytes of the row's 64 rope query gradients (which the
+// query-gradient kernel, the last of the call, overwrites after it has read the delta of its own rows).
+constexpr int DELTA_STRIDE = ROPE / 2;   // in floats
+
+// Eight threads share a row and 64 columns each; rows of all batch elements are numbered through.
+__global__ __launch_bounds__(THREADS) void mla_absorbed_row_statistics_kernel(
+    float* delta, const bf16_t* __restrict__ output_gradient, const bf16_t* __restrict__ output, long long rows) {
+    const int tid = threadIdx.x;
     const int part = tid % 8;
-    const long long row = row0 + local;
+    const long long row = (long long)blockIdx.x * TILE + tid / 8;
     float sum = 0.f;
     if (row < rows) {
-        const bf16_t* a_row = dout_rows + row * RANK + 64 * part;
-        const bf16_t* b_row = out_rows + row * RANK + 64 * part;
+        const bf16_t* a_row = output_gradient + row * RANK + 64 * part;
+        const bf16_t* b_row = output + row * RANK + 64 * part;
 #pragma unroll
         for (int v = 0; v < 8; ++v) {
             const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + 8 * v);
@@ -143,50 +190,53 @@ __device__ __forceinline__ void stage_row_statistics(float* lse2, float* delta, 
     sum += __shfl_xor(sum, 1);
     sum += __shfl_xor(sum, 2);
     sum += __shfl_xor(sum, 4);
-    if (part == 0) {
-        if (row < rows) {
-            const int token = (int)(row / heads);
-            const int head = (int)(row % heads);
-            lse2[local] = lse_batch[(size_t)head * sequence_length + token] * LOG2E;
-            delta[local] = sum;
-            token_of[local] = token;
-        } else {
-            lse2[local] = 0.f;
-            delta[local] = 0.f;
-            token_of[local] = -1;   // sees no key
-        }
+    if (part == 0 && row < rows) delta[row * DELTA_STRIDE] = sum;
+}
+
+// What the gradient formulas need of one row besides its vectors.
+struct RowStatistics {
+    float lse2;    // lse * log2(e)
+    float delta;
+    int token;     // -1: no such row, it sees no key
+};
+
+// Row `row` of the batch element whose rows start at `batch_row0` (thread-per-row: the first 32 threads of a tile).
+__device__ __forceinline__ RowStatistics fetch_row_statistics(const float* delta, const float* lse_batch,
+                                                              long long batch_row0, long long row, long long rows,
+                                                              int heads, int sequence_length) {
+    RowStatistics statistics = {0.f, 0.f, -1};
+    if (row < rows) {
+        const int token = (int)(row / heads);
+        const int head = (int)(row % heads);
+        statistics.lse2 = lse_batch[(size_t)head * sequence_length + token] * LOG2E;
+        statistics.delta = delta[(batch_row0 + row) * DELTA_STRIDE];
+        statistics.token = token;
     }
+    return statistics;
 }
 
 // ---- query gradients -----------------------------------------------------------
 
 struct QueryGradLayout {
-    static constexpr int Q_ROWS = 0;                                          // [32][576] row-major
-    static constexpr int DO_ROWS = Q_ROWS + Tile32<WIDTH>::NATURAL_BYTES;     // [32][512] row-major
-    static constexpr int K_NATURAL = DO_ROWS + Tile32<RANK>::NATURAL_BYTES;   // [32 keys][576]
-    static constexpr int K_TRANSPOSED = K_NATURAL + Tile32<WIDTH>::NATURAL_BYTES;
-    static constexpr int STATS = K_TRANSPOSED + Tile32<WIDTH>::TRANSPOSED_BYTES;
-    static constexpr int LDS_BYTES = STATS + 3 * TILE * 4;
+    static constexpr int KEYS = 0;                             // [32 keys][576]
+    static constexpr int LDS_BYTES = KEYS + Tile32<WIDTH>::BYTES;
 };
 
 __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
-    bf16_t* __restrict__ query_latent_gradient, bf16_t* __restrict__ query_rope_gradient,
-    const bf16_t* __restrict__ output_gradient, const bf16_t* __restrict__ output, const float* __restrict__ logsumexp,
+    bf16_t* query_latent_gradient, bf16_t* query_rope_gradient, const float* delta_of_rows,
+    const bf16_t* __restrict__ output_gradient, const float* __restrict__ logsumexp,
     const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
     const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
     int row_blocks, float scale) {
     using L = QueryGradLayout;
     constexpr int BLOCKS = WIDTH / 32;                 // 18 column blocks of dQ
     constexpr int OWN = (BLOCKS + 3) / 4;              // at most 5 per wave
+    constexpr int QK_STEPS = WIDTH / 16;               // 36
+    constexpr int V_STEPS = RANK / 16;                 // 32
+    constexpr int AHEAD = 6;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* q_rows = lds + L::Q_ROWS;
-    unsigned char* do_rows = lds + L::DO_ROWS;
-    unsigned char* k_natural = lds + L::K_NATURAL;
-    unsigned char* k_transposed = lds + L::K_TRANSPOSED;
-    float* lse2 = reinterpret_cast<float*>(lds + L::STATS);
-    float* delta = lse2 + TILE;
-    int* token_of = reinterpret_cast<int*>(delta + TILE);
+    unsigned char* keys = lds + L::KEYS;
 
     const int tid = threadIdx.x;
     const int wave = tid / 64;
@@ -200,27 +250,48 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
     const long long rows = (long long)T * heads;
     const long long row0 = (long long)row_block * TILE;
     const long long batch_row0 = (long long)batch * rows;
-
-    const bf16_t* ql = query_latent + batch_row0 * RANK;
-    const bf16_t* qr = query_rope + batch_row0 * ROPE;
-    const bf16_t* dout = output_gradient + batch_row0 * RANK;
-    const bf16_t* out = output + batch_row0 * RANK;
     const bf16_t* latent = kv_latent + (size_t)batch * T * RANK;
     const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
 
-    stage_tile<WIDTH, RANK, true, false>(q_rows, nullptr, 0, [&](int r) -> const bf16_t* {
-        return row0 + r < rows ? ql + (row0 + r) * RANK : nullptr; }, tid);
-    stage_tile<WIDTH, ROPE, true, false>(q_rows, nullptr, RANK, [&](int r) -> const bf16_t* {
-        return row0 + r < rows ? qr + (row0 + r) * ROPE : nullptr; }, tid);
-    stage_tile<RANK, RANK, true, false>(do_rows, nullptr, 0, [&](int r) -> const bf16_t* {
-        return row0 + r < rows ? dout + (row0 + r) * RANK : nullptr; }, tid);
-    stage_row_statistics(lse2, delta, token_of, dout, out, logsumexp + (size_t)batch * heads * T, row0, rows, heads, T,
-                         tid);
-    __syncthreads();
+    TileShare<RANK> latent_share;
+    TileShare<ROPE> rope_share;
+    auto fetch_keys = [&](int tile) {
+        const int key0 = tile * TILE;
+        fetch_tile(latent_share, latent + (size_t)key0 * RANK, T - key0, tid);
+        fetch_tile(rope_share, rope + (size_t)key0 * ROPE, T - key0, tid);
+    };
+    fetch_keys(0);
 
-    const float row_lse2 = lse2[lq];
-    const float row_delta = delta[lq];
-    const int row_token = token_of[lq];
+    // this workgroup's rows as B operands (column = row lq), in every wave: the query row and its dO row
+    const long long row = row0 + lq;
+    const bool valid = row < rows;
+    bf16x8 qf[QK_STEPS], dof[V_STEPS];
+    {
+        const size_t r = batch_row0 + (valid ? row : 0);
+#pragma unroll
+        for (int ks = 0; ks < QK_STEPS; ++ks) {
+            u32x4 bits = {0, 0, 0, 0};
+            if (valid) {
+                const bf16_t* source = ks < V_STEPS ? query_latent + r * RANK + 16 * ks + 8 * g
+                                                    : query_rope + r * ROPE + 16 * (ks - V_STEPS) + 8 * g;
+                bits = *reinterpret_cast<const u32x4*>(source);
+            }
+            qf[ks] = __builtin_bit_cast(bf16x8, bits);
+        }
+#pragma unroll
+        for (int ks = 0; ks < V_STEPS; ++ks) {
+            u32x4 bits = {0, 0, 0, 0};
+            if (valid) bits = *reinterpret_cast<const u32x4*>(output_gradient + r * RANK + 16 * ks + 8 * g);
+            dof[ks] = __builtin_bit_cast(bf16x8, bits);
+        }
+    }
+    const RowStatistics statistics = fetch_row_statistics(delta_of_rows, logsumexp + (size_t)batch * heads * T,
+                                                          batch_row0, row, rows, heads, T);
+    const float row_lse2 = statistics.lse2;
+    const float row_delta = statistics.delta;
+    const int row_token = statistics.token;
+    const int transposed_at = transposed_lane_offset<WIDTH>(lane);
+
     const long long last_row = min(rows, row0 + TILE) - 1;
     const int visible = (int)(last_row / heads) + 1;
     const int tiles = (visible + TILE - 1) / TILE;
@@ -232,26 +303,37 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
 
     for (int tile = 0; tile < tiles; ++tile) {
         const int key0 = tile * TILE;
+        __syncthreads();   // the previous tile has been read
+        place_tile<WIDTH>(latent_share, keys, 0, tid);
+        place_tile<WIDTH>(rope_share, keys, RANK, tid);
         __syncthreads();
-        stage_tile<WIDTH, RANK, true, true>(k_natural, k_transposed, 0, [&](int r) -> const bf16_t* {
-            return key0 + r < T ? latent + (size_t)(key0 + r) * RANK : nullptr; }, tid);
-        stage_tile<WIDTH, ROPE, true, true>(k_natural, k_transposed, RANK, [&](int r) -> const bf16_t* {
-            return key0 + r < T ? rope + (size_t)(key0 + r) * ROPE : nullptr; }, tid);
-        __syncthreads();
+        if (tile + 1 < tiles) fetch_keys(tile + 1);   // in flight while this tile is multiplied
 
-        f32x16 s_acc, dp_acc;   // (keys x rows): lane holds row lq and keys key0 + 8*(i/4) + 4*g + i%4
+        // (keys x rows): lane holds row lq and keys key0 + 8*(i/4) + 4*g + i%4.  A key fragment of the latent part
+        // serves the score product and the dP product.
+        f32x16 s_acc, dp_acc;
         clear(s_acc);
         clear(dp_acc);
-#pragma unroll 4
-        for (int ks = 0; ks < WIDTH / 16; ++ks) {
-            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<WIDTH>(k_natural, lq, ks, g),
-                                                            natural_fragment<WIDTH>(q_rows, lq, ks, g), s_acc, 0, 0, 0);
-        }
-#pragma unroll 4
-        for (int ks = 0; ks < RANK / 16; ++ks) {
-            dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<WIDTH>(k_natural, lq, ks, g),
-                                                             natural_fragment<RANK>(do_rows, lq, ks, g), dp_acc, 0, 0, 0);
-        }
+        bf16x8 ring[AHEAD];
+        auto key_fragment = [&](auto tag) { return natural_fragment<WIDTH>(keys, lq, decltype(tag)::value, g); };
+        fill_ring(ring, key_fragment);
+        fragment_stream<QK_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int KS = decltype(tag)::value;
+            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, qf[KS], s_acc, 0, 0, 0);
+            if constexpr (KS < V_STEPS) {
+                dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, dof[KS], dp_acc, 0, 0, 0);
+            }
+        });
+
+        // dQ^T += K^T dS^T for this wave's column blocks; the first fragments are on their way during the softmax
+        auto column_fragment = [&](auto tag) {
+            constexpr int J = decltype(tag)::value / 2;
+            constexpr int N = decltype(tag)::value % 2;
+            const int block = min(wave + 4 * J, BLOCKS - 1);   // the clamped duplicate is never stored
+            return transposed_fragment<WIDTH>(keys, transposed_at, 32 * block, N);
+        };
+        fill_ring(ring, column_fragment);
+
         bf16x8 dsf[2];
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
@@ -271,20 +353,15 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
             }
             dsf[n] = __builtin_bit_cast(bf16x8, packed);
         }
-#pragma unroll
-        for (int j = 0; j < OWN; ++j) {
-            const int block = min(wave + 4 * j, BLOCKS - 1);   // the clamped duplicate is never stored
-#pragma unroll
-            for (int n = 0; n < 2; ++n) {
-                dq_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    transposed_fragment<WIDTH>(k_transposed, 32 * block + lq, n, g), dsf[n], dq_acc[j], 0, 0, 0);
-            }
-        }
+        fragment_stream<2 * OWN>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int J = decltype(tag)::value / 2;
+            constexpr int N = decltype(tag)::value % 2;
+            dq_acc[J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, dsf[N], dq_acc[J], 0, 0, 0);
+        });
     }
 
     // lane holds row lq and columns 32*block + 8*(i/4) + 4*g + i%4
-    const long long row = row0 + lq;
-    if (row < rows) {
+    if (valid) {
 #pragma unroll
         for (int j = 0; j < OWN; ++j) {
             const int block = wave + 4 * j;
@@ -308,29 +385,31 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
 // ---- key gradients -------------------------------------------------------------
 
 struct KeyGradLayout {
-    static constexpr int Q_NATURAL = 0;                                            // [32 rows][576]
-    static constexpr int Q_TRANSPOSED = Q_NATURAL + Tile32<WIDTH>::NATURAL_BYTES;  // [576][32 rows]
-    static constexpr int DO_NATURAL = Q_TRANSPOSED + Tile32<WIDTH>::TRANSPOSED_BYTES;
-    static constexpr int DO_TRANSPOSED = DO_NATURAL + Tile32<RANK>::NATURAL_BYTES;
-    static constexpr int STATS = DO_TRANSPOSED + Tile32<RANK>::TRANSPOSED_BYTES;
+    static constexpr int Q_ROWS = 0;                                  // [32 rows][576]
+    static constexpr int DO_ROWS = Q_ROWS + Tile32<WIDTH>::BYTES;     // [32 rows][512]
+    static constexpr int STATS = DO_ROWS + Tile32<RANK>::BYTES;
     static constexpr int LDS_BYTES = STATS + 3 * TILE * 4;
 };
 
+constexpr int PARTIAL_FLOATS = TILE * WIDTH;   // one slot of partial key gradients: [32 keys][576] fp32
+static_assert(PARTIAL_FLOATS * 4 == index_math::KEY_PARTIAL_BYTES, "slot size");
+
+// `ranges` > 0: workgroup w walks range w of the list of visits; 0: workgroup w walks all visits of key block w
+// (numbered through the batch elements) and writes the gradients itself.
 __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
-    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient,
-    const bf16_t* __restrict__ output_gradient, const bf16_t* __restrict__ output, const float* __restrict__ logsumexp,
-    const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
-    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
-    int key_blocks, float scale) {
+    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
+    const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
+    const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
+    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int batch_size, int sequence_length,
+    int heads, int ranges, float scale) {
     using L = KeyGradLayout;
     constexpr int QK_STEPS = WIDTH / 16;   // 36
     constexpr int V_STEPS = RANK / 16;     // 32
+    constexpr int AHEAD = 6;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* q_natural = lds + L::Q_NATURAL;
-    unsigned char* q_transposed = lds + L::Q_TRANSPOSED;
-    unsigned char* do_natural = lds + L::DO_NATURAL;
-    unsigned char* do_transposed = lds + L::DO_TRANSPOSED;
+    unsigned char* q_rows = lds + L::Q_ROWS;
+    unsigned char* do_rows = lds + L::DO_ROWS;
     float* lse2 = reinterpret_cast<float*>(lds + L::STATS);
     float* delta = lse2 + TILE;
     int* token_of = reinterpret_cast<int*>(delta + TILE);
@@ -341,130 +420,243 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     const int lq = lane % 32;
     const int g = lane / 32;
     const int T = sequence_length;
-
-    const int batch = blockIdx.x / key_blocks;
-    const int key_block = blockIdx.x % key_blocks;   // key block 0 is seen by every row: heaviest first
-    const int k0 = key_block * TILE;
-    const int key = k0 + lq;
     const long long rows = (long long)T * heads;
-    const long long batch_row0 = (long long)batch * rows;
-
-    const bf16_t* ql = query_latent + batch_row0 * RANK;
-    const bf16_t* qr = query_rope + batch_row0 * ROPE;
-    const bf16_t* dout = output_gradient + batch_row0 * RANK;
-    const bf16_t* out = output + batch_row0 * RANK;
-    const bf16_t* latent = kv_latent + (size_t)batch * T * RANK;
-    const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
-
-    // this workgroup's keys as B operands (column = key lq); the value operand is the latent part
-    bf16x8 kf[QK_STEPS];
-    {
-        const bool valid = key < T;
-        const size_t k = valid ? key : 0;
-#pragma unroll
-        for (int ks = 0; ks < QK_STEPS; ++ks) {
-            u32x4 bits = {0, 0, 0, 0};
-            if (valid) {
-                const bf16_t* source = ks < V_STEPS ? latent + k * RANK + 16 * ks + 8 * g
-                                                    : rope + k * ROPE + 16 * (ks - V_STEPS) + 8 * g;
-                bits = *reinterpret_cast<const u32x4*>(source);
-            }
-            kf[ks] = __builtin_bit_cast(bf16x8, bits);
-        }
-    }
-
-    f32x16 latent_acc[4], rope_acc;   // column blocks 4*wave + j of the latent, block wave%2 of the rope part
-#pragma unroll
-    for (int j = 0; j < 4; ++j) clear(latent_acc[j]);
-    clear(rope_acc);
-
     const float c = scale * LOG2E;
-    const long long first_row = (long long)k0 * heads;             // first row that can see key k0
-    const int first_tile = (int)(first_row / TILE);
-    const int last_tile = (int)((rows - 1) / TILE);
+    const int q_transposed_at = transposed_lane_offset<WIDTH>(lane);
+    const int do_transposed_at = transposed_lane_offset<RANK>(lane);
 
-    for (int tile = first_tile; tile <= last_tile; ++tile) {
-        const long long row0 = (long long)tile * TILE;
-        __syncthreads();
-        stage_tile<WIDTH, RANK, true, true>(q_natural, q_transposed, 0, [&](int r) -> const bf16_t* {
-            return row0 + r < rows ? ql + (row0 + r) * RANK : nullptr; }, tid);
-        stage_tile<WIDTH, ROPE, true, true>(q_natural, q_transposed, RANK, [&](int r) -> const bf16_t* {
-            return row0 + r < rows ? qr + (row0 + r) * ROPE : nullptr; }, tid);
-        stage_tile<RANK, RANK, true, true>(do_natural, do_transposed, 0, [&](int r) -> const bf16_t* {
-            return row0 + r < rows ? dout + (row0 + r) * RANK : nullptr; }, tid);
-        stage_row_statistics(lse2, delta, token_of, dout, out, logsumexp + (size_t)batch * heads * T, row0, rows, heads,
-                             T, tid);
-        __syncthreads();
-
-        f32x16 s_acc, dp_acc;   // (rows x keys): lane holds key lq and tile rows 8*(i/4) + 4*g + i%4
-        clear(s_acc);
-        clear(dp_acc);
-#pragma unroll
-        for (int ks = 0; ks < QK_STEPS; ++ks) {
-            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<WIDTH>(q_natural, lq, ks, g), kf[ks], s_acc,
-                                                            0, 0, 0);
-        }
-#pragma unroll
-        for (int ks = 0; ks < V_STEPS; ++ks) {
-            dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(natural_fragment<RANK>(do_natural, lq, ks, g), kf[ks],
-                                                             dp_acc, 0, 0, 0);
-        }
-        bf16x8 pf[2], dsf[2];
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            u32x4 p_packed, ds_packed;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int i4 = 2 * n + half;
-                const int local = 8 * i4 + 4 * g;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
-                const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
-                const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
-                float p[4], ds[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = 4 * i4 + e;
-                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[e]));
-                    if (key > (int)token4[e]) probability = 0.f;
-                    p[e] = probability;
-                    ds[e] = probability * (dp_acc[i] - delta4[e]) * scale;
-                }
-                p_packed[2 * half] = pack_bf16(p[0], p[1]);
-                p_packed[2 * half + 1] = pack_bf16(p[2], p[3]);
-                ds_packed[2 * half] = pack_bf16(ds[0], ds[1]);
-                ds_packed[2 * half + 1] = pack_bf16(ds[2], ds[3]);
-            }
-            pf[n] = __builtin_bit_cast(bf16x8, p_packed);
-            dsf[n] = __builtin_bit_cast(bf16x8, ds_packed);
-        }
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int column = 32 * (4 * wave + j) + lq;
-                latent_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    dsf[n], transposed_fragment<WIDTH>(q_transposed, column, n, g), latent_acc[j], 0, 0, 0);
-                latent_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    pf[n], transposed_fragment<RANK>(do_transposed, column, n, g), latent_acc[j], 0, 0, 0);
-            }
-            rope_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                dsf[n], transposed_fragment<WIDTH>(q_transposed, RANK + 32 * (wave % 2) + lq, n, g), rope_acc, 0, 0, 0);
-        }
+    const index_math::KeyVisits visits = index_math::key_visits(T, heads);
+    const long long per_batch = visits.per_batch();
+    const long long total = per_batch * batch_size;
+    long long position, range_end;
+    if (ranges > 0) {
+        position = index_math::wide_range_begin(total, ranges, blockIdx.x);
+        range_end = index_math::wide_range_begin(total, ranges, blockIdx.x + 1);
+    } else {
+        const int batch = blockIdx.x / visits.key_blocks;
+        const int key_block = blockIdx.x % visits.key_blocks;
+        position = batch * per_batch + visits.before(key_block);
+        range_end = batch * per_batch + visits.before(key_block + 1);
     }
 
-    // lane holds column (block, lq) and keys k0 + 8*(i/4) + 4*g + i%4
+    while (position < range_end) {
+        const int batch = (int)(position / per_batch);
+        const long long within = position - batch * per_batch;
+        const int key_block = visits.block_of(within);
+        const long long block_begin = visits.before(key_block);
+        const long long block_end = visits.before(key_block + 1);
+        const long long segment_end = min(range_end - batch * per_batch, block_end);
+        const int first_tile = visits.first_tile(key_block) + (int)(within - block_begin);
+        const int end_tile = visits.first_tile(key_block) + (int)(segment_end - block_begin);
+        const bool whole = within == block_begin && segment_end == block_end;
+
+        const int k0 = key_block * TILE;
+        const int key = k0 + lq;
+        const long long batch_row0 = (long long)batch * rows;
+        const bf16_t* ql = query_latent + batch_row0 * RANK;
+        const bf16_t* qr = query_rope + batch_row0 * ROPE;
+        const bf16_t* dout = output_gradient + batch_row0 * RANK;
+        const bf16_t* latent = kv_latent + (size_t)batch * T * RANK;
+        const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
+        const float* lse_batch = logsumexp + (size_t)batch * heads * T;
+
+        // this segment's keys as B operands (column = key lq); the value operand is the latent part
+        bf16x8 kf[QK_STEPS];
+        {
+            const bool valid = key < T;
+            const size_t k = valid ? key : 0;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int k = k0 + 8 * (i / 4) + 4 * g + i % 4;
-        if (k < T) {
-            __bf16* latent_row = reinterpret_cast<__bf16*>(kv_latent_gradient) + ((size_t)batch * T + k) * RANK;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) latent_row[32 * (4 * wave + j) + lq] = (__bf16)latent_acc[j][i];
-            if (wave < 2) {
-                __bf16* rope_row = reinterpret_cast<__bf16*>(key_rope_gradient) + ((size_t)batch * T + k) * ROPE;
-                rope_row[32 * wave + lq] = (__bf16)rope_acc[i];
+            for (int ks = 0; ks < QK_STEPS; ++ks) {
+                u32x4 bits = {0, 0, 0, 0};
+                if (valid) {
+                    const bf16_t* source = ks < V_STEPS ? latent + k * RANK + 16 * ks + 8 * g
+                                                        : rope + k * ROPE + 16 * (ks - V_STEPS) + 8 * g;
+                    bits = *reinterpret_cast<const u32x4*>(source);
+                }
+                kf[ks] = __builtin_bit_cast(bf16x8, bits);
             }
         }
+
+        f32x16 latent_acc[4], rope_acc;   // column blocks 4*wave + j of the latent, block wave%2 of the rope part
+#pragma unroll
+        for (int j = 0; j < 4; ++j) clear(latent_acc[j]);
+        clear(rope_acc);
+
+        TileShare<RANK> q_share, do_share;
+        TileShare<ROPE> rope_share;
+        RowStatistics statistics = {0.f, 0.f, -1};
+        auto fetch_rows = [&](int tile) {
+            const long long row0 = (long long)tile * TILE;
+            const int valid_rows = (int)min(rows - row0, (long long)TILE);
+            fetch_tile(q_share, ql + row0 * RANK, valid_rows, tid);
+            fetch_tile(rope_share, qr + row0 * ROPE, valid_rows, tid);
+            fetch_tile(do_share, dout + row0 * RANK, valid_rows, tid);
+            if (tid < TILE) {
+                statistics = fetch_row_statistics(delta_of_rows, lse_batch, batch_row0, row0 + tid, rows, heads, T);
+            }
+        };
+        fetch_rows(first_tile);
+
+        for (int tile = first_tile; tile < end_tile; ++tile) {
+            __syncthreads();   // the previous tile has been read
+            place_tile<WIDTH>(q_share, q_rows, 0, tid);
+            place_tile<WIDTH>(rope_share, q_rows, RANK, tid);
+            place_tile<RANK>(do_share, do_rows, 0, tid);
+            if (tid < TILE) {
+                lse2[tid] = statistics.lse2;
+                delta[tid] = statistics.delta;
+                token_of[tid] = statistics.token;
+            }
+            __syncthreads();
+            if (tile + 1 < end_tile) fetch_rows(tile + 1);   // in flight while this tile is multiplied
+
+            f32x16 s_acc, dp_acc;   // (rows x keys): lane holds key lq and tile rows 8*(i/4) + 4*g + i%4
+            clear(s_acc);
+            clear(dp_acc);
+            bf16x8 ring[AHEAD];
+            auto row_fragment = [&](auto tag) {
+                constexpr int I = decltype(tag)::value;
+                if constexpr (I < QK_STEPS) {
+                    return natural_fragment<WIDTH>(q_rows, lq, I, g);
+                } else {
+                    return natural_fragment<RANK>(do_rows, lq, I - QK_STEPS, g);
+                }
+            };
+            fill_ring(ring, row_fragment);
+            fragment_stream<QK_STEPS + V_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
+                constexpr int I = decltype(tag)::value;
+                if constexpr (I < QK_STEPS) {
+                    s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[I], s_acc, 0, 0, 0);
+                } else {
+                    dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[I - QK_STEPS], dp_acc, 0, 0, 0);
+                }
+            });
+
+            // per 16-row step n: (q columns, dO columns) of the wave's four latent blocks, then its rope block; the
+            // first fragments are on their way during the softmax
+            auto column_fragment = [&](auto tag) {
+                constexpr int N = decltype(tag)::value / 9;
+                constexpr int F = decltype(tag)::value % 9;
+                if constexpr (F == 8) {
+                    return transposed_fragment<WIDTH>(q_rows, q_transposed_at, RANK + 32 * (wave % 2), N);
+                } else if constexpr (F % 2 == 0) {
+                    return transposed_fragment<WIDTH>(q_rows, q_transposed_at, 32 * (4 * wave + F / 2), N);
+                } else {
+                    return transposed_fragment<RANK>(do_rows, do_transposed_at, 32 * (4 * wave + F / 2), N);
+                }
+            };
+            fill_ring(ring, column_fragment);
+
+            bf16x8 pf[2], dsf[2];
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                u32x4 p_packed, ds_packed;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int i4 = 2 * n + half;
+                    const int local = 8 * i4 + 4 * g;
+                    const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
+                    const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
+                    const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+                    float p[4], ds[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int i = 4 * i4 + e;
+                        float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[e]));
+                        if (key > (int)token4[e]) probability = 0.f;
+                        p[e] = probability;
+                        ds[e] = probability * (dp_acc[i] - delta4[e]) * scale;
+                    }
+                    p_packed[2 * half] = pack_bf16(p[0], p[1]);
+                    p_packed[2 * half + 1] = pack_bf16(p[2], p[3]);
+                    ds_packed[2 * half] = pack_bf16(ds[0], ds[1]);
+                    ds_packed[2 * half + 1] = pack_bf16(ds[2], ds[3]);
+                }
+                pf[n] = __builtin_bit_cast(bf16x8, p_packed);
+                dsf[n] = __builtin_bit_cast(bf16x8, ds_packed);
+            }
+            fragment_stream<18>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
+                constexpr int N = decltype(tag)::value / 9;
+                constexpr int F = decltype(tag)::value % 9;
+                if constexpr (F == 8) {
+                    rope_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], fragment, rope_acc, 0, 0, 0);
+                } else if constexpr (F % 2 == 0) {
+                    latent_acc[F / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], fragment, latent_acc[F / 2], 0, 0, 0);
+                } else {
+                    latent_acc[F / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[N], fragment, latent_acc[F / 2], 0, 0, 0);
+                }
+            });
+        }
+
+        // lane holds column (block, lq) and keys k0 + 8*(i/4) + 4*g + i%4
+        if (whole) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int k = k0 + 8 * (i / 4) + 4 * g + i % 4;
+                if (k < T) {
+                    __bf16* latent_row = reinterpret_cast<__bf16*>(kv_latent_gradient) + ((size_t)batch * T + k) * RANK;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) latent_row[32 * (4 * wave + j) + lq] = (__bf16)latent_acc[j][i];
+                    if (wave < 2) {
+                        __bf16* rope_row = reinterpret_cast<__bf16*>(key_rope_gradient) + ((size_t)batch * T + k) * ROPE;
+                        rope_row[32 * wave + lq] = (__bf16)rope_acc[i];
+                    }
+                }
+            }
+        } else {
+            float* slot = partial_slots +
+                ((long long)blockIdx.x + (long long)batch * visits.key_blocks + key_block) * PARTIAL_FLOATS;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float* slot_row = slot + (8 * (i / 4) + 4 * g + i % 4) * WIDTH;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) slot_row[32 * (4 * wave + j) + lq] = latent_acc[j][i];
+                if (wave < 2) slot_row[RANK + 32 * wave + lq] = rope_acc[i];
+            }
+        }
+        position = batch * per_batch + segment_end;
+    }
+}
+
+// Sums the partial key gradients of every key block whose visits were cut, in range order.  Workgroup (x, y)
+// takes the y-th 1/REDUCTION_PARTS of key block x (numbered through the batch elements), a thread four
+// neighbouring columns of one key; a block that one range held whole wrote its gradients itself.
+constexpr int REDUCTION_PARTS = PARTIAL_FLOATS / 4 / THREADS;   // 18
+static_assert(REDUCTION_PARTS * THREADS * 4 == PARTIAL_FLOATS, "slot size");
+
+__global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
+    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient,
+    const float* __restrict__ partial_slots, int sequence_length, int heads, int batch_size, int ranges) {
+    const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
+    const long long per_batch = visits.per_batch();
+    const long long total = per_batch * batch_size;
+    const int batch = blockIdx.x / visits.key_blocks;
+    const int key_block = blockIdx.x % visits.key_blocks;
+    const long long begin = batch * per_batch + visits.before(key_block);
+    const long long end = batch * per_batch + visits.before(key_block + 1);
+    const long long first_range = index_math::wide_range_of(total, ranges, begin);
+    const long long last_range = index_math::wide_range_of(total, ranges, end - 1);
+    if (first_range == last_range) return;
+
+    const int index = blockIdx.y * THREADS + threadIdx.x;   // which four floats of the slot
+    const float* first_slot = partial_slots + (first_range + blockIdx.x) * PARTIAL_FLOATS + 4 * index;
+    const int parts = (int)(last_range - first_range) + 1;
+    f32x4 sum = *reinterpret_cast<const f32x4*>(first_slot);
+    for (int part = 1; part < parts; ++part) {
+        const f32x4 value = *reinterpret_cast<const f32x4*>(first_slot + (long long)part * PARTIAL_FLOATS);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum[e] += value[e];
+    }
+    const int key = key_block * TILE + (4 * index) / WIDTH;
+    const int column = (4 * index) % WIDTH;
+    if (key < sequence_length) {
+        u32x2 packed;
+        packed.x = pack_bf16(sum[0], sum[1]);
+        packed.y = pack_bf16(sum[2], sum[3]);
+        bf16_t* destination = column < RANK
+            ? kv_latent_gradient + ((size_t)batch * sequence_length + key) * RANK + column
+            : key_rope_gradient + ((size_t)batch * sequence_length + key) * ROPE + (column - RANK);
+        *reinterpret_cast<u32x2*>(destination) = packed;
     }
 }
 
@@ -472,6 +664,18 @@ template <typename Kernel>
 void raise_lds_limit(Kernel kernel, int bytes) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   bytes));
+}
+
+int device_compute_units() {
+    static thread_local int device_of = -1;
+    static thread_local int units = 0;
+    int device = 0;
+    HIP_CHECK(hipGetDevice(&device));
+    if (device != device_of) {
+        HIP_CHECK(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+        device_of = device;
+    }
+    return units;
 }
 
 }  // namespace
@@ -482,27 +686,48 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
                                     const bf16_t* query_latent, const bf16_t* query_rope, const bf16_t* kv_latent,
                                     const bf16_t* key_rope, int batch_size, int sequence_length, int heads, float scale,
                                     hipStream_t stream) {
+    const long long rows = (long long)sequence_length * heads;
+    const long long row_blocks = (rows + TILE - 1) / TILE;
+    if (row_blocks * batch_size > 0x7fffffffLL) {
+        throw std::invalid_argument("MLA backward: batch*tokens*heads exceeds the grid limit");
+    }
+    if (reinterpret_cast<uintptr_t>(query_latent_gradient) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(query_rope_gradient) % 16 != 0) {
+        throw std::invalid_argument("MLA backward: the query gradients must be aligned to 16 bytes");
+    }
     static thread_local bool prepared = false;
     if (!prepared) {
         raise_lds_limit(mla_absorbed_query_gradient_kernel, QueryGradLayout::LDS_BYTES);
         raise_lds_limit(mla_absorbed_key_gradient_kernel, KeyGradLayout::LDS_BYTES);
         prepared = true;
     }
-    const long long rows = (long long)sequence_length * heads;
-    const long long row_blocks = (rows + TILE - 1) / TILE;
-    const long long key_blocks = (sequence_length + TILE - 1) / TILE;
-    if (row_blocks * batch_size > 0x7fffffffLL) {
-        throw std::invalid_argument("MLA backward: batch*tokens*heads exceeds the grid limit");
+    // scratch memory until the last launch: delta in the rope query gradients, partial key gradients in the latent ones
+    float* delta = reinterpret_cast<float*>(query_rope_gradient);
+    float* partial_slots = reinterpret_cast<float*>(query_latent_gradient);
+    const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
+    const long long blocks = (long long)visits.key_blocks * batch_size;
+    const long long total = visits.per_batch() * batch_size;
+    const long long ranges = index_math::key_gradient_ranges(total, blocks, visits.row_tiles,
+                                                             rows * batch_size * RANK * 2, device_compute_units());
+
+    hipLaunchKernelGGL(mla_absorbed_row_statistics_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS), 0,
+                       stream, delta, output_gradient, output, rows * batch_size);
+    HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)(ranges > 0 ? ranges : blocks)), dim3(THREADS),
+                       KeyGradLayout::LDS_BYTES, stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta,
+                       output_gradient, logsumexp, query_latent, query_rope, kv_latent, key_rope, batch_size,
+                       sequence_length, heads, (int)ranges, scale);
+    HIP_CHECK(hipGetLastError());
+    if (ranges > 0) {
+        hipLaunchKernelGGL(mla_absorbed_key_reduction_kernel, dim3((unsigned)blocks, REDUCTION_PARTS), dim3(THREADS), 0, stream,
+                           kv_latent_gradient, key_rope_gradient, partial_slots, sequence_length, heads, batch_size,
+                           (int)ranges);
+        HIP_CHECK(hipGetLastError());
     }
     hipLaunchKernelGGL(mla_absorbed_query_gradient_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS),
-                       QueryGradLayout::LDS_BYTES, stream, query_latent_gradient, query_rope_gradient, output_gradient,
-                       output, logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length, heads,
+                       QueryGradLayout::LDS_BYTES, stream, query_latent_gradient, query_rope_gradient, delta,
+                       output_gradient, logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length, heads,
                        (int)row_blocks, scale);
-    HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)(key_blocks * batch_size)), dim3(THREADS),
-                       KeyGradLayout::LDS_BYTES, stream, kv_latent_gradient, key_rope_gradient, output_gradient, output,
-                       logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length, heads,
-                       (int)key_blocks, scale);
     HIP_CHECK(hipGetLastError());
 }
 

@@ -259,6 +259,79 @@ void check_decode_loads() {
     }
 }
 
+// ---- absorbed backward: the list of (key block, row tile) visits.  A row tile is visited by a key block exactly when
+// one of its rows can see one of the block's keys; the closed forms agree with enumeration; the ranges partition the
+// list; (range, block) pairs that hold part of a block own distinct slots below the slot count the cut was sized for.
+void check_key_visits() {
+    for (int heads : {1, 2, 3, 4, 8, 16, 20, 128}) {
+        for (int tokens : {1, 5, 31, 32, 33, 96, 128, 257, 512, 1000}) {
+            if ((long long)heads * tokens > 40000) continue;
+            const KeyVisits visits = key_visits(tokens, heads);
+            const long long rows = (long long)heads * tokens;
+            EXPECT(visits.key_blocks == (tokens + 31) / 32 && visits.row_tiles == (rows + 31) / 32, "counts");
+            long long before = 0;
+            for (int kb = 0; kb < visits.key_blocks; ++kb) {
+                EXPECT(visits.before(kb) == before, "heads %d tokens %d block %d: before %lld vs %lld", heads, tokens, kb, visits.before(kb), before);
+                int first = -1, count = 0;
+                for (int tile = 0; tile < visits.row_tiles; ++tile) {
+                    const long long last_row = std::min<long long>(rows, 32LL * (tile + 1)) - 1;
+                    if (last_row / heads >= 32 * kb) {   // the tile's last token sees the block's first key
+                        if (first < 0) first = tile;
+                        ++count;
+                    }
+                }
+                EXPECT(count >= 1 && first == visits.first_tile(kb), "heads %d tokens %d block %d: first tile %d vs %d", heads, tokens, kb, first, visits.first_tile(kb));
+                for (long long v = before; v < before + count; v += std::max(1, count / 7)) EXPECT(visits.block_of(v) == kb, "block_of");
+                EXPECT(visits.block_of(before + count - 1) == kb, "block_of last");
+                before += count;
+            }
+            EXPECT(visits.per_batch() == before, "per_batch");
+            for (int batch : {1, 2, 3}) {
+                const long long total = before * batch, blocks = (long long)visits.key_blocks * batch;
+                for (int units : {4, 256}) {
+                    for (long long scratch : {0LL, rows * batch * 1024, rows * batch * 1024 / 3, 1LL << 40}) {
+                        const long long ranges = key_gradient_ranges(total, blocks, visits.row_tiles, scratch, units);
+                        if (ranges == 0) continue;
+                        EXPECT(ranges >= 2 && ranges <= units && ranges + blocks <= scratch / KEY_PARTIAL_BYTES && 2 * ranges <= total,
+                               "ranges %lld blocks %lld scratch %lld", ranges, blocks, scratch);
+                        std::set<long long> slots;
+                        long long covered = 0;
+                        for (long long r = 0; r < ranges; ++r) {
+                            const long long begin = wide_range_begin(total, ranges, r), end = wide_range_begin(total, ranges, r + 1);
+                            EXPECT(end > begin, "empty range");
+                            EXPECT(wide_range_of(total, ranges, begin) == r && wide_range_of(total, ranges, end - 1) == r, "range_of");
+                            long long position = begin;
+                            while (position < end) {   // the kernel's walk
+                                const int b = (int)(position / before);
+                                const long long within = position - b * before;
+                                const int kb = visits.block_of(within);
+                                const long long segment_end = std::min(end - b * before, visits.before(kb + 1));
+                                const bool whole = within == visits.before(kb) && segment_end == visits.before(kb + 1);
+                                if (!whole) {
+                                    const long long slot = r + (long long)b * visits.key_blocks + kb;
+                                    EXPECT(slot < scratch / KEY_PARTIAL_BYTES, "slot %lld", slot);
+                                    EXPECT(slots.insert(slot).second, "slot %lld used twice", slot);
+                                    // the reduction finds it: the block's first range + offset
+                                    const long long g_begin = b * before + visits.before(kb);
+                                    const long long first_range = wide_range_of(total, ranges, g_begin);
+                                    const long long last_range = wide_range_of(total, ranges, b * before + visits.before(kb + 1) - 1);
+                                    EXPECT(first_range < last_range && r >= first_range && r <= last_range, "reduction range");
+                                } else {
+                                    const long long g_begin = b * before + visits.before(kb);
+                                    EXPECT(wide_range_of(total, ranges, g_begin) == wide_range_of(total, ranges, b * before + visits.before(kb + 1) - 1), "whole block");
+                                }
+                                covered += segment_end - within;
+                                position = b * before + segment_end;
+                            }
+                        }
+                        EXPECT(covered == total, "covered %lld of %lld", covered, total);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- decode: the ranges partition the list of positions, their lengths differ by at most one, every tile of every
 // sequence is computed by exactly one range, and (range, sequence) pairs that hold part of a sequence own distinct slots
 void check_decode_ranges() {
@@ -396,7 +469,8 @@ int main() {
     check_forward_items();
     check_decode_loads<16>();
     check_decode_loads<8>();
-    check_decode_loads<32>();   // the query rows of a wave (32 rows, 36 loads, wave 0 of the template)
+    check_decode_loads<32>();
+    check_key_visits();
     check_decode_ranges();
     check_decode_layout();
     if (failures) {
