@@ -14,8 +14,9 @@
 // 64-wide vectors.  Every product runs on bf16 MFMA 32x32x16 with fp32
 // accumulation on operands kept in LDS, 32 rows or keys at a time, each tile
 // stored row-major once: where its row index is the contraction index the
-// fragments come through transposing reads.  The next tile is fetched into
-// registers while the current one is multiplied.
+// fragments come through transposing reads.  While a tile is multiplied the
+// next one moves from registers into a second LDS buffer and the one after
+// that is on its way from memory.
 //
 // Four launches, in this order (the order matters: the first three use the
 // query-gradient buffers, which the last one overwrites, as scratch memory):
@@ -26,19 +27,18 @@
 //                     workgroups with far too unequal work.  The (key block, row
 //                     tile) visits form one list, cut into equal ranges, one per
 //                     compute unit (index_math.h); a workgroup holds the keys of a
-//                     block in registers, walks its row tiles, forms S and dP of the
-//                     tile in every wave and accumulates its own four latent column
+//                     block in registers and walks its row tiles: every wave forms one
+//                     quadrant of S and dP of the tile, the quadrants of P and dS meet
+//                     in LDS, and every wave accumulates its own four latent column
 //                     blocks (key path and value path in the same accumulator) plus
 //                     a rope column block.  A range that holds all visits of a key
 //                     block writes the gradients, otherwise an fp32 partial result
 //                     into the latent query gradient buffer.
 //   reduction         sums the partial results of each cut key block in range order.
 //   query gradients   a workgroup owns 32 rows and walks the keys up to the last
-//                     token of those rows.  Every wave forms the 32x32 S^T and dP^T
-//                     of the tile, and accumulates dQ^T for its own share of the 18
-//                     column blocks.
-//
-// The score products are repeated by the four waves of a workgroup.
+//                     token of those rows.  Every wave forms one quadrant of S^T and
+//                     dP^T of the tile, the quadrants of dS^T meet in LDS, and every
+//                     wave accumulates dQ^T for its own share of the 18 column blocks.
 #include "attn_kernels.h"
 #include "hip_common.h"
 #include "index_math.h"
@@ -162,6 +162,51 @@ __device__ __forceinline__ void fill_ring(bf16x8 (&ring)[AHEAD], Fragment&& frag
     static_for<0, AHEAD>([&](auto tag) { ring[decltype(tag)::value] = fragment(tag); });
 }
 
+// The score products of a 32 x 32 tile are split over the four waves: each forms one 16 x 16 quadrant (16x16x32
+// MFMA: lane l holds column l%16 and rows 4*(l/16) .. +3 of its quadrant), applies the softmax gradient to it and
+// leaves its P / dS values in an LDS tile [32 columns][32 rows] of bf16, from which every wave reads the whole
+// tile as an operand of the 32x32x16 products: lane l takes column l%32, rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}
+// (g = l/32), the row order of the transposing reads that feed the other operand.  72-byte pitch: the 8-byte
+// accesses of 32 lanes fall into different banks.
+constexpr int EXCHANGE_PITCH = 2 * TILE + 8;
+constexpr int EXCHANGE_BYTES = TILE * EXCHANGE_PITCH;
+
+// four neighbouring rows (from `row`, a multiple of 4) of column `column`
+__device__ __forceinline__ void exchange_store(unsigned char* exchange, int column, int row, const float (&value)[4]) {
+    u32x2 packed;
+    packed.x = pack_bf16(value[0], value[1]);
+    packed.y = pack_bf16(value[2], value[3]);
+    *reinterpret_cast<u32x2*>(exchange + column * EXCHANGE_PITCH + 2 * row) = packed;
+}
+
+__device__ __forceinline__ bf16x8 exchange_fragment(const unsigned char* exchange, int lq, int g, int n) {
+    const unsigned char* at = exchange + lq * EXCHANGE_PITCH + 2 * (16 * n + 4 * g);
+    const u32x2 low = *reinterpret_cast<const u32x2*>(at);
+    const u32x2 high = *reinterpret_cast<const u32x2*>(at + 16);
+    return __builtin_bit_cast(bf16x8, u32x4{low.x, low.y, high.x, high.y});
+}
+
+// Operand of the 16x16x32 products out of a row-major tile: row `row` (of the wave's 16), k-step s of 32 columns.
+template <int D>
+__device__ __forceinline__ bf16x8 quadrant_fragment(const unsigned char* tile, int row, int s, int quad) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * Tile32<D>::PITCH + 64 * s + 16 * quad);
+}
+
+// The same operand straight from memory: 32 columns per step, latent part first, then the rope part.
+template <int STEPS>
+__device__ __forceinline__ void fetch_quadrant_operand(bf16x8 (&operand)[STEPS], const bf16_t* latent_row,
+                                                       const bf16_t* rope_row, bool valid, int quad) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        u32x4 bits = {0, 0, 0, 0};
+        if (valid) {
+            const bf16_t* source = s < RANK / 32 ? latent_row + 32 * s + 8 * quad : rope_row + 32 * (s - RANK / 32) + 8 * quad;
+            bits = *reinterpret_cast<const u32x4*>(source);
+        }
+        operand[s] = __builtin_bit_cast(bf16x8, bits);
+    }
+}
+
 // delta = sum(dO * O) of a row is kept in the first four bytes of the row's 64 rope query gradients (which the
 // query-gradient kernel, the last of the call, overwrites after it has read the delta of its own rows).
 constexpr int DELTA_STRIDE = ROPE / 2;   // in floats
@@ -218,8 +263,9 @@ __device__ __forceinline__ RowStatistics fetch_row_statistics(const float* delta
 // ---- query gradients -----------------------------------------------------------
 
 struct QueryGradLayout {
-    static constexpr int KEYS = 0;                             // [32 keys][576]
-    static constexpr int LDS_BYTES = KEYS + Tile32<WIDTH>::BYTES;
+    static constexpr int BUFFER_BYTES = Tile32<WIDTH>::BYTES;  // [32 keys][576]
+    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;          // the tile being multiplied and the next one
+    static constexpr int LDS_BYTES = EXCHANGE + EXCHANGE_BYTES;
 };
 
 __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
@@ -236,7 +282,6 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
     constexpr int AHEAD = 6;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* keys = lds + L::KEYS;
 
     const int tid = threadIdx.x;
     const int wave = tid / 64;
@@ -260,37 +305,36 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
         fetch_tile(latent_share, latent + (size_t)key0 * RANK, T - key0, tid);
         fetch_tile(rope_share, rope + (size_t)key0 * ROPE, T - key0, tid);
     };
+    auto place_keys = [&](int tile) {
+        unsigned char* keys = lds + (tile & 1) * L::BUFFER_BYTES;
+        place_tile<WIDTH>(latent_share, keys, 0, tid);
+        place_tile<WIDTH>(rope_share, keys, RANK, tid);
+    };
     fetch_keys(0);
 
-    // this workgroup's rows as B operands (column = row lq), in every wave: the query row and its dO row
-    const long long row = row0 + lq;
-    const bool valid = row < rows;
-    bf16x8 qf[QK_STEPS], dof[V_STEPS];
-    {
-        const size_t r = batch_row0 + (valid ? row : 0);
-#pragma unroll
-        for (int ks = 0; ks < QK_STEPS; ++ks) {
-            u32x4 bits = {0, 0, 0, 0};
-            if (valid) {
-                const bf16_t* source = ks < V_STEPS ? query_latent + r * RANK + 16 * ks + 8 * g
-                                                    : query_rope + r * ROPE + 16 * (ks - V_STEPS) + 8 * g;
-                bits = *reinterpret_cast<const u32x4*>(source);
-            }
-            qf[ks] = __builtin_bit_cast(bf16x8, bits);
-        }
-#pragma unroll
-        for (int ks = 0; ks < V_STEPS; ++ks) {
-            u32x4 bits = {0, 0, 0, 0};
-            if (valid) bits = *reinterpret_cast<const u32x4*>(output_gradient + r * RANK + 16 * ks + 8 * g);
-            dof[ks] = __builtin_bit_cast(bf16x8, bits);
-        }
-    }
+    // this wave's quadrant of the score tile: keys 16*key_half .. +15 x rows 16*row_half .. +15.  Its rows as B
+    // operands (column = row l16): the query row and its dO row
+    constexpr int Q_STEPS = WIDTH / 32;   // 18
+    constexpr int O_STEPS = RANK / 32;    // 16
+    const int key_half = wave / 2;
+    const int row_half = wave % 2;
+    const int l16 = lane % 16;
+    const int quad = lane / 16;
+    const long long own_row = row0 + 16 * row_half + l16;
+    const bool own_valid = own_row < rows;
+    const size_t own = batch_row0 + (own_valid ? own_row : 0);
+    bf16x8 qf[Q_STEPS], dof[O_STEPS];
+    fetch_quadrant_operand(qf, query_latent + own * RANK, query_rope + own * ROPE, own_valid, quad);
+    fetch_quadrant_operand(dof, output_gradient + own * RANK, nullptr, own_valid, quad);
     const RowStatistics statistics = fetch_row_statistics(delta_of_rows, logsumexp + (size_t)batch * heads * T,
-                                                          batch_row0, row, rows, heads, T);
+                                                          batch_row0, own_row, rows, heads, T);
     const float row_lse2 = statistics.lse2;
     const float row_delta = statistics.delta;
     const int row_token = statistics.token;
     const int transposed_at = transposed_lane_offset<WIDTH>(lane);
+    unsigned char* exchange = lds + L::EXCHANGE;
+    const long long row = row0 + lq;   // the row whose gradient this lane ends up with
+    const bool valid = row < rows;
 
     const long long last_row = min(rows, row0 + TILE) - 1;
     const int visible = (int)(last_row / heads) + 1;
@@ -301,27 +345,32 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
 #pragma unroll
     for (int j = 0; j < OWN; ++j) clear(dq_acc[j]);
 
+    // Tile t is multiplied out of buffer t % 2 while tile t + 1 goes from registers into the other buffer and
+    // tile t + 2 is on its way from memory: a fetch has a whole step to arrive, and a step has one barrier.
+    place_keys(0);
+    if (tiles > 1) fetch_keys(1);
     for (int tile = 0; tile < tiles; ++tile) {
         const int key0 = tile * TILE;
-        __syncthreads();   // the previous tile has been read
-        place_tile<WIDTH>(latent_share, keys, 0, tid);
-        place_tile<WIDTH>(rope_share, keys, RANK, tid);
-        __syncthreads();
-        if (tile + 1 < tiles) fetch_keys(tile + 1);   // in flight while this tile is multiplied
+        const unsigned char* keys = lds + (tile & 1) * L::BUFFER_BYTES;
+        __syncthreads();   // this tile is in place, the other buffer has been read
+        if (tile + 1 < tiles) {
+            place_keys(tile + 1);
+            if (tile + 2 < tiles) fetch_keys(tile + 2);
+        }
 
-        // (keys x rows): lane holds row lq and keys key0 + 8*(i/4) + 4*g + i%4.  A key fragment of the latent part
-        // serves the score product and the dP product.
-        f32x16 s_acc, dp_acc;
-        clear(s_acc);
-        clear(dp_acc);
+        // (keys x rows) quadrant: lane holds row l16 and keys 4*quad .. +3 of the wave's halves.  A key fragment of
+        // the latent part serves the score product and the dP product.
+        f32x4 s_acc = {0.f, 0.f, 0.f, 0.f}, dp_acc = {0.f, 0.f, 0.f, 0.f};
         bf16x8 ring[AHEAD];
-        auto key_fragment = [&](auto tag) { return natural_fragment<WIDTH>(keys, lq, decltype(tag)::value, g); };
+        auto key_fragment = [&](auto tag) {
+            return quadrant_fragment<WIDTH>(keys, 16 * key_half + l16, decltype(tag)::value, quad);
+        };
         fill_ring(ring, key_fragment);
-        fragment_stream<QK_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
-            constexpr int KS = decltype(tag)::value;
-            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, qf[KS], s_acc, 0, 0, 0);
-            if constexpr (KS < V_STEPS) {
-                dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, dof[KS], dp_acc, 0, 0, 0);
+        fragment_stream<Q_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int S = decltype(tag)::value;
+            s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, qf[S], s_acc, 0, 0, 0);
+            if constexpr (S < O_STEPS) {
+                dp_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, dof[S], dp_acc, 0, 0, 0);
             }
         });
 
@@ -334,25 +383,21 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
         };
         fill_ring(ring, column_fragment);
 
+        {
+            float ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = key0 + 16 * key_half + 4 * quad + i;
+                float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -row_lse2));
+                if (k > row_token) probability = 0.f;
+                ds[i] = probability * (dp_acc[i] - row_delta) * scale;
+            }
+            exchange_store(exchange, 16 * row_half + l16, 16 * key_half + 4 * quad, ds);   // [row][key]
+        }
+        __syncthreads();   // the four quadrants are in place
         bf16x8 dsf[2];
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            u32x4 packed;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float ds[2];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const int i = 8 * n + 2 * j + e;
-                    const int k = key0 + 8 * (i / 4) + 4 * g + i % 4;
-                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -row_lse2));
-                    if (k > row_token) probability = 0.f;
-                    ds[e] = probability * (dp_acc[i] - row_delta) * scale;
-                }
-                packed[j] = pack_bf16(ds[0], ds[1]);
-            }
-            dsf[n] = __builtin_bit_cast(bf16x8, packed);
-        }
+        for (int n = 0; n < 2; ++n) dsf[n] = exchange_fragment(exchange, lq, g, n);
         fragment_stream<2 * OWN>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
             constexpr int J = decltype(tag)::value / 2;
             constexpr int N = decltype(tag)::value % 2;
@@ -388,7 +433,9 @@ struct KeyGradLayout {
     static constexpr int Q_ROWS = 0;                                  // [32 rows][576]
     static constexpr int DO_ROWS = Q_ROWS + Tile32<WIDTH>::BYTES;     // [32 rows][512]
     static constexpr int STATS = DO_ROWS + Tile32<RANK>::BYTES;
-    static constexpr int LDS_BYTES = STATS + 3 * TILE * 4;
+    static constexpr int BUFFER_BYTES = STATS + 3 * TILE * 4;
+    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;                 // the tile being multiplied and the next one
+    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_BYTES;   // P and dS
 };
 
 constexpr int PARTIAL_FLOATS = TILE * WIDTH;   // one slot of partial key gradients: [32 keys][576] fp32
@@ -403,16 +450,13 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int batch_size, int sequence_length,
     int heads, int ranges, float scale) {
     using L = KeyGradLayout;
-    constexpr int QK_STEPS = WIDTH / 16;   // 36
-    constexpr int V_STEPS = RANK / 16;     // 32
+    constexpr int Q_STEPS = WIDTH / 32;    // 18
+    constexpr int O_STEPS = RANK / 32;     // 16
     constexpr int AHEAD = 6;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* q_rows = lds + L::Q_ROWS;
-    unsigned char* do_rows = lds + L::DO_ROWS;
-    float* lse2 = reinterpret_cast<float*>(lds + L::STATS);
-    float* delta = lse2 + TILE;
-    int* token_of = reinterpret_cast<int*>(delta + TILE);
+    unsigned char* p_exchange = lds + L::EXCHANGE;
+    unsigned char* ds_exchange = p_exchange + EXCHANGE_BYTES;
 
     const int tid = threadIdx.x;
     const int wave = tid / 64;
@@ -424,6 +468,10 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     const float c = scale * LOG2E;
     const int q_transposed_at = transposed_lane_offset<WIDTH>(lane);
     const int do_transposed_at = transposed_lane_offset<RANK>(lane);
+    const int row_half = wave / 2;
+    const int key_half = wave % 2;
+    const int l16 = lane % 16;
+    const int quad = lane / 16;
 
     const index_math::KeyVisits visits = index_math::key_visits(T, heads);
     const long long per_batch = visits.per_batch();
@@ -460,21 +508,13 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
         const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
         const float* lse_batch = logsumexp + (size_t)batch * heads * T;
 
-        // this segment's keys as B operands (column = key lq); the value operand is the latent part
-        bf16x8 kf[QK_STEPS];
+        // this wave's quadrant of the score tile: rows 16*row_half .. +15 x keys 16*key_half .. +15.  Its keys as
+        // B operands (column = key l16); the value operand is the latent part
+        bf16x8 kf[Q_STEPS];
         {
-            const bool valid = key < T;
-            const size_t k = valid ? key : 0;
-#pragma unroll
-            for (int ks = 0; ks < QK_STEPS; ++ks) {
-                u32x4 bits = {0, 0, 0, 0};
-                if (valid) {
-                    const bf16_t* source = ks < V_STEPS ? latent + k * RANK + 16 * ks + 8 * g
-                                                        : rope + k * ROPE + 16 * (ks - V_STEPS) + 8 * g;
-                    bits = *reinterpret_cast<const u32x4*>(source);
-                }
-                kf[ks] = __builtin_bit_cast(bf16x8, bits);
-            }
+            const int own_key = k0 + 16 * key_half + l16;
+            const size_t k = own_key < T ? own_key : 0;
+            fetch_quadrant_operand(kf, latent + k * RANK, rope + k * ROPE, own_key < T, quad);
         }
 
         f32x16 latent_acc[4], rope_acc;   // column blocks 4*wave + j of the latent, block wave%2 of the rope part
@@ -495,40 +535,61 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
                 statistics = fetch_row_statistics(delta_of_rows, lse_batch, batch_row0, row0 + tid, rows, heads, T);
             }
         };
+        auto place_rows = [&](int tile) {
+            unsigned char* buffer = lds + ((tile - first_tile) & 1) * L::BUFFER_BYTES;
+            place_tile<WIDTH>(q_share, buffer + L::Q_ROWS, 0, tid);
+            place_tile<WIDTH>(rope_share, buffer + L::Q_ROWS, RANK, tid);
+            place_tile<RANK>(do_share, buffer + L::DO_ROWS, 0, tid);
+            if (tid < TILE) {
+                float* lse2 = reinterpret_cast<float*>(buffer + L::STATS);
+                lse2[tid] = statistics.lse2;
+                lse2[TILE + tid] = statistics.delta;
+                reinterpret_cast<int*>(lse2)[2 * TILE + tid] = statistics.token;
+            }
+        };
+        // Tile t is multiplied out of one buffer while tile t + 1 goes from registers into the other and tile
+        // t + 2 is on its way from memory: a fetch has a whole step to arrive, and a step has one barrier.
         fetch_rows(first_tile);
+        __syncthreads();   // the previous segment has been read
+        place_rows(first_tile);
+        if (first_tile + 1 < end_tile) fetch_rows(first_tile + 1);
 
         for (int tile = first_tile; tile < end_tile; ++tile) {
-            __syncthreads();   // the previous tile has been read
-            place_tile<WIDTH>(q_share, q_rows, 0, tid);
-            place_tile<WIDTH>(rope_share, q_rows, RANK, tid);
-            place_tile<RANK>(do_share, do_rows, 0, tid);
-            if (tid < TILE) {
-                lse2[tid] = statistics.lse2;
-                delta[tid] = statistics.delta;
-                token_of[tid] = statistics.token;
+            const unsigned char* buffer = lds + ((tile - first_tile) & 1) * L::BUFFER_BYTES;
+            const unsigned char* q_rows = buffer + L::Q_ROWS;
+            const unsigned char* do_rows = buffer + L::DO_ROWS;
+            const float* lse2 = reinterpret_cast<const float*>(buffer + L::STATS);
+            const float* delta = lse2 + TILE;
+            const int* token_of = reinterpret_cast<const int*>(delta + TILE);
+            __syncthreads();   // this tile is in place, the other buffer has been read
+            if (tile + 1 < end_tile) {
+                place_rows(tile + 1);
+                if (tile + 2 < end_tile) fetch_rows(tile + 2);
             }
-            __syncthreads();
-            if (tile + 1 < end_tile) fetch_rows(tile + 1);   // in flight while this tile is multiplied
 
-            f32x16 s_acc, dp_acc;   // (rows x keys): lane holds key lq and tile rows 8*(i/4) + 4*g + i%4
-            clear(s_acc);
-            clear(dp_acc);
+            // (rows x keys) quadrant: lane holds key l16 and rows 4*quad .. +3 of the wave's halves; the score and dP
+            // products take turns
+            f32x4 s_acc = {0.f, 0.f, 0.f, 0.f}, dp_acc = {0.f, 0.f, 0.f, 0.f};
             bf16x8 ring[AHEAD];
             auto row_fragment = [&](auto tag) {
                 constexpr int I = decltype(tag)::value;
-                if constexpr (I < QK_STEPS) {
-                    return natural_fragment<WIDTH>(q_rows, lq, I, g);
+                if constexpr (I >= 2 * O_STEPS) {
+                    return quadrant_fragment<WIDTH>(q_rows, 16 * row_half + l16, I - O_STEPS, quad);
+                } else if constexpr (I % 2 == 0) {
+                    return quadrant_fragment<WIDTH>(q_rows, 16 * row_half + l16, I / 2, quad);
                 } else {
-                    return natural_fragment<RANK>(do_rows, lq, I - QK_STEPS, g);
+                    return quadrant_fragment<RANK>(do_rows, 16 * row_half + l16, I / 2, quad);
                 }
             };
             fill_ring(ring, row_fragment);
-            fragment_stream<QK_STEPS + V_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
+            fragment_stream<Q_STEPS + O_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
                 constexpr int I = decltype(tag)::value;
-                if constexpr (I < QK_STEPS) {
-                    s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[I], s_acc, 0, 0, 0);
+                if constexpr (I >= 2 * O_STEPS) {
+                    s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I - O_STEPS], s_acc, 0, 0, 0);
+                } else if constexpr (I % 2 == 0) {
+                    s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I / 2], s_acc, 0, 0, 0);
                 } else {
-                    dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, kf[I - QK_STEPS], dp_acc, 0, 0, 0);
+                    dp_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I / 2], dp_acc, 0, 0, 0);
                 }
             });
 
@@ -547,33 +608,29 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
             };
             fill_ring(ring, column_fragment);
 
+            {
+                const int local = 16 * row_half + 4 * quad;
+                const int own_key = k0 + 16 * key_half + l16;
+                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
+                const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
+                const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+                float p[4], ds[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[i]));
+                    if (own_key > (int)token4[i]) probability = 0.f;
+                    p[i] = probability;
+                    ds[i] = probability * (dp_acc[i] - delta4[i]) * scale;
+                }
+                exchange_store(p_exchange, 16 * key_half + l16, local, p);     // [key][row]
+                exchange_store(ds_exchange, 16 * key_half + l16, local, ds);
+            }
+            __syncthreads();   // the four quadrants are in place
             bf16x8 pf[2], dsf[2];
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                u32x4 p_packed, ds_packed;
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int i4 = 2 * n + half;
-                    const int local = 8 * i4 + 4 * g;
-                    const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
-                    const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
-                    const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
-                    float p[4], ds[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int i = 4 * i4 + e;
-                        float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[e]));
-                        if (key > (int)token4[e]) probability = 0.f;
-                        p[e] = probability;
-                        ds[e] = probability * (dp_acc[i] - delta4[e]) * scale;
-                    }
-                    p_packed[2 * half] = pack_bf16(p[0], p[1]);
-                    p_packed[2 * half + 1] = pack_bf16(p[2], p[3]);
-                    ds_packed[2 * half] = pack_bf16(ds[0], ds[1]);
-                    ds_packed[2 * half + 1] = pack_bf16(ds[2], ds[3]);
-                }
-                pf[n] = __builtin_bit_cast(bf16x8, p_packed);
-                dsf[n] = __builtin_bit_cast(bf16x8, ds_packed);
+                pf[n] = exchange_fragment(p_exchange, lq, g, n);
+                dsf[n] = exchange_fragment(ds_exchange, lq, g, n);
             }
             fragment_stream<18>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
                 constexpr int N = decltype(tag)::value / 9;
