@@ -6,25 +6,25 @@
 // the decomposition below is built around 64-lane MFMA waves and the 160 KB
 // LDS and shares nothing with their per-head scalar loops.
 //
-// Rows and tiles
+// Rows and units
 //   A workgroup (4 waves) owns 128 "rows" -- the heads of one sequence in
 //   decode, consecutive (token, head) pairs in prefill -- and walks the key
-//   stream in tiles of 64 tokens.  Every row of a workgroup reads the same
-//   keys, so a 72 KB tile is fetched from HBM once and feeds 128 rows x
+//   stream in units of 32 tokens.  Every row of a workgroup reads the same
+//   keys, so a 36 KB unit is fetched from HBM once and feeds 128 rows x
 //   (576 + 512) x 2 flop per token: the only way the 242 flop/byte of the
 //   H = 128 decode stays on the HBM roofline.  Each wave owns 32 rows: the
-//   scores are produced transposed, S^T (64 keys x 32 rows) = K_tile Q^T with
+//   scores are produced transposed, S^T (32 keys x 32 rows) = K_unit Q^T with
 //   Q held in registers (36 k-steps), and O^T (512 x 32 rows) += V^T P^T is
 //   accumulated in 256 accumulator registers per lane.
 //
 // One LDS copy serves K and V
-//   V is the first 512 columns of the same rows.  The tile is stored once,
+//   V is the first 512 columns of the same rows.  A unit is stored once,
 //   row-major, and read two ways: 16-byte row reads for the K operand, and
 //   ds_read_b64_tr_b16 (a 4 keys x 16 columns block transposed across 16
-//   lanes) for the V^T operand.  Two stages of 72 KB double-buffer the stream.
+//   lanes) for the V^T operand.  A ring of four 36 KB slots holds the stream.
 //
 // Global -> LDS without registers
-//   Tiles arrive by global_load_lds (16 bytes per lane, a wave instruction
+//   Units arrive by global_load_lds (16 bytes per lane, a wave instruction
 //   fills 1 KB of consecutive LDS).  With no padding possible inside that 1 KB
 //   the bank spread comes from a swizzle applied on the global side: the
 //   16-byte chunk c of row r lives at slot 72*r + (c ^ f(r)), f(r) = the three
@@ -34,7 +34,7 @@
 //   base plus an immediate.
 //
 // Scheduling (decode)
-//   The tiles of all sequences form one list that is cut into equal ranges,
+//   The 64-token tiles of all sequences form one list that is cut into equal ranges,
 //   one per workgroup (one workgroup per CU), so uneven lengths balance to
 //   within a tile.  The cut is a small table (the plan) that a one-workgroup
 //   kernel derives from the lengths on the device, so the call stays
@@ -63,13 +63,11 @@ namespace {
 constexpr int RANK = 512;
 constexpr int ROPE = 64;
 constexpr int WIDTH = RANK + ROPE;
-constexpr int BN = 64;                      // keys per tile
+constexpr int BN = 64;                      // keys per tile, the grain of the decode work list
 constexpr int ROWS = 128;                   // rows per workgroup
 constexpr int THREADS = 256;
 constexpr int CHUNKS = WIDTH / 8;           // 72 16-byte chunks per key row
 constexpr int ROW_BYTES = CHUNKS * 16;      // 1152
-constexpr int STAGE_BYTES = BN * ROW_BYTES; // 73728
-constexpr int LOADS_PER_THREAD = BN * CHUNKS / THREADS;  // 18
 constexpr int KSTEPS = WIDTH / 16;          // 36
 constexpr int DBLOCKS = RANK / 32;          // 16
 constexpr int EPILOGUE_PITCH = 1024 + 16;   // bytes per staged output row
@@ -92,88 +90,6 @@ struct KeyStream {
     const int* block_table;    // nullptr: tokens are stored contiguously
     int page_size;
 };
-
-// Where one 64-token tile comes from and goes to.  Tokens past the last visible
-// one are clamped to it (their rows are zeroed after arrival), so no byte
-// outside the visible part of the sequence is ever read.
-//
-// Wave w fills rows 16w .. 16w+15 (18 instructions of 64 slots = 16 rows of 72
-// slots), so every row / position split is a compile-time constant plus one
-// compare on the lane id.
-//
-// `contiguous`: the tile is one run of 576-wide rows (packed cache, and either
-// no paging or pages that hold whole tiles): a uniform 64-bit base plus a
-// 32-bit per-lane offset, about eight integer ops per load.  Such loads are
-// cheap enough to be issued one at a time between the MFMA groups of the tile
-// being consumed, which keeps the memory pipeline fed without ever stalling a
-// wave on a full request queue.
-struct TileSource {
-    const bf16_t* tile_base;   // contiguous form only
-    unsigned lds_base;         // LDS byte offset of this wave's 18 KB
-    int key0;
-    int row_limit;             // rows above it are clamped (>= 0: the tile holds a visible token)
-    bool contiguous;
-    bool enabled;
-};
-
-__device__ __forceinline__ TileSource locate_tile(unsigned char* stage_base, const KeyStream& keys, int key0,
-                                                  int last_token, int wave, bool enabled) {
-    TileSource source;
-    const bool paged = keys.block_table != nullptr;
-    const bool page_holds_tile = !paged || (keys.page_size % BN == 0);
-    const bool packed = keys.rope == keys.latent + RANK && keys.latent_stride == WIDTH && keys.rope_stride == WIDTH;
-    source.contiguous = packed && page_holds_tile;
-    source.enabled = enabled;
-    source.key0 = key0;
-    source.row_limit = last_token - key0;
-    source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(stage_base) + wave * (LOADS_PER_THREAD * 1024));
-    source.tile_base = keys.latent;
-    if (enabled && source.contiguous) {
-        long long tile_physical = key0;
-        if (paged) {
-            const int page = keys.block_table[key0 / keys.page_size];
-            tile_physical = (long long)page * keys.page_size + key0 % keys.page_size;
-        }
-        source.tile_base = keys.latent + tile_physical * WIDTH;
-    }
-    return source;
-}
-
-// Load number i (0..17) of a contiguous tile; i is a constant after unrolling
-// (offsets: index_math::contiguous_load_offset).
-__device__ __forceinline__ void issue_contiguous_load(const TileSource& source, int wave, int i, int lane) {
-    direct_load_16_offset(source.tile_base, index_math::contiguous_load_offset<ROW_BYTES>(wave, i, lane, source.row_limit),
-                          source.lds_base + i * 1024);
-}
-
-// All 18 loads of a tile at once (first tile of a walk, and every tile of the
-// general form: per-lane page lookup and separate latent / rope tensors).
-__device__ __forceinline__ void issue_tile(const TileSource& source, const KeyStream& keys, int wave) {
-    if (!source.enabled) return;
-    if (source.contiguous) {
-#pragma unroll
-        for (int i = 0; i < LOADS_PER_THREAD; ++i) issue_contiguous_load(source, wave, i, fresh_lane_id());
-        return;
-    }
-    const int lane = fresh_lane_id();
-    const bool paged = keys.block_table != nullptr;
-#pragma unroll 1
-    for (int i = 0; i < LOADS_PER_THREAD; ++i) {
-        const int slot = 64 * i + lane;
-        const int local_row = slot / CHUNKS;
-        const int position = slot % CHUNKS;
-        const int chunk = position ^ swizzle_of_row(local_row);
-        const int token = source.key0 + min(16 * wave + local_row, source.row_limit);
-        long long physical = token;
-        if (paged) {
-            const int page = keys.block_table[token / keys.page_size];
-            physical = (long long)page * keys.page_size + token % keys.page_size;
-        }
-        const bf16_t* address = chunk < RANK / 8 ? keys.latent + physical * keys.latent_stride + 8 * chunk
-                                                 : keys.rope + physical * keys.rope_stride + 8 * (chunk - RANK / 8);
-        direct_load_16(address, source.lds_base + i * 1024);
-    }
-}
 
 // Score-chain MFMAs with the accumulator held in ordinary vector registers.
 // The compiler's own MFMAs take accumulator-file destinations in a kernel this
@@ -228,213 +144,11 @@ struct RowState {
     float row_sum;    // this lane's share of the normaliser
 };
 
-// Head room (log2 units) put between the first tile's maximum and the fixed
-// reference of the fast path, and the excess over the reference at which the
-// fast path gives up (2^80 per term leaves 2^47 of fp32 range for the sums).
+// Head room (log2 units) put between the first unit's maximum and the softmax
+// reference of a walk, and the excess over the reference at which the reference
+// is raised (2^80 per term leaves 2^47 of fp32 range for the sums).
 constexpr float FAST_HEADROOM = 40.0f;
 constexpr float FAST_LIMIT = 80.0f;
-
-// One tile for one wave: S^T = K Q^T, softmax against `limit` visible keys for
-// this lane's row, O^T += V^T P^T.
-//
-// SAFE == false (the path that normally runs): the reference is fixed once,
-// FAST_HEADROOM above the row maximum of the first tile, so the 256 output
-// accumulators are never rescaled and nothing conditional touches them (a
-// conditional rescale makes the compiler copy the whole accumulator file at
-// the join).  Scores may exceed the reference by up to FAST_LIMIT before a
-// term gets near the top of the fp32 range; `risk` reports a row that came
-// closer than that, in which case the caller discards the result and repeats
-// the walk with SAFE == true.
-// SAFE == true: textbook online softmax, the reference follows the running
-// maximum and the accumulators are rescaled on every half tile.
-template <bool SAFE>
-__device__ __forceinline__ void process_tile(RowState& state, bool& risk, const bf16x8 (&qf)[KSTEPS],
-                                             const unsigned char* stage, int key0, int limit, int wave_min_limit,
-                                             bool first, float c, int lane_id, const TileSource& next_tile, int wave) {
-    // The per-lane LDS offsets below are recomputed for every tile from an
-    // lane id read afresh (volatile, so nothing derived from it is hoisted): kept
-    // live across the loop they would be the registers that no longer fit and
-    // get spilled, and a scratch reload inside the loop stalls on the tile
-    // prefetch.
-    (void)lane_id;
-    const int lane = fresh_lane_id();
-    const int lq = lane % 32;
-    const int g = lane / 32;
-
-    // K operand: row 32*mb + lq, 16-byte chunk 2*ks + g.  (2*ks+g) ^ f only mixes
-    // the low three bits, i.e. stays inside the 128-byte group ks/4.
-    const int swz = swizzle_of_row(lq);  // rows lq and lq+32 share f (f ignores bits >= 4 of the row)
-    const unsigned char* k_row = stage + lq * ROW_BYTES;
-    const unsigned char* k_lane[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) k_lane[j] = k_row + ((2 * j + g) ^ swz) * 16;
-
-    // V^T operand through transposing reads.  In a block of 16 lanes, lane s
-    // points at row 4*g + s/4 (+8 for the second read), columns 4*(s%4)..+3 of
-    // the 16-column group 16*(block%2); the instruction hands lane i column i
-    // of the four rows.  Together: MFMA row l%32, keys {4g..4g+3, 8+4g..8+4g+3}
-    // of each 16-key step, the k-order P^T carries from the C layout.
-    const int s16 = lane % 16;
-    const int block = lane / 16;
-    const int row1 = 4 * g + s16 / 4;
-    const int f1 = swizzle_of_row(row1);
-    const int chunk_low = (2 * (block % 2) + (s16 % 4) / 2) ^ (f1 & 3);
-    // Bit 2 of f (= bit 1 of the row) moves a row's data by one 64-byte column
-    // block: rows 2,3 (mod 4) keep column block d at position block d ^ 1.  The
-    // lanes addressing those rows therefore read 64 bytes further (even d) or
-    // nearer (odd d), which two base pointers per read turn back into immediates.
-    const int flip = 64 * ((row1 >> 1) & 1);
-    const unsigned char* v_lane1 = stage + row1 * ROW_BYTES + chunk_low * 16 + 8 * (s16 & 1);
-    const unsigned char* v_lane2 = stage + (row1 + 8) * ROW_BYTES + (chunk_low ^ 1) * 16 + 8 * (s16 & 1);
-    const unsigned char* v_base1[2] = {v_lane1 + flip, v_lane1 - flip};
-    const unsigned char* v_base2[2] = {v_lane2 + flip, v_lane2 - flip};
-
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    typedef __attribute__((address_space(3))) s16x4* tr_pointer;
-
-    // The tile is consumed in two halves of 32 keys so that only 16 score and 8
-    // probability registers are live beside the 256 accumulators and 144 Q
-    // registers.  Operand reads are software-pipelined by hand in groups of four
-    // MFMAs (the scheduler barrier keeps the compiler from hoisting a whole
-    // half's reads, which would push Q out to scratch).
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-        // The 256 output accumulators fill the accumulator register file exactly,
-        // and a compiler-issued MFMA would want 16 more of them for the scores.
-        // The score chain is therefore issued by hand with its accumulator in
-        // ordinary registers (score_mfma_*).
-        f32x16 s_acc, s_odd;
-        {
-            constexpr int WIDTH_K = 4;   // K fragments per pipeline group
-            constexpr int GROUPS = KSTEPS / WIDTH_K;
-            bf16x8 current[WIDTH_K], next[WIDTH_K];
-            auto fragment = [&](int ks) {
-                return *reinterpret_cast<const bf16x8*>(k_lane[ks % 4] + mb * 32 * ROW_BYTES + (ks / 4) * 128);
-            };
-#pragma unroll
-            for (int j = 0; j < WIDTH_K; ++j) current[j] = fragment(j);
-#pragma unroll
-            for (int group = 0; group < GROUPS; ++group) {
-                if (group + 1 < GROUPS) {
-#pragma unroll
-                    for (int j = 0; j < WIDTH_K; ++j) next[j] = fragment(WIDTH_K * (group + 1) + j);
-                }
-#pragma unroll
-                for (int j = 0; j < WIDTH_K; ++j) {
-                    // two interleaved chains (even / odd k-steps): a dependent MFMA
-                    // would otherwise wait out the previous one's full latency
-                    const int ks = WIDTH_K * group + j;
-                    f32x16& chain = (ks % 2 == 0) ? s_acc : s_odd;
-                    if (ks < 2) {
-                        score_mfma_first(chain, current[j], qf[ks]);
-                    } else if (ks >= KSTEPS - 2) {
-                        score_mfma_last(chain, current[j], qf[ks]);
-                    } else {
-                        score_mfma(chain, current[j], qf[ks]);
-                    }
-                }
-                // the next tile's loads ride along with the first half's MFMA groups
-                if (mb == 0 && next_tile.enabled && next_tile.contiguous) issue_contiguous_load(next_tile, wave, group, lane);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 0; j < WIDTH_K; ++j) current[j] = next[j];
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s_acc[i] += s_odd[i];
-        }
-
-        if (key0 + 32 * mb + 32 > wave_min_limit) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int k = key0 + 32 * mb + 8 * (i / 4) + 4 * g + (i % 4);
-                if (k >= limit) s_acc[i] = -INFINITY;
-            }
-        }
-
-        float tile_max = s_acc[0];
-#pragma unroll
-        for (int i = 1; i < 16; ++i) tile_max = fmaxf(tile_max, s_acc[i]);
-        tile_max = half_wave_max(tile_max) * c;  // log2 units from here on
-
-        if (SAFE) {
-            const float new_reference = fmaxf(state.reference, tile_max);
-            const float alpha = __builtin_amdgcn_exp2f(state.reference - new_reference);
-            state.reference = new_reference;
-            state.row_sum *= alpha;
-#pragma unroll
-            for (int d = 0; d < DBLOCKS; ++d) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) state.o[d][i] *= alpha;
-                __builtin_amdgcn_sched_barrier(0);  // one block at a time through the ordinary registers
-            }
-        } else {
-            if (first && mb == 0) state.reference = tile_max + FAST_HEADROOM;
-            risk = risk || (tile_max - state.reference > FAST_LIMIT);
-        }
-
-        const float offset = state.reference;
-        bf16x8 pf[2];
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            u32x4 packed;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = 8 * n + 2 * j;
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -offset));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[i + 1], c, -offset));
-                state.row_sum += p0 + p1;
-                packed[j] = pack_bf16(p0, p1);
-            }
-            pf[n] = __builtin_bit_cast(bf16x8, packed);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-
-        {
-            // 32 MFMAs (2 key steps x 16 column blocks) in 8 groups of four column blocks
-            constexpr int WIDTH_G = 4;
-            constexpr int GROUPS = 2 * DBLOCKS / WIDTH_G;
-            s16x4 cur_lo[WIDTH_G], cur_hi[WIDTH_G], next_lo[WIDTH_G], next_hi[WIDTH_G];
-            auto step_of = [&](int group, int j) {
-                const int n = group / (DBLOCKS / WIDTH_G);
-                const int d = WIDTH_G * (group % (DBLOCKS / WIDTH_G)) + j;
-                return (2 * mb + n) * 16 * ROW_BYTES + d * 64;
-            };
-#pragma unroll
-            for (int j = 0; j < WIDTH_G; ++j) {
-                cur_lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base1[j % 2] + step_of(0, j)));
-                cur_hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base2[j % 2] + step_of(0, j)));
-            }
-#pragma unroll
-            for (int group = 0; group < GROUPS; ++group) {
-                if (group + 1 < GROUPS) {
-#pragma unroll
-                    for (int j = 0; j < WIDTH_G; ++j) {
-                        next_lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base1[j % 2] + step_of(group + 1, j)));
-                        next_hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_pointer)(v_base2[j % 2] + step_of(group + 1, j)));
-                    }
-                }
-                const int n = group / (DBLOCKS / WIDTH_G);
-#pragma unroll
-                for (int j = 0; j < WIDTH_G; ++j) {
-                    const int d = WIDTH_G * (group % (DBLOCKS / WIDTH_G)) + j;
-                    const s16x8 both = __builtin_shufflevector(cur_lo[j], cur_hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
-                    state.o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n], state.o[d], 0, 0, 0);
-                }
-                if (mb == 0 && next_tile.enabled && next_tile.contiguous) {
-                    issue_contiguous_load(next_tile, wave, KSTEPS / 4 + group, lane);
-                    if (group == GROUPS - 1) issue_contiguous_load(next_tile, wave, LOADS_PER_THREAD - 1, lane);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 0; j < WIDTH_G; ++j) {
-                    cur_lo[j] = next_lo[j];
-                    cur_hi[j] = next_hi[j];
-                }
-            }
-        }
-    }
-}
 
 // Column of the output a lane's accumulator register stands for.
 __device__ __forceinline__ constexpr int output_column(int d, int i4, int g) {
@@ -489,16 +203,6 @@ __device__ __forceinline__ void store_partial(const RowState& state, unsigned ch
     }
 }
 
-// Zero the rows of a landed tile that lie past the end of the sequence, so that
-// stale cache contents (possibly NaN) cannot reach the V operand.
-__device__ __forceinline__ void zero_tail_rows(unsigned char* stage, int first_invalid_row, int tid) {
-    const int chunks = (BN - first_invalid_row) * CHUNKS;
-    const u32x4 zero = {0, 0, 0, 0};
-    for (int index = tid; index < chunks; index += THREADS) {
-        *reinterpret_cast<u32x4*>(stage + first_invalid_row * ROW_BYTES + index * 16) = zero;
-    }
-}
-
 __device__ __forceinline__ void load_query(bf16x8 (&qf)[KSTEPS], const bf16_t* latent_row, const bf16_t* rope_row,
                                            bool valid, int g) {
 #pragma unroll
@@ -522,77 +226,15 @@ __device__ __forceinline__ void reset(RowState& state) {
     state.row_sum = 0.f;
 }
 
-// Walk tiles [tile_begin, tile_end) of one key stream for the 128 rows of this
-// workgroup, starting from cleared accumulators.  `limit` is this lane's row's
-// number of visible keys; every row must see at least one key of the first
-// tile.  Every wave processes every tile (rows that see nothing of a tile
-// simply get zero probabilities), so the accumulators never pass through a
-// conditional.  Returns this wave's overflow-risk flag (always false for SAFE).
-template <bool SAFE>
-__device__ __forceinline__ bool walk_tiles(RowState& state, const bf16x8 (&qf)[KSTEPS], unsigned char* lds,
-                                           const KeyStream& keys, int tile_begin, int tile_end, int tokens, int limit,
-                                           float c, int tid) {
-    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int lane = tid % 64;
-    int wave_min_limit = limit;  // wave-uniform: below it no masking is needed
-#pragma unroll
-    for (int offset = 1; offset < 64; offset <<= 1) {
-        wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, offset));
-    }
-    wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
-    reset(state);
-    bool risk = false;
-    const int last_token = tokens - 1;
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
-        unsigned char* stage = lds + (tile & 1) * STAGE_BYTES;
-        // This tile was requested while the previous one was consumed (the first one by
-        // walk_rows, ahead of the query loads, which this wait drains as well: a wait
-        // for them further down would also wait for the prefetch kept in flight there).
-        wait_vector_memory<0>();
-        workgroup_barrier();   // everybody's share has landed, everybody has left the previous tile
-        const int key0 = tile * BN;
-        if (key0 + BN > tokens) {
-            zero_tail_rows(stage, tokens - key0, tid);
-            workgroup_barrier();
-        }
-        // The other stage was last read for tile-1, which every wave has left.
-        const TileSource next_tile = locate_tile(lds + ((tile + 1) & 1) * STAGE_BYTES, keys, (tile + 1) * BN, last_token,
-                                                 wave, tile + 1 < tile_end);
-        if (!next_tile.contiguous) issue_tile(next_tile, keys, wave);
-        process_tile<SAFE>(state, risk, qf, stage, key0, limit, wave_min_limit, tile == tile_begin, c, lane, next_tile,
-                           wave);
-    }
-    workgroup_barrier();   // the stages are free: the caller stages its results through them
-    return risk;
-}
-
-// Loads the query fragments of this lane's row and walks the tiles with one
-// variant.  Returns whether any wave of the workgroup reported overflow risk
-// (workgroup-uniform; always false for SAFE).
-template <bool SAFE>
-__device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_latent_row,
-                                          const bf16_t* query_rope_row, bool valid, unsigned char* lds,
-                                          const KeyStream& keys, int tile_begin, int tile_end, int tokens, int limit,
-                                          float c, int tid) {
-    // the first tile goes on its way before the query rows: both latencies overlap
-    issue_tile(locate_tile(lds + (tile_begin & 1) * STAGE_BYTES, keys, tile_begin * BN, tokens - 1,
-                           __builtin_amdgcn_readfirstlane(tid / 64), true), keys, __builtin_amdgcn_readfirstlane(tid / 64));
-    bf16x8 qf[KSTEPS];
-    load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
-    const bool risk = walk_tiles<SAFE>(state, qf, lds, keys, tile_begin, tile_end, tokens, limit, c, tid);
-    if (SAFE) return false;
-    return __syncthreads_or(risk) != 0;
-}
-
 // ----------------------------------------------------------------------------
-// The decode walk of the fast path (SAFE == false): 32-key units, one matrix stream
+// The walk: 32-key units, one matrix stream
 // ----------------------------------------------------------------------------
 //
 // With one wave per SIMD nothing hides the vector arithmetic of the softmax unless the
-// wave's own instruction stream does: the tile loop above computes scores, then
-// probabilities, then the output update, and the matrix pipeline idles through the
-// middle third.  Here the key stream is consumed in units of 32 keys and the work of
-// consecutive units is overlapped by hand:
+// wave's own instruction stream does: a loop that computes scores, then probabilities,
+// then the output update leaves the matrix pipeline idle through the middle third.  Here
+// the key stream is consumed in units of 32 keys and the work of consecutive units is
+// overlapped by hand:
 //
 //     step u:   S(u+1) = K(u+1) Q^T   36 MFMAs, with the softmax of S(u) -> P(u)
 //                                     (exp2, sums, bf16 packing) issued between them
@@ -603,7 +245,7 @@ __device__ __forceinline__ bool walk_rows(RowState& state, const bf16_t* query_l
 // time (one being accumulated, one being turned into probabilities), so the steps
 // alternate between two register sets.
 //
-// Units sit in a ring of four LDS slots (the same 144 KB as the two tile stages).
+// Units sit in a ring of four LDS slots (144 KB).
 // Unit u+3 is requested during step u into the slot that unit u-1 left at the end of
 // step u-1; unit u+1, requested two steps earlier, must have landed when step u
 // starts: the wave waits for all but its youngest nine loads (its share of unit
@@ -616,7 +258,6 @@ constexpr int UNIT_BYTES = UNIT * ROW_BYTES;              // 36 KB
 constexpr int UNIT_SLOTS = 4;
 constexpr int UNIT_LOADS = UNIT * CHUNKS / THREADS;       // 9 wave instructions of 1 KB per wave and unit
 constexpr int STREAM_RING = 6;                            // fragments read ahead of the MFMA that takes them
-static_assert(UNIT_SLOTS * UNIT_BYTES == 2 * STAGE_BYTES, "the unit ring occupies the two tile stages");
 static_assert(UNIT_LOADS * THREADS == UNIT * CHUNKS, "unit loads must divide evenly");
 
 struct UnitSource {
@@ -719,7 +360,7 @@ __device__ __forceinline__ void issue_unit_load(const UnitSource& source, const 
 }
 
 // All nine loads of a unit at once: the first units of a walk, and every unit of the
-// general form (per-lane page lookup).
+// general form (per-lane page lookup, or latent and rope parts in tensors of their own).
 __device__ __forceinline__ void issue_unit(const UnitSource& source, const FullUnitOffsets& offsets, const KeyStream& keys,
                                            int wave) {
     if (!source.enabled) return;
@@ -729,15 +370,21 @@ __device__ __forceinline__ void issue_unit(const UnitSource& source, const FullU
         for (int i = 0; i < UNIT_LOADS; ++i) issue_unit_load(source, offsets, wave, i, lane);
         return;
     }
+    const bool paged = keys.block_table != nullptr;
 #pragma unroll 1
     for (int i = 0; i < UNIT_LOADS; ++i) {
         const int slot = 64 * i + lane;
         const int row = (UNIT / 4) * wave + slot / CHUNKS;
         const int chunk = (slot % CHUNKS) ^ swizzle_of_row(row);
         const int token = source.key0 + min(row, source.row_limit);
-        const int page = keys.block_table[token / keys.page_size];
-        const long long physical = (long long)page * keys.page_size + token % keys.page_size;
-        direct_load_16(keys.latent + physical * WIDTH + 8 * chunk, source.lds_base + i * 1024);
+        long long physical = token;
+        if (paged) {
+            const int page = keys.block_table[token / keys.page_size];
+            physical = (long long)page * keys.page_size + token % keys.page_size;
+        }
+        const bf16_t* address = chunk < RANK / 8 ? keys.latent + physical * keys.latent_stride + 8 * chunk
+                                                 : keys.rope + physical * keys.rope_stride + 8 * (chunk - RANK / 8);
+        direct_load_16(address, source.lds_base + i * 1024);
     }
 }
 
@@ -855,7 +502,7 @@ __device__ __forceinline__ void raise_reference(RowState& state, float& offset, 
 template <bool HAS_NEXT>
 __device__ __forceinline__ void unit_step(RowState& state, f32x16& scores, f32x16& next_scores,
                                           const bf16x8 (&qf)[KSTEPS], const UnitReads& reads,
-                                          const unsigned char* current, const unsigned char* next, int key0, int tokens,
+                                          const unsigned char* current, const unsigned char* next, int key0, int tokens,  // tokens: of the lane's row
                                           float c, const UnitSource& request, const FullUnitOffsets& offsets,
                                           const KeyStream& keys, int wave) {
     constexpr int SCORE_MFMAS = HAS_NEXT ? KSTEPS : 0;
@@ -947,12 +594,16 @@ __device__ __forceinline__ void unit_step(RowState& state, f32x16& scores, f32x1
     });
 }
 
-// Walk tiles [tile_begin, tile_end) of one sequence of the decode cache for the 128 heads of
-// this workgroup with the unit stream, from cleared accumulators.  Every lane's row sees all
-// `tokens` keys (see raise_reference for what happens when a row outruns its softmax reference).
-__device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_row, bool valid, unsigned char* lds,
-                                           const KeyStream& keys, int tile_begin, int tile_end, int tokens, float c,
-                                           int tid, bool cold) {
+// Walk tiles [tile_begin, tile_end) of one sequence of keys for the 128 rows of this workgroup
+// with the unit stream, from cleared accumulators (see raise_reference for what happens when a
+// row outruns its softmax reference).  Decode: the rows are the heads of one sequence, each sees
+// all `tokens` keys of the packed cache.  PREFILL: the rows are (token, head) pairs, a lane's row
+// sees the first `row_tokens` <= `tokens` keys (at least one), and the latent and rope parts of
+// the keys lie in tensors of their own.
+template <bool PREFILL>
+__device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_latent_row, const bf16_t* query_rope_row,
+                                           bool valid, unsigned char* lds, const KeyStream& keys, int tile_begin,
+                                           int tile_end, int tokens, int row_tokens, float c, int tid, bool cold) {
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int last_token = tokens - 1;
     const int unit_begin = (BN / UNIT) * tile_begin;
@@ -963,6 +614,8 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     // of its latency: then only what the first scores need is asked for first, the rest once that has arrived.
     UnitCursor cursor;
     cursor.init(keys, unit_begin, last_token);
+    if constexpr (PREFILL) cursor.contiguous = false;   // latent and rope parts come from tensors of their own
+    const int visible = PREFILL ? row_tokens : tokens;   // keys the lane's row sees
     FullUnitOffsets offsets;
     offsets.init(wave, fresh_lane_id());
     issue_unit(cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
@@ -970,7 +623,7 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     const UnitSource third = cursor.next(lds, keys, last_token, wave, unit_end);
     if (!cold) issue_unit(second, offsets, keys, wave);
     bf16x8 qf[KSTEPS];
-    load_query(qf, query_row, query_row + RANK, valid, (tid % 64) / 32);
+    load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
     if (!cold) issue_unit(third, offsets, keys, wave);
     reset(state);
     UnitReads reads;
@@ -987,7 +640,7 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     f32x16 scores_a, scores_b;
     unit_scores(scores_a, qf, slot_of(unit_begin), reads);
     {
-        mask_unit_scores(scores_a, unit_begin * UNIT, tokens, fresh_lane_id() / 32);
+        mask_unit_scores(scores_a, unit_begin * UNIT, visible, fresh_lane_id() / 32);
         float first_max = scores_a[0];
 #pragma unroll
         for (int i = 1; i < 16; ++i) first_max = fmaxf(first_max, scores_a[i]);
@@ -1007,13 +660,13 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     int unit = unit_begin;
     for (; unit + 1 < unit_end; ++unit) {
         synchronise(unit);
-        unit_step<true>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, tokens, c,
+        unit_step<true>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit + 1), unit * UNIT, visible, c,
                         cursor.next(lds, keys, last_token, wave, unit_end), offsets, keys, wave);
         // the next unit's scores take the place of this unit's (eight moves against a stream of 68 MFMAs)
         move_scores(scores_a, scores_b);
     }
     UnitSource nothing = {};
-    unit_step<false>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, tokens, c, nothing,
+    unit_step<false>(state, scores_a, scores_b, qf, reads, slot_of(unit), slot_of(unit), unit * UNIT, visible, c, nothing,
                      offsets, keys, wave);
     workgroup_barrier();   // the slots are free: the caller stages its results through them
 }
@@ -1241,7 +894,8 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
         keys.rope_stride = WIDTH;
         keys.block_table = block_table + (size_t)sequence * pages_per_sequence;
         keys.page_size = page_size;
-        walk_units(state, query_row, valid, lds, keys, tile_begin, tile_end, tokens, c, tid, position == range_begin);
+        walk_units<false>(state, query_row, query_row + RANK, valid, lds, keys, tile_begin, tile_end, tokens, tokens, c, tid,
+                          position == range_begin);
         const float total_sum = half_wave_sum(state.row_sum);
 
         if (whole) {
@@ -1406,10 +1060,8 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
     keys.rope_stride = ROPE;
     keys.block_table = nullptr;
     keys.page_size = 0;
-    // This entry point is kept for interface parity at the reference's shapes; it
-    // always takes the rescaling variant, which needs no overflow fallback.
-    walk_rows<true>(state, query_latent + global_row * RANK, query_rope + global_row * ROPE, valid, lds, keys, 0,
-                    tiles_of(visible), visible, token + 1, c, tid);
+    walk_units<true>(state, query_latent + global_row * RANK, query_rope + global_row * ROPE, valid, lds, keys, 0,
+                     tiles_of(visible), visible, valid ? token + 1 : visible, c, tid, true);
 
     if (!wave_active) return;
     const float total_sum = half_wave_sum(state.row_sum);
@@ -1424,7 +1076,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_forward_kernel(
     });
 }
 
-constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+constexpr int LDS_BYTES = UNIT_SLOTS * UNIT_BYTES;
 
 template <typename Kernel>
 void allow_large_lds(Kernel kernel) {
