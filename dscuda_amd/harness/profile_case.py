@@ -9,9 +9,10 @@ profiled ones.
     rocprofv3 --pmc SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES -d out -- python3 dscuda_amd/harness/profile_case.py decode
 
 Workloads: forward / backward (B=1, S, H=128, 192|128), decode (B=64, H=128,
-lengths ~ U[1024, 8192] seed 3), flash (B=1, H=8, S=512, D=64), copy (a plain
-16-byte-per-lane copy of 1 GiB, the calibration kernel for FETCH_SIZE /
-WRITE_SIZE).
+lengths ~ U[1024, 8192] seed 3), flash (B=1, H=8, S=512, D=64), absorbed (the
+reference's own prefill entry points, forward then backward, B=1, T=S, H heads,
+512 latent + 64 rope), copy (a plain 16-byte-per-lane copy of 1 GiB, the
+calibration kernel for FETCH_SIZE / WRITE_SIZE).
 """
 
 from __future__ import annotations
@@ -27,7 +28,7 @@ if str(ROOT) not in sys.path:
 
 def main():
     parser = argparse.ArgumentParser(description=__doc__)
-    parser.add_argument("workload", choices=("forward", "backward", "decode", "flash", "copy"))
+    parser.add_argument("workload", choices=("forward", "backward", "decode", "flash", "absorbed", "copy"))
     parser.add_argument("--steps", type=int, default=3)
     parser.add_argument("--seq", type=int, default=4096)
     parser.add_argument("--heads", type=int, default=128)
@@ -70,6 +71,19 @@ def main():
         lse = torch.empty(b, h, 1, device=device)
         scale = configs.c_float(192 ** -0.5)
         call = lambda: ops.mla_decode(query, paged, table, dl, scale, splits=8, workspace=workspace, out=out, lse=lse)
+    elif args.workload == "absorbed":
+        tokens, h = args.seq, args.heads
+        ql, qr = randn((1, tokens, h, 512), 0.25), randn((1, tokens, h, 64), 0.25)
+        latent, kr = randn((1, tokens, 512), 0.25), randn((1, tokens, 64), 0.25)
+        dout = randn((1, tokens, h, 512), 0.2)
+        out = torch.empty(1, tokens, h, 512, device=device, dtype=torch.bfloat16)
+        lse = torch.empty(1, h, tokens, device=device)
+        scale = configs.c_float(576 ** -0.5)
+        grads = tuple(torch.empty_like(x) for x in (ql, qr, latent, kr))
+
+        def call():
+            ops.mla_forward(ql, qr, latent, kr, scale, out, lse)
+            ops.mla_backward(dout, out, lse, ql, qr, latent, kr, scale, grads)
     elif args.workload == "flash":
         q, k, v = randn((1, 512, 8, 64), 1.0), randn((1, 512, 8, 64), 1.0), randn((1, 512, 8, 64), 1.0)
         out, lse = torch.empty_like(q), torch.empty(1, 8, 512, device=device)
