@@ -273,6 +273,56 @@ DSCUDA_HOST_DEVICE inline long long wide_range_of(long long total, long long ran
     return ((position + 1) * ranges - 1) / total;
 }
 
+// Large inputs (the query and dO rows of a batch element no longer stay in the caches): equal ranges would have
+// every workgroup stream its own stretch of rows from memory, one pass over all rows per key block.  Instead the
+// row tiles are cut into intervals of `length` tiles and the work into items (interval, key block), numbered
+// interval by interval, so that the workgroups running at any time walk the same few intervals and all but
+// the first of them find the rows in the caches.  Item (i, kb) exists when the block sees the interval
+// (kb * heads < end of interval i), covers the block's tiles inside it, and leaves its partial result in the
+// slot of its own number (none when it is the block's only item, i.e. the block starts in the last interval).
+struct KeyIntervals {
+    int length;      // row tiles per interval
+    int intervals;
+    int heads;
+    int key_blocks;
+    int row_tiles;
+
+    DSCUDA_HOST_DEVICE int end_of(int interval) const {
+        const long long end = (long long)(interval + 1) * length;
+        return end < row_tiles ? (int)end : row_tiles;
+    }
+    DSCUDA_HOST_DEVICE int blocks_in(int interval) const {   // key blocks 0 .. blocks_in-1 see the interval
+        const int seen = (end_of(interval) + heads - 1) / heads;
+        return seen < key_blocks ? seen : key_blocks;
+    }
+    DSCUDA_HOST_DEVICE long long items_before(int interval) const {
+        long long items = 0;
+        for (int i = 0; i < interval; ++i) items += blocks_in(i);
+        return items;
+    }
+    DSCUDA_HOST_DEVICE long long items() const { return items_before(intervals); }
+    DSCUDA_HOST_DEVICE int first_interval(int key_block) const { return (int)((long long)key_block * heads / length); }
+    // item number (within its batch element) -> interval, key block
+    DSCUDA_HOST_DEVICE void locate(long long item, int& interval, int& key_block) const {
+        interval = 0;
+        while (item >= blocks_in(interval)) {
+            item -= blocks_in(interval);
+            ++interval;
+        }
+        key_block = (int)item;
+    }
+};
+
+DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int heads, int length) {
+    KeyIntervals cut;
+    cut.length = length;
+    cut.heads = heads;
+    cut.key_blocks = (sequence_length + 31) / 32;
+    cut.row_tiles = (int)(((long long)sequence_length * heads + 31) / 32);
+    cut.intervals = (cut.row_tiles + length - 1) / length;
+    return cut;
+}
+
 constexpr long long KEY_PARTIAL_BYTES = 32LL * 576 * 4;   // one slot: [32 keys][576] fp32
 
 // How many ranges the list is cut into when `scratch_bytes` are there for the slots: one per compute unit if the

@@ -43,7 +43,9 @@
 #include "hip_common.h"
 #include "index_math.h"
 
+#include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <stdexcept>
 #include <type_traits>
 #include <string>
@@ -441,14 +443,15 @@ struct KeyGradLayout {
 constexpr int PARTIAL_FLOATS = TILE * WIDTH;   // one slot of partial key gradients: [32 keys][576] fp32
 static_assert(PARTIAL_FLOATS * 4 == index_math::KEY_PARTIAL_BYTES, "slot size");
 
-// `ranges` > 0: workgroup w walks range w of the list of visits; 0: workgroup w walks all visits of key block w
-// (numbered through the batch elements) and writes the gradients itself.
+// `interval_length` > 0: workgroup w takes item w of the interval cut (index_math.h), slot w.  Otherwise `ranges` > 0:
+// workgroup w walks range w of the list of visits; 0: workgroup w walks all visits of key block w (numbered through
+// the batch elements) and writes the gradients itself.
 __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
     const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
     const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
     const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int batch_size, int sequence_length,
-    int heads, int ranges, float scale) {
+    int heads, int ranges, int interval_length, float scale) {
     using L = KeyGradLayout;
     constexpr int Q_STEPS = WIDTH / 32;    // 18
     constexpr int O_STEPS = RANK / 32;     // 16
@@ -477,7 +480,16 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     const long long per_batch = visits.per_batch();
     const long long total = per_batch * batch_size;
     long long position, range_end;
-    if (ranges > 0) {
+    if (interval_length > 0) {
+        const index_math::KeyIntervals cut = index_math::key_intervals(T, heads, interval_length);
+        const long long items = cut.items();
+        const int batch = (int)(blockIdx.x / items);
+        int interval, key_block;
+        cut.locate(blockIdx.x - batch * items, interval, key_block);
+        const int first = max(interval * interval_length, visits.first_tile(key_block));
+        position = batch * per_batch + visits.before(key_block) + (first - visits.first_tile(key_block));
+        range_end = position + (cut.end_of(interval) - first);
+    } else if (ranges > 0) {
         position = index_math::wide_range_begin(total, ranges, blockIdx.x);
         range_end = index_math::wide_range_begin(total, ranges, blockIdx.x + 1);
     } else {
@@ -549,6 +561,8 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
         };
         // Tile t is multiplied out of one buffer while tile t + 1 goes from registers into the other and tile
         // t + 2 is on its way from memory: a fetch has a whole step to arrive, and a step has one barrier.
+        // (A second register set, for a fetch two steps ahead, was tried: the compiler waits for all
+        // outstanding loads before the first use of any, so the depth is lost, and the kernel spills.)
         fetch_rows(first_tile);
         __syncthreads();   // the previous segment has been read
         place_rows(first_tile);
@@ -661,8 +675,9 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
                 }
             }
         } else {
-            float* slot = partial_slots +
-                ((long long)blockIdx.x + (long long)batch * visits.key_blocks + key_block) * PARTIAL_FLOATS;
+            const long long slot_number =
+                interval_length > 0 ? (long long)blockIdx.x : (long long)blockIdx.x + (long long)batch * visits.key_blocks + key_block;
+            float* slot = partial_slots + slot_number * PARTIAL_FLOATS;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float* slot_row = slot + (8 * (i / 4) + 4 * g + i % 4) * WIDTH;
@@ -675,7 +690,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     }
 }
 
-// Sums the partial key gradients of every key block whose visits were cut, in range order.  Workgroup (x, y)
+// Sums the partial key gradients of every key block whose visits were cut, in range (or interval) order.  Workgroup (x, y)
 // takes the y-th 1/REDUCTION_PARTS of key block x (numbered through the batch elements), a thread four
 // neighbouring columns of one key; a block that one range held whole wrote its gradients itself.
 constexpr int REDUCTION_PARTS = PARTIAL_FLOATS / 4 / THREADS;   // 18
@@ -683,26 +698,42 @@ static_assert(REDUCTION_PARTS * THREADS * 4 == PARTIAL_FLOATS, "slot size");
 
 __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
     bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient,
-    const float* __restrict__ partial_slots, int sequence_length, int heads, int batch_size, int ranges) {
+    const float* __restrict__ partial_slots, int sequence_length, int heads, int batch_size, int ranges,
+    int interval_length) {
     const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
-    const long long per_batch = visits.per_batch();
-    const long long total = per_batch * batch_size;
     const int batch = blockIdx.x / visits.key_blocks;
     const int key_block = blockIdx.x % visits.key_blocks;
-    const long long begin = batch * per_batch + visits.before(key_block);
-    const long long end = batch * per_batch + visits.before(key_block + 1);
-    const long long first_range = index_math::wide_range_of(total, ranges, begin);
-    const long long last_range = index_math::wide_range_of(total, ranges, end - 1);
-    if (first_range == last_range) return;
-
     const int index = blockIdx.y * THREADS + threadIdx.x;   // which four floats of the slot
-    const float* first_slot = partial_slots + (first_range + blockIdx.x) * PARTIAL_FLOATS + 4 * index;
-    const int parts = (int)(last_range - first_range) + 1;
-    f32x4 sum = *reinterpret_cast<const f32x4*>(first_slot);
-    for (int part = 1; part < parts; ++part) {
-        const f32x4 value = *reinterpret_cast<const f32x4*>(first_slot + (long long)part * PARTIAL_FLOATS);
+    f32x4 sum;
+    if (interval_length > 0) {
+        // the block's items: one per interval from the one its first tile lies in, slot = item number
+        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, interval_length);
+        const int first = cut.first_interval(key_block);
+        if (first == cut.intervals - 1) return;
+        long long slot = batch * cut.items() + cut.items_before(first) + key_block;
+        sum = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
+        for (int interval = first + 1; interval < cut.intervals; ++interval) {
+            slot += cut.blocks_in(interval - 1);
+            const f32x4 value = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sum[e] += value[e];
+            for (int e = 0; e < 4; ++e) sum[e] += value[e];
+        }
+    } else {
+        const long long per_batch = visits.per_batch();
+        const long long total = per_batch * batch_size;
+        const long long begin = batch * per_batch + visits.before(key_block);
+        const long long end = batch * per_batch + visits.before(key_block + 1);
+        const long long first_range = index_math::wide_range_of(total, ranges, begin);
+        const long long last_range = index_math::wide_range_of(total, ranges, end - 1);
+        if (first_range == last_range) return;
+        const float* first_slot = partial_slots + (first_range + blockIdx.x) * PARTIAL_FLOATS + 4 * index;
+        const int parts = (int)(last_range - first_range) + 1;
+        sum = *reinterpret_cast<const f32x4*>(first_slot);
+        for (int part = 1; part < parts; ++part) {
+            const f32x4 value = *reinterpret_cast<const f32x4*>(first_slot + (long long)part * PARTIAL_FLOATS);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] += value[e];
+        }
     }
     const int key = key_block * TILE + (4 * index) / WIDTH;
     const int column = (4 * index) % WIDTH;
@@ -721,6 +752,20 @@ template <typename Kernel>
 void raise_lds_limit(Kernel kernel, int bytes) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   bytes));
+}
+
+constexpr long long LARGE_INPUT_BYTES = 64LL << 20;   // per batch element, against 32 MB of L2 and 256 MB behind it
+constexpr int INTERVAL_TILES = 256;                   // 18 MB of rows
+
+// DSCUDA_AMD_KEY_INTERVAL_TILES in the environment (read once per process) forces the interval cut with that many
+// row tiles per interval at any size the slots allow: the cut can then be exercised at sizes a test can check.
+int forced_interval_tiles() {
+    static const int forced = [] {
+        const char* text = std::getenv("DSCUDA_AMD_KEY_INTERVAL_TILES");
+        const long value = text ? std::strtol(text, nullptr, 10) : 0;
+        return value > 0 && value < (1 << 24) ? (int)value : 0;
+    }();
+    return forced;
 }
 
 int device_compute_units() {
@@ -764,21 +809,40 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
     const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
     const long long blocks = (long long)visits.key_blocks * batch_size;
     const long long total = visits.per_batch() * batch_size;
-    const long long ranges = index_math::key_gradient_ranges(total, blocks, visits.row_tiles,
-                                                             rows * batch_size * RANK * 2, device_compute_units());
+    const long long scratch_bytes = rows * batch_size * RANK * 2;
+    // Rows that outgrow the caches (query and dO rows of a batch element, 2176 bytes per row): the interval cut
+    int interval_length = 0;
+    long long grid = 0;
+    const int forced = forced_interval_tiles();
+    if (forced > 0 || rows * (2 * RANK + ROPE) * 2 > LARGE_INPUT_BYTES) {
+        const int tiles = forced > 0 ? forced : INTERVAL_TILES;
+        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles);
+        const long long items = cut.items() * batch_size;
+        // enough items to keep every compute unit busy through several rounds, and a slot for each
+        if ((forced > 0 || items >= 4LL * device_compute_units()) && items <= scratch_bytes / index_math::KEY_PARTIAL_BYTES &&
+            items <= 0x7fffffffLL) {
+            interval_length = tiles;
+            grid = items;
+        }
+    }
+    long long ranges = 0;
+    if (interval_length == 0) {
+        ranges = index_math::key_gradient_ranges(total, blocks, visits.row_tiles, scratch_bytes, device_compute_units());
+        grid = ranges > 0 ? ranges : blocks;
+    }
 
     hipLaunchKernelGGL(mla_absorbed_row_statistics_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS), 0,
                        stream, delta, output_gradient, output, rows * batch_size);
     HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)(ranges > 0 ? ranges : blocks)), dim3(THREADS),
-                       KeyGradLayout::LDS_BYTES, stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta,
-                       output_gradient, logsumexp, query_latent, query_rope, kv_latent, key_rope, batch_size,
-                       sequence_length, heads, (int)ranges, scale);
+    hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)grid), dim3(THREADS), KeyGradLayout::LDS_BYTES,
+                       stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta, output_gradient, logsumexp,
+                       query_latent, query_rope, kv_latent, key_rope, batch_size, sequence_length, heads, (int)ranges,
+                       interval_length, scale);
     HIP_CHECK(hipGetLastError());
-    if (ranges > 0) {
-        hipLaunchKernelGGL(mla_absorbed_key_reduction_kernel, dim3((unsigned)blocks, REDUCTION_PARTS), dim3(THREADS), 0, stream,
-                           kv_latent_gradient, key_rope_gradient, partial_slots, sequence_length, heads, batch_size,
-                           (int)ranges);
+    if (ranges > 0 || interval_length > 0) {
+        hipLaunchKernelGGL(mla_absorbed_key_reduction_kernel, dim3((unsigned)blocks, REDUCTION_PARTS), dim3(THREADS), 0,
+                           stream, kv_latent_gradient, key_rope_gradient, partial_slots, sequence_length, heads,
+                           batch_size, (int)ranges, interval_length);
         HIP_CHECK(hipGetLastError());
     }
     hipLaunchKernelGGL(mla_absorbed_query_gradient_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS),

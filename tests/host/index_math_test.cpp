@@ -332,6 +332,44 @@ void check_key_visits() {
     }
 }
 
+// ---- absorbed backward, interval cut: the items cover every (key block, row tile) visit exactly once, item numbers
+// are a bijection, a block has one item exactly when it starts in the last interval
+void check_key_intervals() {
+    for (int heads : {1, 3, 8, 16, 128}) {
+        for (int tokens : {1, 33, 257, 512, 1000}) {
+            if ((long long)heads * tokens > 70000) continue;
+            for (int length : {1, 2, 7, 64, 100000}) {
+                const KeyIntervals cut = key_intervals(tokens, heads, length);
+                const KeyVisits visits = key_visits(tokens, heads);
+                EXPECT(cut.key_blocks == visits.key_blocks && cut.row_tiles == visits.row_tiles, "counts");
+                std::vector<int> seen((size_t)cut.key_blocks * cut.row_tiles, 0), parts(cut.key_blocks, 0);
+                long long item = 0;
+                for (int i = 0; i < cut.intervals; ++i) {
+                    EXPECT(cut.items_before(i) == item, "items_before");
+                    for (int kb = 0; kb < cut.blocks_in(i); ++kb, ++item) {
+                        int interval, key_block;
+                        cut.locate(item, interval, key_block);
+                        EXPECT(interval == i && key_block == kb, "locate %lld: %d %d vs %d %d", item, interval, key_block, i, kb);
+                        EXPECT(cut.first_interval(kb) <= i, "first_interval");
+                        const int lo = std::max(i * length, visits.first_tile(kb)), hi = cut.end_of(i);
+                        EXPECT(lo < hi, "empty item heads %d tokens %d length %d interval %d block %d", heads, tokens, length, i, kb);
+                        for (int tile = lo; tile < hi; ++tile) ++seen[(size_t)kb * cut.row_tiles + tile];
+                        ++parts[kb];
+                    }
+                }
+                EXPECT(item == cut.items(), "items");
+                for (int kb = 0; kb < cut.key_blocks; ++kb) {
+                    EXPECT(parts[kb] == cut.intervals - cut.first_interval(kb), "parts of block %d: %d", kb, parts[kb]);
+                    for (int tile = 0; tile < cut.row_tiles; ++tile) {
+                        EXPECT(seen[(size_t)kb * cut.row_tiles + tile] == (tile >= visits.first_tile(kb) ? 1 : 0), "visit (%d, %d) seen %d times", kb, tile,
+                               seen[(size_t)kb * cut.row_tiles + tile]);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- decode: the ranges partition the list of positions, their lengths differ by at most one, every tile of every
 // sequence is computed by exactly one range, and (range, sequence) pairs that hold part of a sequence own distinct slots
 void check_decode_ranges() {
@@ -471,6 +509,7 @@ int main() {
     check_decode_loads<8>();
     check_decode_loads<32>();
     check_key_visits();
+    check_key_intervals();
     check_decode_ranges();
     check_decode_layout();
     if (failures) {

@@ -92,13 +92,16 @@ def test_backward_workload_3(cuda):
 
 # ---- absorbed backward (dscuda_mla_backward) ------------------------------------
 
-@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 96, 20), (1, 1024, 16)])
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 96, 20), (1, 1024, 16),
+                                                                                             (1, 256, 128), (2, 160, 128)])
 def test_absorbed_backward(cuda, batch, tokens, heads):
     """Shapes of benchmarks/mla.py:34-45; dO = 0.2 * N(0,1) as at :108; saved O (bf16) and LSE
     come from the oracle forward as at :68,113-117."""
     ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
     g = torch.Generator().manual_seed(77)
-    dout = (torch.randn(batch, tokens, heads, 512, generator=g) * 0.2).bfloat16()
+    # dLatent sums over all heads: with 128 of them dO is scaled down so that the sums stay where half a bf16 ulp
+    # (the rounding of the result itself) is below the tolerance
+    dout = (torch.randn(batch, tokens, heads, 512, generator=g) * (0.2 if heads <= 32 else 0.05)).bfloat16()
     mask = oracle.causal_mask(tokens)
     out, lse = oracle.mla_forward(ql, qr, c, kr, scale, mask)
     announce("mla_backward", dict(B=batch, T=tokens, H=heads))
@@ -148,6 +151,23 @@ def test_backward_in_chunks_of_pairs(cuda, batch, seq, heads, budget_pairs, expe
                              str(expected_chunk)], cwd=root, env=environment, capture_output=True, text=True, timeout=300)
     assert result.returncode == 0, result.stdout[-2000:] + result.stderr[-4000:]
     assert "chunked backward ok" in result.stdout
+
+
+@pytest.mark.parametrize("batch,tokens,heads,interval_tiles", [
+    (1, 256, 128, 256),   # 4 intervals, 20 items: key block 0 has four parts, the last two blocks one
+    (2, 160, 128, 100),   # two batch elements, a short last interval, interval ends inside key blocks
+    (1, 512, 8, 7),       # many short intervals
+    (2, 257, 4, 1000),    # one interval: every key block whole
+])
+def test_absorbed_backward_interval_cut(cuda, batch, tokens, heads, interval_tiles):
+    """The cut of the key gradients for inputs that outgrow the caches (items of one interval of row tiles and one
+    key block, dealt to the XCDs), forced at sizes the oracle can check."""
+    environment = dict(os.environ, DSCUDA_AMD_KEY_INTERVAL_TILES=str(interval_tiles))
+    root = Path(__file__).resolve().parents[1]
+    result = subprocess.run([sys.executable, "-m", "tests.absorbed_interval_case", str(batch), str(tokens), str(heads)],
+                            cwd=root, env=environment, capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stdout[-2000:] + result.stderr[-4000:]
+    assert "interval cut ok" in result.stdout
 
 
 def test_backward_workspace_is_bounded(cuda):
