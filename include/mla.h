@@ -49,9 +49,12 @@ void mla_compressed_attention_forward_cuda(
 
 // Absorbed-query MLA backward, recomputing probabilities from the saved FP32
 // logsumexp.  Replaces reference include/mla.h:35-53.  The four gradient
-// buffers are overwritten; every gradient row has exactly one writer, so the
-// result is deterministic and needs no workspace (the reference's ownership
-// rule, kernels/attention/mla/sm89.cu:2).
+// buffers are overwritten, the caller passes no workspace, and the result does
+// not depend on timing: every gradient element is written by one thread and
+// every sum has a fixed order (the reference's ownership rule,
+// kernels/attention/mla/sm89.cu:2, kept as determinism).  Until the last of the
+// call's launches the two query-gradient buffers hold intermediate values (row
+// statistics, partial key gradients); both must be aligned to 16 bytes.
 void mla_compressed_attention_backward_cuda(
     __hip_bfloat16* query_latent_gradient,
     __hip_bfloat16* query_rope_gradient,
