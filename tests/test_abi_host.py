@@ -74,6 +74,9 @@ def test_mla_shape_errors_round_trip_without_a_gpu():
         "MLA requires C=512 and RoPE=64"
     assert "positive" in _status_and_message(lib, "mla", forward(*null * 6, 0, 8, 2, 512, 64, 1.0, None))
     assert "positive" in _status_and_message(lib, "mla", decode(*null * 7, 1, 8, 512, 64, 64, 4, 0, 1.0, None))
+    # the backward keeps intermediate values in its query-gradient outputs: 16-byte alignment is checked first
+    misaligned = [0x1008, 0x2000] + [0x3000] * 9
+    assert "aligned to 16 bytes" in _status_and_message(lib, "mla", backward(*misaligned, 1, 8, 2, 512, 64, 1.0, None))
     prefill = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
     assert "(d_qk,d_v)" in _status_and_message(lib, "mla", prefill(*null * 5, 1, 8, 2, 96, 96, 1.0, None))
     prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
