@@ -36,7 +36,7 @@ COMMON_FLAGS = [
 ]
 
 LIBRARIES = {
-    "libdscuda_mla_bench.so": ["api_mla", "attn_fwd", "attn_bwd", "mla_absorbed", "mla_decode", "rope"],
+    "libdscuda_mla_bench.so": ["api_mla", "attn_fwd", "attn_bwd", "mla_absorbed", "mla_decode", "mla_projection", "rope"],
     "libdscuda_flash_attention_bench.so": ["api_flash", "attn_fwd", "attn_bwd"],
 }
 

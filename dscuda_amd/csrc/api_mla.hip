@@ -209,6 +209,24 @@ void rope_apply_cuda(__hip_bfloat16* tensor, const int* positions, int batch_siz
     rope_apply_dispatch(tensor, positions, batch_size, sequence_length, heads, width, rope_offset, rope_size, theta, stream);
 }
 
+void mla_absorb_query_cuda(__hip_bfloat16* query_latent, const __hip_bfloat16* query_nope, const __hip_bfloat16* w_uk,
+                           long long tokens, int heads, long long query_nope_token_stride,
+                           long long query_nope_head_stride, long long query_latent_token_stride,
+                           long long query_latent_head_stride, long long weight_head_stride, hipStream_t stream) {
+    mla_absorb_query_dispatch(query_latent, query_nope, w_uk, tokens, heads, query_nope_token_stride,
+                              query_nope_head_stride, query_latent_token_stride, query_latent_head_stride,
+                              weight_head_stride, stream);
+}
+
+void mla_unabsorb_output_cuda(__hip_bfloat16* output, const __hip_bfloat16* output_latent, const __hip_bfloat16* w_uv,
+                              long long tokens, int heads, long long output_latent_token_stride,
+                              long long output_latent_head_stride, long long output_token_stride,
+                              long long output_head_stride, long long weight_head_stride, hipStream_t stream) {
+    mla_unabsorb_output_dispatch(output, output_latent, w_uv, tokens, heads, output_latent_token_stride,
+                                 output_latent_head_stride, output_token_stride, output_head_stride,
+                                 weight_head_stride, stream);
+}
+
 }  // namespace dscuda
 
 namespace {
@@ -327,5 +345,29 @@ extern "C" int dscuda_rope_apply(__hip_bfloat16* tensor, const int* positions, i
                                  int width, int rope_offset, int rope_size, float theta, hipStream_t stream) {
     return guarded([&] {
         dscuda::rope_apply_cuda(tensor, positions, batch, sequence, heads, width, rope_offset, rope_size, theta, stream);
+    });
+}
+
+extern "C" int dscuda_mla_absorb_query(__hip_bfloat16* query_latent, const __hip_bfloat16* query_nope,
+                                       const __hip_bfloat16* w_uk, long long tokens, int heads,
+                                       long long query_nope_token_stride, long long query_nope_head_stride,
+                                       long long query_latent_token_stride, long long query_latent_head_stride,
+                                       long long weight_head_stride, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_absorb_query_cuda(query_latent, query_nope, w_uk, tokens, heads, query_nope_token_stride,
+                                      query_nope_head_stride, query_latent_token_stride, query_latent_head_stride,
+                                      weight_head_stride, stream);
+    });
+}
+
+extern "C" int dscuda_mla_unabsorb_output(__hip_bfloat16* output, const __hip_bfloat16* output_latent,
+                                          const __hip_bfloat16* w_uv, long long tokens, int heads,
+                                          long long output_latent_token_stride, long long output_latent_head_stride,
+                                          long long output_token_stride, long long output_head_stride,
+                                          long long weight_head_stride, hipStream_t stream) {
+    return guarded([&] {
+        dscuda::mla_unabsorb_output_cuda(output, output_latent, w_uv, tokens, heads, output_latent_token_stride,
+                                         output_latent_head_stride, output_token_stride, output_head_stride,
+                                         weight_head_stride, stream);
     });
 }

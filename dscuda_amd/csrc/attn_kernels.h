@@ -36,6 +36,20 @@ void attention_backward_dispatch(__hip_bfloat16* query_gradient, __hip_bfloat16*
 void rope_apply_dispatch(__hip_bfloat16* tensor, const int* positions, int batch_size, int sequence_length, int heads,
                          int width, int rope_offset, int rope_size, float theta, hipStream_t stream);
 
+// mla_projection.hip -- the per-head projections either side of absorbed attention: q_latent = q_nope W_UK and
+// out = o_latent W_UV^T, both weights [heads, 128, 512] (head h at weight + h * weight_head_stride); token t, head h
+// of a tensor at base + t * token_stride + h * head_stride (elements).
+void mla_absorb_query_dispatch(__hip_bfloat16* query_latent, const __hip_bfloat16* query_nope,
+                               const __hip_bfloat16* weight, long long tokens, int heads,
+                               long long query_nope_token_stride, long long query_nope_head_stride,
+                               long long query_latent_token_stride, long long query_latent_head_stride,
+                               long long weight_head_stride, hipStream_t stream);
+void mla_unabsorb_output_dispatch(__hip_bfloat16* output, const __hip_bfloat16* output_latent,
+                                  const __hip_bfloat16* weight, long long tokens, int heads,
+                                  long long output_latent_token_stride, long long output_latent_head_stride,
+                                  long long output_token_stride, long long output_head_stride,
+                                  long long weight_head_stride, hipStream_t stream);
+
 // mla_absorbed.hip -- absorbed (C=512, R=64) causal forward and backward with
 // one shared latent KV head.
 void mla_absorbed_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const __hip_bfloat16* query_latent,

@@ -38,6 +38,9 @@ class _Mla:
         self.decode_static = bind(lib, "dscuda_mla_decode_static", [P] * 6 + [I] * 7 + [F, P])
         self.workspace = bind(lib, "dscuda_mla_workspace_elements", [I] * 4, ctypes.c_size_t)
         self.rope_apply = bind(lib, "dscuda_rope_apply", [P] * 2 + [I] * 6 + [F, P])
+        L = ctypes.c_longlong
+        self.absorb_query = bind(lib, "dscuda_mla_absorb_query", [P] * 3 + [L, I] + [L] * 5 + [P])
+        self.unabsorb_output = bind(lib, "dscuda_mla_unabsorb_output", [P] * 3 + [L, I] + [L] * 5 + [P])
         self.prefill_forward = bind(lib, "dscuda_mla_prefill_forward", [P] * 5 + [I] * 5 + [F, P])
         self.prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
         self.prefill_workspace = bind(
@@ -232,6 +235,53 @@ def rope_apply(tensor, rope_offset=0, rope_size=None, theta=10000.0, positions=N
     checked(lib.lib, "mla", lib.rope_apply(tensor.data_ptr(), positions.data_ptr() if positions is not None else None,
                                            b, s, h, w, rope_offset, rope_size, theta, stream()))
     return tensor
+
+
+def _head_rows(name, tensor, width):
+    """(tokens, heads, token stride, head stride) of a bf16 [..., H, >= width] view whose leading dimensions are
+    laid out one behind the other and whose last dimension is contiguous."""
+    if not tensor.is_cuda:
+        raise RuntimeError("dscuda_amd operators need GPU tensors; there is no CPU path")
+    if tensor.dtype != torch.bfloat16 or tensor.dim() < 3 or tensor.shape[-1] != width or tensor.stride(-1) != 1:
+        raise ValueError(f"{name}: a bf16 [..., H, {width}] tensor with a contiguous last dimension is required")
+    heads, token_stride = tensor.shape[-2], tensor.stride(-3)
+    tokens = 1
+    for size, stride in zip(reversed(tensor.shape[:-2]), reversed(tensor.stride()[:-2])):
+        if size != 1 and stride != token_stride * tokens:
+            raise ValueError(f"{name}: the token dimensions must be laid out one behind the other")
+        tokens *= size
+    return tokens, heads, token_stride, tensor.stride(-2)
+
+
+def mla_absorb_query(query_nope, w_uk, out=None):
+    """q_latent[..., h, :] = q_nope[..., h, :] @ w_uk[h]  (dscuda_mla_absorb_query).  query_nope: [..., H, 128] (may be
+    the nope columns of a wider tensor), w_uk: [H, 128, 512] (may be a slice of wkv_b), out: [..., H, 512] (may be
+    the latent columns of the packed decode query)."""
+    tokens, heads, x_token, x_head = _head_rows("mla_absorb_query", query_nope, 128)
+    if out is None:
+        out = torch.empty(*query_nope.shape[:-1], 512, device=query_nope.device, dtype=torch.bfloat16)
+    out_tokens, out_heads, y_token, y_head = _head_rows("mla_absorb_query", out, 512)
+    if (out_tokens, out_heads) != (tokens, heads) or tuple(w_uk.shape) != (heads, 128, 512) or w_uk.stride()[1:] != (512, 1):
+        raise ValueError("mla_absorb_query: shapes do not fit")
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.absorb_query(out.data_ptr(), query_nope.data_ptr(), w_uk.data_ptr(), tokens, heads,
+                                             x_token, x_head, y_token, y_head, w_uk.stride(0), stream()))
+    return out
+
+
+def mla_unabsorb_output(output_latent, w_uv, out=None):
+    """out[..., h, :] = output_latent[..., h, :] @ w_uv[h].T  (dscuda_mla_unabsorb_output).  output_latent:
+    [..., H, 512], w_uv: [H, 128, 512] (may be a slice of wkv_b), out: [..., H, 128]."""
+    tokens, heads, x_token, x_head = _head_rows("mla_unabsorb_output", output_latent, 512)
+    if out is None:
+        out = torch.empty(*output_latent.shape[:-1], 128, device=output_latent.device, dtype=torch.bfloat16)
+    out_tokens, out_heads, y_token, y_head = _head_rows("mla_unabsorb_output", out, 128)
+    if (out_tokens, out_heads) != (tokens, heads) or tuple(w_uv.shape) != (heads, 128, 512) or w_uv.stride()[1:] != (512, 1):
+        raise ValueError("mla_unabsorb_output: shapes do not fit")
+    lib = mla_library()
+    checked(lib.lib, "mla", lib.unabsorb_output(out.data_ptr(), output_latent.data_ptr(), w_uv.data_ptr(), tokens, heads,
+                                                x_token, x_head, y_token, y_head, w_uv.stride(0), stream()))
+    return out
 
 
 def flash_backward_workspace(batch, seq, q_heads, kv_heads, dim, device="cuda"):

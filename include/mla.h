@@ -263,6 +263,42 @@ void rope_apply_cuda(
     float theta,
     hipStream_t stream = nullptr);
 
+// The per-head projections either side of absorbed attention, which the reference leaves to its
+// caller (reference/python/sources.json:2, "No ... model projections"); no counterpart there:
+//     absorb     query_latent[t, h, c] = sum_d query_nope[t, h, d]  * w_uk[h, d, c]     d < 128, c < 512
+//     un-absorb  output[t, h, d]       = sum_c output_latent[t, h, c] * w_uv[h, d, c]
+// Both weights are [heads, 128, 512] BF16 (head h at w + h * weight_head_stride elements): the two
+// halves of DeepSeek-V3's wkv_b viewed as [heads, 256, 512], stride 256 * 512.  Token t, head h of a
+// tensor lies at base + t * token_stride + h * head_stride (elements), so the absorb can read the nope
+// columns of a [B,S,H,192] query and write the latent columns of the packed [B,S,H,576] decode query
+// directly.  BF16 in and out, FP32 accumulation.  All tensors aligned to 16 bytes, all strides multiples
+// of 8 elements.
+void mla_absorb_query_cuda(
+    __hip_bfloat16* query_latent,
+    const __hip_bfloat16* query_nope,
+    const __hip_bfloat16* w_uk,
+    long long tokens,
+    int heads,
+    long long query_nope_token_stride,
+    long long query_nope_head_stride,
+    long long query_latent_token_stride,
+    long long query_latent_head_stride,
+    long long weight_head_stride,
+    hipStream_t stream = nullptr);
+
+void mla_unabsorb_output_cuda(
+    __hip_bfloat16* output,
+    const __hip_bfloat16* output_latent,
+    const __hip_bfloat16* w_uv,
+    long long tokens,
+    int heads,
+    long long output_latent_token_stride,
+    long long output_latent_head_stride,
+    long long output_token_stride,
+    long long output_head_stride,
+    long long weight_head_stride,
+    hipStream_t stream = nullptr);
+
 }  // namespace dscuda
 
 // ---- C ABI (libdscuda_mla_bench.so) ----------------------------------------
@@ -345,5 +381,20 @@ int dscuda_rope_apply(
     __hip_bfloat16* tensor, const int* positions,
     int batch, int sequence, int heads, int width, int rope_offset, int rope_size, float theta,
     hipStream_t stream);
+
+// additive (no counterpart in the reference): see dscuda::mla_absorb_query_cuda / mla_unabsorb_output_cuda above
+int dscuda_mla_absorb_query(
+    __hip_bfloat16* query_latent, const __hip_bfloat16* query_nope, const __hip_bfloat16* w_uk,
+    long long tokens, int heads,
+    long long query_nope_token_stride, long long query_nope_head_stride,
+    long long query_latent_token_stride, long long query_latent_head_stride,
+    long long weight_head_stride, hipStream_t stream);
+
+int dscuda_mla_unabsorb_output(
+    __hip_bfloat16* output, const __hip_bfloat16* output_latent, const __hip_bfloat16* w_uv,
+    long long tokens, int heads,
+    long long output_latent_token_stride, long long output_latent_head_stride,
+    long long output_token_stride, long long output_head_stride,
+    long long weight_head_stride, hipStream_t stream);
 
 }  // extern "C"

@@ -19,7 +19,10 @@ fp64 tensors), the mathematics the reference defines for this path:
 
 The per-head (128 nope + 64 rope | 128 v) prefill forward/backward named by
 the headline configurations has no counterpart in the reference; its oracle
-is textbook causal attention with ``d_v != d_qk`` in the same style.
+is textbook causal attention with ``d_v != d_qk`` in the same style.  The
+two per-head projections either side of absorbed attention are likewise
+outside the reference (``reference/python/sources.json:2``); their oracle is
+one einsum each.
 
 How each function is pinned (see ``tests/test_oracle_pins.py``):
 
@@ -43,6 +46,11 @@ mla_decode             SDPA with a length mask; equals row T-1 of the
                        causal prefill when len == T; closed form of
                        ``benchmark_mla_decode.cu:42-48``
 pack_cache             closed form (identity table, zero padding)
+absorb_query,          fp64 triple-loop brute force; the identity absorption
+unabsorb_output        rests on: scores and outputs of per-head attention
+                       over k_nope = latent W_UK^T, v = latent W_UV^T equal
+                       those of absorbed attention between the two
+                       projections (a transposed or swapped weight fails it)
 =====================  =====================================================
 
 No function here is "parity unpinned".  The reference holds no golden
@@ -236,3 +244,16 @@ def error_stats(actual, expected):
     """(max-abs, mean-abs) of actual - expected, both taken in fp64."""
     diff = (actual.double() - expected.double()).abs()
     return diff.max().item(), diff.mean().item()
+
+
+def absorb_query(query_nope, w_uk):
+    """q_latent[..., h, c] = sum_d q_nope[..., h, d] * w_uk[h, d, c] in fp32: the step before absorbed attention that
+    the reference leaves to its caller (reference/python/sources.json:2).  Operand order as in the absorbed path of
+    DeepSeek-V3's inference/model.py (q_nope times the first 128 rows per head of wkv_b)."""
+    return torch.einsum("...hd,hdc->...hc", _compute(query_nope), _compute(w_uk))
+
+
+def unabsorb_output(output_latent, w_uv):
+    """out[..., h, d] = sum_c output_latent[..., h, c] * w_uv[h, d, c] in fp32: the step after absorbed attention
+    (the latent output times the last 128 rows per head of wkv_b, same source)."""
+    return torch.einsum("...hc,hdc->...hd", _compute(output_latent), _compute(w_uv))

@@ -301,3 +301,41 @@ def test_pack_cache_closed_form():
 def test_workspace_elements():
     assert oracle.decode_workspace_elements(2, 3, 8, 512) == 2 * 3 * 8 * 514
     assert oracle.decode_workspace_elements(64, 128, 8, 512) == 64 * 128 * 8 * 514
+
+
+def test_projections_brute_force_and_absorption_identity():
+    """absorb_query / unabsorb_output against explicit loops in fp64, and the identity that makes absorption valid:
+    per-head attention with k_nope = latent W_UK^T and v = latent W_UV^T gives the same output as absorbed attention
+    over the latent itself between the two projections."""
+    g = torch.Generator().manual_seed(11)
+    tokens, heads, d, c = 5, 3, 128, 512
+    q_nope = torch.randn(tokens, heads, d, generator=g, dtype=torch.float64)
+    w_uk = torch.randn(heads, d, c, generator=g, dtype=torch.float64) * 0.05
+    w_uv = torch.randn(heads, d, c, generator=g, dtype=torch.float64) * 0.05
+    latent = torch.randn(tokens, c, generator=g, dtype=torch.float64)
+    q_latent = oracle.absorb_query(q_nope.float(), w_uk.float()).double()
+    for t_index in (0, 4):
+        for h in range(heads):
+            for col in (0, 77, 511):
+                expected = sum(q_nope[t_index, h, k] * w_uk[h, k, col] for k in range(d))
+                assert abs(q_latent[t_index, h, col] - expected) < 1e-4
+    o_latent = torch.randn(tokens, heads, c, generator=g, dtype=torch.float64)
+    out = oracle.unabsorb_output(o_latent.float(), w_uv.float()).double()
+    for t_index in (1, 3):
+        for h in range(heads):
+            for col in (0, 64, 127):
+                expected = sum(o_latent[t_index, h, k] * w_uv[h, col, k] for k in range(c))
+                assert abs(out[t_index, h, col] - expected) < 1e-3
+    # the identity, in fp64 through the same functions
+    q_abs = oracle.absorb_query(q_nope, w_uk)                        # [T, H, C]
+    scale = 0.1
+    mask = oracle.causal_mask(tokens)
+    scores_absorbed = torch.einsum("thc,sc->hts", q_abs, latent) * scale
+    k_nope = torch.einsum("sc,hdc->shd", latent, w_uk)               # [S, H, D]
+    scores_heads = torch.einsum("thd,shd->hts", q_nope, k_nope) * scale
+    assert (scores_absorbed - scores_heads).abs().max() < 1e-9
+    p = torch.softmax(scores_heads.masked_fill(~mask, float("-inf")), dim=-1)
+    v = torch.einsum("sc,hdc->shd", latent, w_uv)
+    out_heads = torch.einsum("hts,shd->thd", p, v)
+    out_absorbed = oracle.unabsorb_output(torch.einsum("hts,sc->thc", p, latent), w_uv)
+    assert (out_heads - out_absorbed).abs().max() < 1e-9
