@@ -93,7 +93,8 @@ def test_backward_workload_3(cuda):
 # ---- absorbed backward (dscuda_mla_backward) ------------------------------------
 
 @pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 96, 20), (1, 1024, 16),
-                                                                                             (1, 256, 128), (2, 160, 128)])
+                                                                                             (1, 256, 128), (2, 160, 128),
+                                                                                             (1, 33, 160), (2, 50, 1)])
 def test_absorbed_backward(cuda, batch, tokens, heads):
     """Shapes of benchmarks/mla.py:34-45; dO = 0.2 * N(0,1) as at :108; saved O (bf16) and LSE
     come from the oracle forward as at :68,113-117."""

@@ -243,7 +243,8 @@ def test_decode_workload_4(cuda):
 
 # ---- absorbed causal prefill forward (dscuda_mla_forward) ----------------------
 
-@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 200, 128), (1, 1024, 16)])
+@pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL +
+                         [(1, 200, 128), (1, 1024, 16), (1, 33, 160), (2, 50, 1), (1, 70, 100)])
 def test_absorbed_forward(cuda, batch, tokens, heads):
     ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
     announce("mla_forward", dict(B=batch, T=tokens, H=heads))
@@ -252,6 +253,30 @@ def test_absorbed_forward(cuda, batch, tokens, heads):
     expected, expected_lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, oracle.causal_mask(tokens))
     assert_close_bf16("O", out, expected)
     assert_close_lse("LSE", lse, expected_lse)
+
+
+def test_absorbed_forward_large_scores_raise_the_reference(cuda):
+    """The prefill form of the same walk: late keys aligned with the queries give scores far above what the first
+    keys gave, rows of one workgroup see different numbers of keys, and the rows that meet the hot keys raise
+    their softmax reference while the others (earlier tokens) never see them."""
+    batch, tokens, heads = 1, 300, 8
+    g = torch.Generator().manual_seed(14)
+    direction = torch.randn(576, generator=g)
+    query = (direction[None, None, None, :] + 0.1 * torch.randn(batch, tokens, heads, 576, generator=g)).bfloat16()
+    keys = (torch.randn(batch, tokens, 576, generator=g) * 0.05).bfloat16()
+    for first, last, factor in [(100, 110, 1.0), (200, 260, 4.0)]:
+        keys[:, first:last] = (direction * factor).bfloat16()
+    ql, qr = query[..., :512].contiguous(), query[..., 512:].contiguous()
+    c, kr = keys[..., :512].contiguous(), keys[..., 512:].contiguous()
+    scale = 1.0
+    announce("mla_forward raised reference")
+    out, lse = ops.mla_forward(ql.to(cuda), qr.to(cuda), c.to(cuda), kr.to(cuda), scale)
+    torch.cuda.synchronize()
+    expected, expected_lse = oracle.mla_forward_unrounded(ql, qr, c, kr, scale, oracle.causal_mask(tokens))
+    assert expected_lse.max() > 500 and expected_lse[..., :100].max() < 200
+    torch.testing.assert_close(out.cpu().float(), expected, atol=8e-3, rtol=8e-3)
+    worst = ((lse.cpu() - expected_lse).abs() / expected_lse.abs().clamp_min(1)).max().item()
+    assert worst <= 1e-5
 
 
 def test_absorbed_forward_closed_form_constant_fill(cuda):
