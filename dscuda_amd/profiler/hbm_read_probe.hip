@@ -7,7 +7,9 @@
 //   lds         the decode kernel's own instruction: each wave streams 1 KB per instruction
 //               straight into LDS (global_load_lds_dwordx4), 36 KB units through a ring of four
 //               slots with one, two or three units in flight per workgroup, one workgroup per
-//               compute unit.
+//               compute unit;
+//   both        four waves of a workgroup stream into LDS while four others read into registers,
+//               each over its own share of the buffer.
 //
 // Usage: hbm_read_probe [MiB = 1024] [iterations = 20]
 // Prints one line per form and launch shape, and "HBM_READ_PROBE best_GBps=..." at the end.
@@ -78,6 +80,50 @@ __global__ __launch_bounds__(256) void read_into_lds(const unsigned char* data, 
     sink[(size_t)blockIdx.x * 256 + threadIdx.x] = reinterpret_cast<const unsigned*>(lds)[threadIdx.x];
 }
 
+// Both forms in one workgroup of eight waves: waves 0-3 stream units [0, units) into LDS (three in flight), waves
+// 4-7 read the 16-byte pieces [first_piece, count) into registers.  If the two together draw more than either
+// alone, what limits the LDS form is its request path and not the memory.
+__global__ __launch_bounds__(512) void read_both(const unsigned char* data, int units, size_t first_piece, size_t count,
+                                                 unsigned* sink) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int lane = threadIdx.x % 64;
+    unsigned folded = 0;
+    if (wave < 4) {
+        const unsigned lds_base = dscuda::lds_offset_of(lds);
+        int issued = 0;
+        for (int unit = blockIdx.x; unit < units; unit += gridDim.x, ++issued) {
+            const unsigned char* source = data + (size_t)unit * UNIT_BYTES + wave * (WAVE_LOADS * 1024);
+            const unsigned target = lds_base + (issued % SLOTS) * UNIT_BYTES + wave * (WAVE_LOADS * 1024);
+#pragma unroll
+            for (int i = 0; i < WAVE_LOADS; ++i) dscuda::direct_load_16_offset(source, i * 1024 + lane * 16, target + i * 1024);
+            dscuda::wait_vector_memory<2 * WAVE_LOADS>();
+        }
+        dscuda::wait_vector_memory<0>();
+    } else {
+        constexpr int UNROLL = 8;
+        const uint4* pieces = reinterpret_cast<const uint4*>(data);
+        const size_t stride = (size_t)gridDim.x * 256;
+        size_t i = first_piece + (size_t)blockIdx.x * 256 + (threadIdx.x - 256);
+        uint4 total = {0, 0, 0, 0};
+        for (; i + (UNROLL - 1) * stride < count; i += UNROLL * stride) {
+            uint4 piece[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) piece[u] = pieces[i + u * stride];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                total.x ^= piece[u].x;
+                total.y ^= piece[u].y;
+                total.z ^= piece[u].z;
+                total.w ^= piece[u].w;
+            }
+        }
+        folded = total.x ^ total.y ^ total.z ^ total.w;
+    }
+    __syncthreads();
+    sink[(size_t)blockIdx.x * 512 + threadIdx.x] = folded ^ reinterpret_cast<const unsigned*>(lds)[threadIdx.x % 256];
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -134,6 +180,16 @@ int main(int argc, char** argv) {
               [&] { read_into_lds<2><<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, words); });
         timed("lds x3", 256, (double)units * UNIT_BYTES,
               [&] { read_into_lds<3><<<256, 256, SLOTS * UNIT_BYTES>>>(data.get(), units, words); });
+        PROFILER_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(read_both),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, SLOTS * UNIT_BYTES));
+        for (int tenths : {3, 4, 5, 6}) {   // share of the buffer that goes through registers
+            const size_t first_piece = (size_t)units * (10 - tenths) / 10 * UNIT_BYTES / sizeof(uint4);
+            const int lds_units = (int)(first_piece * sizeof(uint4) / UNIT_BYTES);
+            char form[32];
+            std::snprintf(form, sizeof form, "both .%d", tenths);
+            timed(form, 256, (double)lds_units * UNIT_BYTES + (double)(count - first_piece) * sizeof(uint4),
+                  [&] { read_both<<<256, 512, SLOTS * UNIT_BYTES>>>(data.get(), lds_units, first_piece, count, words); });
+        }
         std::printf("check passed\nHBM_READ_PROBE bytes=%zu best_GBps=%.1f\n", bytes, best);
         PROFILER_HIP_CHECK(hipEventDestroy(start));
         PROFILER_HIP_CHECK(hipEventDestroy(stop));
