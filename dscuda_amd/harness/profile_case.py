@@ -11,8 +11,9 @@ profiled ones.
 Workloads: forward / backward (B=1, S, H=128, 192|128), decode (B=64, H=128,
 lengths ~ U[1024, 8192] seed 3), flash (B=1, H=8, S=512, D=64), absorbed (the
 reference's own prefill entry points, forward then backward, B=1, T=S, H heads,
-512 latent + 64 rope), copy (a plain 16-byte-per-lane copy of 1 GiB, the
-calibration kernel for FETCH_SIZE / WRITE_SIZE).
+512 latent + 64 rope), projection (the W_UK absorb and W_UV un-absorb of S tokens x
+H heads), copy (a plain 16-byte-per-lane copy of 1 GiB, the calibration kernel for
+FETCH_SIZE / WRITE_SIZE).
 """
 
 from __future__ import annotations
@@ -28,7 +29,7 @@ if str(ROOT) not in sys.path:
 
 def main():
     parser = argparse.ArgumentParser(description=__doc__)
-    parser.add_argument("workload", choices=("forward", "backward", "decode", "flash", "absorbed", "copy"))
+    parser.add_argument("workload", choices=("forward", "backward", "decode", "flash", "absorbed", "projection", "copy"))
     parser.add_argument("--steps", type=int, default=3)
     parser.add_argument("--seq", type=int, default=4096)
     parser.add_argument("--heads", type=int, default=128)
@@ -84,6 +85,16 @@ def main():
         def call():
             ops.mla_forward(ql, qr, latent, kr, scale, out, lse)
             ops.mla_backward(dout, out, lse, ql, qr, latent, kr, scale, grads)
+    elif args.workload == "projection":
+        tokens, h = args.seq, args.heads
+        wkv_b = randn((h, 256, 512), 0.06)
+        q_nope, o_latent = randn((1, tokens, h, 128), 0.5), randn((1, tokens, h, 512), 0.5)
+        q_latent = torch.empty(1, tokens, h, 512, device=device, dtype=torch.bfloat16)
+        o = torch.empty(1, tokens, h, 128, device=device, dtype=torch.bfloat16)
+
+        def call():
+            ops.mla_absorb_query(q_nope, wkv_b[:, :128], out=q_latent)
+            ops.mla_unabsorb_output(o_latent, wkv_b[:, 128:], out=o)
     elif args.workload == "flash":
         q, k, v = randn((1, 512, 8, 64), 1.0), randn((1, 512, 8, 64), 1.0), randn((1, 512, 8, 64), 1.0)
         out, lse = torch.empty_like(q), torch.empty(1, 8, 512, device=device)

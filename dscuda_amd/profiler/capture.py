@@ -96,6 +96,8 @@ def metric_cases(suite):
     add("flash_forward_S512_H8_D64", "flash forward B=1 H=8 S=512 D=64", "flash", 300, 100, ["attention_forward"])
     add("mla_absorbed_T4096_H128", "absorbed MLA prefill forward + backward (dscuda_mla_forward / _backward) B=1 T=4096 H=128",
         "absorbed", 6, 3, ["mla_absorbed"])
+    add("mla_projection_T4096_H128", "W_UK absorb and W_UV un-absorb of 4096 tokens x 128 heads", "projection", 60, 20,
+        ["mla_absorb_query", "mla_unabsorb_output"])
     if suite == "full":
         add("mla_prefill_forward_S16384_H128", "MLA prefill forward B=1 S=16384 H=128 192/128", "forward", 16, 8,
             ["attention_forward"], "--seq", 16384)
