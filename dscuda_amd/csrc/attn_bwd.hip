@@ -640,7 +640,8 @@ __global__ __launch_bounds__(KV_THREADS) void attention_key_value_gradient_kerne
                     dsf[QB][N][2 * HALF] = pack_bf16(ds[0], ds[1]);
                     dsf[QB][N][2 * HALF + 1] = pack_bf16(ds[2], ds[3]);
                 });
-                *reinterpret_cast<u32x4*>(block + (ds_slot[N] + QB * 2048)) = dsf[QB][N];
+                // written once, read by the next kernel: kept out of the way of the tiles other workgroups re-read
+                __builtin_nontemporal_store(dsf[QB][N], reinterpret_cast<u32x4*>(block + (ds_slot[N] + QB * 2048)));
             });
             // dK += dS^T Q
             static_for<0, DK_MFMAS>([&](auto k_tag) {
@@ -766,8 +767,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
             const int part = load % 8;
             const unsigned char* block =
                 ds_head + (size_t)ds_block_index(kb, tile_index[t], query_tiles) * DS_BLOCK_BYTES + half * C::DS_HALF;
-            direct_load_16_offset(block, (unsigned)(part * 1024 + lane * 16),
-                                  target + C::K_BYTES + t * C::DS_HALF + part * 1024);
+            direct_load_16_offset_streaming(block, (unsigned)(part * 1024 + lane * 16),
+                                            target + C::K_BYTES + t * C::DS_HALF + part * 1024);
         }
     };
 

@@ -118,6 +118,15 @@ __device__ __forceinline__ void direct_load_16_offset(const void* uniform_base, 
                  : "memory", "m0");
 }
 
+// The same for data that is read once (a stream that should not push what others re-read out of the caches).
+__device__ __forceinline__ void direct_load_16_offset_streaming(const void* uniform_base, unsigned byte_offset,
+                                                                unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                 :
+                 : "v"(byte_offset), "s"(uniform_base), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
 // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
 // vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt/lgkmcnt unconstrained).
 template <int COUNT>

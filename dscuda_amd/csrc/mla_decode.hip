@@ -356,7 +356,7 @@ __device__ __forceinline__ void issue_unit_load(const UnitSource& source, const 
     const unsigned offset = source.full
         ? offsets.of[i]
         : index_math::contiguous_load_offset<ROW_BYTES, UNIT / 4>(wave, i, lane, source.row_limit);
-    direct_load_16_offset(source.base, offset, source.lds_base + i * 1024);
+    direct_load_16_offset_streaming(source.base, offset, source.lds_base + i * 1024);   // the cache is read once per call
 }
 
 // All nine loads of a unit at once: the first units of a walk, and every unit of the
