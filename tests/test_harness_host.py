@@ -148,6 +148,13 @@ def test_entry_point_needs_a_gpu():
     assert result.returncode != 0 and "needs a GPU" in result.stderr
 
 
+def test_the_benchmark_measures_one_gpu_only():
+    result = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                            cwd=ROOT, timeout=120)
+    assert result.returncode != 0
+    assert "one GPU" in result.stdout + result.stderr and result.stdout.count("{") == 0
+
+
 # ---- the PyTorch expressions the harness times and checks against, pinned on the CPU against the oracle -----------
 
 def test_harness_reference_matches_the_oracle_for_causal_attention():
