@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 from pathlib import Path
 
 import torch
@@ -54,6 +55,18 @@ def checked(lib, prefix, status):
     if status:
         error = bind(lib, f"dscuda_{prefix}_last_error", [], ctypes.c_char_p)
         raise RuntimeError(error().decode())
+
+
+def leave(status: int = 0):
+    """End a finished process that holds a GPU context: wait for the device, flush what was printed, and exit
+    without the exit-time teardown of the interpreter and the GPU libraries.  That teardown has ended such a
+    process in std::terminate ("terminate called without an active exception", status -6) after all of its
+    results were out.  Not for a run under a profiler: its tool writes the trace at exit."""
+    if torch.cuda.is_available() and torch.cuda.is_initialized():
+        torch.cuda.synchronize()
+    sys.stdout.flush()
+    sys.stderr.flush()
+    os._exit(status)
 
 
 def pointers(tensors):

@@ -151,7 +151,10 @@ def main(argv=None):
                     parser.error("No matching operations.")
                 continue
             print(text, end="")
+    return args
 
 
 if __name__ == "__main__":
-    main()
+    if not main().profile:   # a profiler around the process needs the ordinary exit
+        from dscuda_amd.harness import common
+        common.leave()

@@ -9,7 +9,7 @@ import sys
 
 import torch
 
-from dscuda_amd.harness import configs, ops
+from dscuda_amd.harness import common, configs, ops
 from oracle import attention_oracle as oracle
 from tests.parity import assert_close_bf16
 
@@ -33,3 +33,4 @@ def main(batch, tokens, heads):
 
 if __name__ == "__main__":
     main(*map(int, sys.argv[1:4]))
+    common.leave()
