@@ -278,12 +278,17 @@ def markdown_table(rows):
     return lines
 
 
-def portable(command: str) -> str:
-    """The recorded command with the checkout's location taken out: paths relative to the repository root,
-    the interpreter as `python3`."""
+def portable(command: str, out: Path) -> str:
+    """The recorded command with the checkout's location taken out: paths relative to the repository root
+    (recognised by the top-level folder of the raw output `out`, the package and the build folder), the
+    interpreter as `python3`."""
+    try:
+        raw = out.resolve().relative_to(ROOT.resolve()).parts[0]
+    except (ValueError, IndexError):
+        raw = out.name
     words = []
     for word in shlex.split(command):
-        for anchor in ("gpurun_out/", "dscuda_amd/", "build/"):
+        for anchor in (raw + "/", "dscuda_amd/", "build/"):
             cut = word.find("/" + anchor)
             if cut >= 0:
                 word = word[cut + 1:]
@@ -301,7 +306,7 @@ def write_case(case, rows, out, profiles, factors):
     for pass_name in PASSES:
         recorded = out / case.stem / pass_name / "command.txt"
         if recorded.exists():
-            lines.append(f"- {pass_name}: `{portable(recorded.read_text().strip())}`")
+            lines.append(f"- {pass_name}: `{portable(recorded.read_text().strip(), out)}`")
     lines += ["", f"Counter calibration from the 1 GiB copy: FETCH_SIZE x {factors[0]:.3f}, WRITE_SIZE x {factors[1]:.3f}.",
               "Durations are the mean of the second half of the launches of the timing pass.", ""]
     lines += markdown_table(rows)
@@ -341,7 +346,7 @@ def main(argv=None):
     parser.add_argument("family", choices=sorted(FAMILIES))
     parser.add_argument("suite", nargs="?", default="quick", choices=("quick", "full"))
     parser.add_argument("mode", nargs="?", default="profile", choices=("profile", "extract"))
-    parser.add_argument("--out", type=Path, default=ROOT / "gpurun_out" / "capture")
+    parser.add_argument("--out", type=Path, default=ROOT / "profiler_out" / "capture", help="raw profiler output")
     parser.add_argument("--profiles", type=Path, default=ROOT / "profiles")
     parser.add_argument("--only", action="append", default=[], help="case stems to run (default: all)")
     parser.add_argument("--passes", default=",".join(DEFAULT_PASSES))
