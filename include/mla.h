@@ -111,17 +111,17 @@ void mla_decode_forward_cuda(
 // kernels; the pattern of FlashMLA's get_mla_metadata, reference/python/flashmla.py:41-63) --
 //
 // Every decode call first turns the cache lengths into a small table: the tile
-// prefix of the batch, its cut into one range per workgroup and the per-sequence
-// tickets the ranges merge by.  mla_decode_forward_cuda builds that table inside
-// its workspace on every call.  A caller that decodes several layers (or steps)
-// over the same lengths builds it once:
+// prefix of the batch and its cut into one range per workgroup.
+// mla_decode_forward_cuda derives that table from the lengths on every call (for
+// the merge it leaves a copy inside its workspace).  A caller that decodes several
+// layers (or steps) over the same lengths builds it once:
 //     plan = device buffer of mla_decode_plan_elements(B, H, splits, C) ints
 //     mla_decode_plan_cuda(plan, lengths, B, H, C, splits, stream)
 //     for each layer: mla_decode_forward_planned_cuda(..., workspace, plan, ...)
 // The plan depends on the lengths, B, H and splits (all must be the same in the
-// calls that use it) and on nothing else.  The calls keep per-sequence counters
-// inside the plan and return them to zero, so calls that share a plan must be
-// ordered (one stream, or events): two of them in flight at once race.
+// calls that use it) and on the device's compute-unit count, and on nothing else.
+// The calls only read it: any number of them may share one plan, in any order and
+// on any streams (each with a workspace of its own).
 std::size_t mla_decode_plan_elements(
     int batch_size,
     int heads,
