@@ -212,7 +212,9 @@ void mla_prefill_forward_cuda(
 // (logsumexp in log2 units and delta = sum(dO * O), 128 floats per 64-query
 // tile) followed by the BF16 dS blocks the key/value-gradient pass hands to the
 // query-gradient pass, 16 KB per causal (128-key block, 64-query tile) pair --
-// about S*S bytes per (batch, head).  0 for non-positive sizes.
+// about S*S bytes per (batch, head), for as many (batch, head) pairs at a time as
+// fit 3 GiB (at least one): the two passes run over the pairs in chunks that share
+// that set of blocks.  0 for non-positive sizes.
 std::size_t mla_prefill_backward_workspace_elements(
     int batch_size,
     int sequence_length,
