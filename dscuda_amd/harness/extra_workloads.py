@@ -102,6 +102,27 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
     except Exception as error:
         results["mla_absorbed_T4096_H128"] = {"error": str(error)}
 
+    # the projections either side of the absorbed kernels, 4096 tokens x 128 heads: memory-bound by design
+    # (x and y rows once, the head's 128 KB weight from L2), so the rate is bytes of x + y + w over time
+    try:
+        tokens = 4096
+        nope = draw((tokens, heads, 128), 0.5)
+        weight = draw((heads, 128, 512), 0.05)
+        latent_rows = torch.empty(tokens, heads, 512, device=device, dtype=torch.bfloat16)
+        back = torch.empty(tokens, heads, 128, device=device, dtype=torch.bfloat16)
+        moved = (nope.numel() + latent_rows.numel() + weight.numel()) * 2
+        ms, _ = event_time_ms(lambda: ops.mla_absorb_query(nope, weight, latent_rows), 40, 10)
+        results["mla_absorb_query_T4096_H128"] = {"us": ms * 1000.0, "gbs": moved / ms / 1e6, "bytes": moved,
+                                                  "frac_of_hbm_peak": moved / ms / 1e6 / PEAK_HBM_GBS,
+                                                  "entry": "dscuda_mla_absorb_query"}
+        ms, _ = event_time_ms(lambda: ops.mla_unabsorb_output(latent_rows, weight, back), 40, 10)
+        results["mla_unabsorb_output_T4096_H128"] = {"us": ms * 1000.0, "gbs": moved / ms / 1e6, "bytes": moved,
+                                                     "frac_of_hbm_peak": moved / ms / 1e6 / PEAK_HBM_GBS,
+                                                     "entry": "dscuda_mla_unabsorb_output"}
+        del nope, weight, latent_rows, back
+    except Exception as error:
+        results["mla_projection_T4096_H128"] = {"error": str(error)}
+
     # for scale only: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this chip with random
     # operands, timed the same way; a plain GEMM is the practical ceiling of any MFMA-bound kernel here
     try:
