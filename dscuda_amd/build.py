@@ -47,8 +47,6 @@ PROGRAMS = {
     "benchmark_mla_decode": ("benchmark_mla_decode.cpp", "libdscuda_mla_bench.so"),
     "benchmark_mla_prefill": ("benchmark_mla_prefill.cpp", "libdscuda_mla_bench.so"),
     "benchmark_flash_attention": ("benchmark_flash_attention.cpp", "libdscuda_flash_attention_bench.so"),
-    "hbm_read_probe": ("hbm_read_probe.hip", "libdscuda_mla_bench.so"),   # links nothing of the library; one recipe for all
-    "issue_probe": ("issue_probe.hip", "libdscuda_mla_bench.so"),
 }
 PROFILER = ROOT / "dscuda_amd" / "profiler"
 

@@ -64,6 +64,10 @@ std::size_t flash_attention_backward_workspace_elements(int batch_size, int sequ
     return attention_backward_workspace_elements(batch_size, sequence_length, query_heads, key_value_heads);
 }
 
+void flash_attention_backward_set_workspace_limit(std::size_t bytes) {
+    attention_backward_set_workspace_limit(bytes);
+}
+
 void flash_attention_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
                                    __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
                                    const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
@@ -105,7 +109,17 @@ extern "C" int dscuda_flash_forward(__hip_bfloat16* output, float* logsumexp, co
 
 extern "C" std::size_t dscuda_flash_backward_workspace_elements(int batch, int sequence, int query_heads,
                                                                 int key_value_heads, int dimension) {
-    return dscuda::flash_attention_backward_workspace_elements(batch, sequence, query_heads, key_value_heads, dimension);
+    try {
+        return dscuda::flash_attention_backward_workspace_elements(batch, sequence, query_heads, key_value_heads,
+                                                                   dimension);
+    } catch (const std::exception& error) {
+        last_error = error.what();
+        return 0;
+    }
+}
+
+extern "C" void dscuda_flash_backward_set_workspace_limit(std::size_t bytes) {
+    dscuda::flash_attention_backward_set_workspace_limit(bytes);
 }
 
 extern "C" int dscuda_flash_backward(__hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,

@@ -38,17 +38,10 @@ void check_positive(const char* what, int batch_size, int tokens, int heads) {
 // looked up once per device and every use below goes through that pointer.
 __device__ __align__(256) unsigned char static_decode_scratch[MLA_DECODE_STATIC_SCRATCH_BYTES];
 
-constexpr int MAX_DEVICES = 64;
-
 float* static_decode_scratch_of_current_device() {
     static std::mutex guard;
-    static void* address_of_device[MAX_DEVICES] = {};
-    int device = 0;
-    HIP_CHECK(hipGetDevice(&device));
-    if (device < 0 || device >= MAX_DEVICES) {
-        throw std::runtime_error("MLA decode (static workspace): device index " + std::to_string(device) +
-                                 " is beyond the " + std::to_string(MAX_DEVICES) + " devices supported");
-    }
+    static void* address_of_device[hip_common::MAX_DEVICES] = {};
+    const int device = hip_common::current_device();
     std::lock_guard<std::mutex> lock(guard);
     if (address_of_device[device] == nullptr) {
         void* address = nullptr;
@@ -188,6 +181,14 @@ std::size_t mla_prefill_backward_workspace_elements(int batch_size, int sequence
     return attention_backward_workspace_elements(batch_size, sequence_length, heads, heads);
 }
 
+void mla_prefill_backward_set_workspace_limit(std::size_t bytes) {
+    attention_backward_set_workspace_limit(bytes);
+}
+
+void mla_backward_set_key_interval_tiles(int tiles) {
+    mla_absorbed_backward_set_key_interval_tiles(tiles);
+}
+
 void mla_prefill_backward_cuda(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
                                __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
                                const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
@@ -272,7 +273,9 @@ extern "C" int dscuda_mla_backward(__hip_bfloat16* dquery, __hip_bfloat16* dquer
 }
 
 extern "C" std::size_t dscuda_mla_workspace_elements(int batch, int heads, int splits, int rank) {
-    return dscuda::mla_decode_workspace_elements(batch, heads, splits, rank);
+    std::size_t elements = 0;
+    guarded([&] { elements = dscuda::mla_decode_workspace_elements(batch, heads, splits, rank); });
+    return elements;
 }
 
 extern "C" int dscuda_mla_decode(__hip_bfloat16* output, float* lse, const __hip_bfloat16* query,
@@ -286,7 +289,9 @@ extern "C" int dscuda_mla_decode(__hip_bfloat16* output, float* lse, const __hip
 }
 
 extern "C" std::size_t dscuda_mla_decode_plan_elements(int batch, int heads, int splits, int rank) {
-    return dscuda::mla_decode_plan_elements(batch, heads, splits, rank);
+    std::size_t elements = 0;
+    guarded([&] { elements = dscuda::mla_decode_plan_elements(batch, heads, splits, rank); });
+    return elements;   // 0 with the message set when the arguments admit no plan
 }
 
 extern "C" int dscuda_mla_decode_plan(int* plan, const int* lengths, int batch, int heads, int rank, int splits,
@@ -326,7 +331,19 @@ extern "C" int dscuda_mla_prefill_forward(__hip_bfloat16* output, float* lse, co
 
 extern "C" std::size_t dscuda_mla_prefill_backward_workspace_elements(int batch, int sequence, int heads,
                                                                       int qk_head_size, int v_head_size) {
-    return dscuda::mla_prefill_backward_workspace_elements(batch, sequence, heads, qk_head_size, v_head_size);
+    std::size_t elements = 0;
+    guarded([&] {
+        elements = dscuda::mla_prefill_backward_workspace_elements(batch, sequence, heads, qk_head_size, v_head_size);
+    });
+    return elements;
+}
+
+extern "C" void dscuda_mla_prefill_backward_set_workspace_limit(std::size_t bytes) {
+    dscuda::mla_prefill_backward_set_workspace_limit(bytes);
+}
+
+extern "C" void dscuda_mla_backward_set_key_interval_tiles(int tiles) {
+    dscuda::mla_backward_set_key_interval_tiles(tiles);
 }
 
 extern "C" int dscuda_mla_prefill_backward(__hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,

@@ -926,17 +926,15 @@ void raise_lds_limit(Kernel kernel, int bytes) {
 // tens of gigabytes if every pair kept its own.  The two gradient passes therefore run over the pairs in chunks that
 // share one set of dS blocks of at most DS_BUDGET_BYTES (the chunk of a launch is a multiple of 8 pairs when it can
 // be: one pair at a time per XCD); the statistics, small, are computed for all pairs at once.
-// DSCUDA_AMD_DS_BUDGET_BYTES in the environment (read once) replaces the budget: for tests of the chunked path at
-// small sizes, and for callers who would rather trade launches for memory.
+// attention_backward_set_workspace_limit replaces the budget for the whole process: for callers who would rather
+// trade launches for memory (and for tests of the chunked path at small sizes).
 constexpr long long DS_BUDGET_BYTES = 3LL << 30;
 
+std::atomic<long long> ds_budget_override{0};
+
 long long ds_budget_bytes() {
-    static const long long budget = [] {
-        const char* text = std::getenv("DSCUDA_AMD_DS_BUDGET_BYTES");
-        const long long value = text ? std::strtoll(text, nullptr, 10) : 0;
-        return value > 0 ? value : DS_BUDGET_BYTES;
-    }();
-    return budget;
+    const long long value = ds_budget_override.load(std::memory_order_relaxed);
+    return value > 0 ? value : DS_BUDGET_BYTES;
 }
 
 struct BackwardShape {
@@ -986,12 +984,11 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
     }
     float* statistics = workspace;
     unsigned char* ds_blocks = reinterpret_cast<unsigned char*>(workspace + shape.statistics_floats);
-    static thread_local bool prepared = false;
-    if (!prepared) {
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] {
         raise_lds_limit(attention_key_value_gradient_kernel<DQK, DV>, KC::LDS_BYTES);
         raise_lds_limit(attention_query_gradient_kernel<DQK>, QC::LDS_BYTES);
-        prepared = true;
-    }
+    });
     hipLaunchKernelGGL((attention_backward_statistics_kernel<DV>), dim3((unsigned)((padded_rows + 15) / 16)), dim3(256),
                        0, stream, statistics, output_gradient, output, logsumexp, batch_size, sequence_length, heads,
                        shape.query_tiles);
@@ -1014,6 +1011,10 @@ void launch_backward(bf16_t* query_gradient, bf16_t* key_gradient, bf16_t* value
 }
 
 }  // namespace
+
+void attention_backward_set_workspace_limit(std::size_t bytes) {
+    ds_budget_override.store(bytes > (std::size_t)1 << 62 ? 1LL << 62 : (long long)bytes, std::memory_order_relaxed);
+}
 
 std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads, int kv_heads) {
     if (kv_heads <= 0 || heads % kv_heads != 0) {

@@ -756,12 +756,11 @@ void launch_forward(bf16_t* output, float* logsumexp, const bf16_t* query, const
     }
     auto kernel = attention_forward_kernel<DQK, DV, NWAVES>;
     if (C::LDS_BYTES > 64 * 1024) {
-        static thread_local bool raised = false;  // attribute is per function, setting it is idempotent
-        if (!raised) {
+        static hip_common::OncePerDevice raised;
+        raised.run([&] {
             HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES));
-            raised = true;
-        }
+        });
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::THREADS), C::LDS_BYTES, stream, output, logsumexp, query,
                        key, value, sequence_length, query_heads, key_value_heads, query_blocks, scale);
@@ -784,12 +783,7 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
         throw std::invalid_argument("attention forward: key_value_heads * head size is too large");
     }
     // one workgroup per compute unit (the LDS footprint admits no second one)
-    static thread_local int compute_units = 0;
-    if (compute_units == 0) {
-        int device = 0;
-        HIP_CHECK(hipGetDevice(&device));
-        HIP_CHECK(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
-    }
+    const int compute_units = hip_common::compute_units_of_current_device();
     const int clusters = (batch_heads % PingPong::CLUSTERS == 0 && compute_units >= PingPong::CLUSTERS)
                              ? PingPong::CLUSTERS : 1;
     long long grid = compute_units / clusters * clusters;
@@ -798,12 +792,11 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
         grid = items_per_cluster * clusters;
     }
     auto kernel = attention_forward_pingpong_kernel<DQK, DV>;
-    static thread_local bool raised = false;
-    if (!raised) {
+    static hip_common::OncePerDevice raised;
+    raised.run([&] {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-        raised = true;
-    }
+    });
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::THREADS), LDS_BYTES, stream, output, logsumexp, query,
                        key, value, sequence_length, query_heads, key_value_heads, query_blocks, (int)batch_heads,
                        clusters, scale);

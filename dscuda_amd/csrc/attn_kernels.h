@@ -24,6 +24,9 @@ void attention_forward_dispatch(__hip_bfloat16* output, float* logsumexp, const 
 // statistics and the bf16 dS blocks handed from the dK/dV kernel to the dQ pass.
 std::size_t attention_backward_workspace_elements(int batch_size, int sequence_length, int heads, int kv_heads);
 
+// Bytes the dS blocks of one chunk of (batch, key/value head) pairs may take (0: the built-in 3 GiB); process-wide.
+void attention_backward_set_workspace_limit(std::size_t bytes);
+
 void attention_backward_dispatch(__hip_bfloat16* query_gradient, __hip_bfloat16* key_gradient,
                                  __hip_bfloat16* value_gradient, const __hip_bfloat16* output_gradient,
                                  const __hip_bfloat16* output, const float* logsumexp, const __hip_bfloat16* query,
@@ -64,6 +67,9 @@ void mla_absorbed_backward_dispatch(__hip_bfloat16* query_latent_gradient, __hip
                                     const __hip_bfloat16* query_rope, const __hip_bfloat16* kv_latent,
                                     const __hip_bfloat16* key_rope, int batch_size, int sequence_length, int heads,
                                     float scale, hipStream_t stream);
+
+// > 0: the key-gradient pass cuts its work by intervals of that many row tiles at any size; 0: its own choice.
+void mla_absorbed_backward_set_key_interval_tiles(int tiles);
 
 // mla_decode.hip -- absorbed single-token decode over a paged latent cache.  `plan` is
 // the int table mla_decode_plan_dispatch writes for the same batch, heads and splits

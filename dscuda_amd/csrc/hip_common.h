@@ -24,6 +24,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 #include <sstream>
@@ -46,6 +47,54 @@ inline void hip_check(hipError_t result, const char* expression, const char* fil
 #define HIP_CHECK(expression) ::dscuda::hip_check((expression), #expression, __FILE__, __LINE__)
 
 using bf16_t = __hip_bfloat16;
+
+// What the host side remembers per device: attributes of a kernel (hipFuncSetAttribute acts on
+// the current device's copy of the function) and device properties are set or asked once for
+// each device a thread makes current, not once per thread or per process.
+namespace hip_common {
+
+constexpr int MAX_DEVICES = 64;
+
+inline int current_device() {
+    int device = 0;
+    HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= MAX_DEVICES) {
+        throw std::runtime_error("device index " + std::to_string(device) + " is beyond the " +
+                                 std::to_string(MAX_DEVICES) + " devices this library keeps state for");
+    }
+    return device;
+}
+
+// Runs `prepare` the first time it is asked to on each device.  Two threads may both run it for
+// the same device (the preparation is idempotent); none skips it before it has completed once.
+class OncePerDevice {
+public:
+    template <typename Prepare>
+    void run(Prepare&& prepare) {
+        const int device = current_device();
+        if (!done_[device].load(std::memory_order_acquire)) {
+            prepare();
+            done_[device].store(true, std::memory_order_release);
+        }
+    }
+
+private:
+    std::atomic<bool> done_[MAX_DEVICES] = {};
+};
+
+// Compute units of the current device, asked once per device.
+inline int compute_units_of_current_device() {
+    static std::atomic<int> units_of_device[MAX_DEVICES] = {};
+    const int device = current_device();
+    int units = units_of_device[device].load(std::memory_order_relaxed);
+    if (units == 0) {
+        HIP_CHECK(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+        units_of_device[device].store(units, std::memory_order_relaxed);
+    }
+    return units;
+}
+
+}  // namespace hip_common
 
 #if defined(__HIP_DEVICE_COMPILE__) || defined(__HIPCC__)
 

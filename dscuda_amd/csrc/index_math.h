@@ -359,6 +359,13 @@ DSCUDA_HOST_DEVICE inline long long plan_first_sequence_at(int batch) { return P
 DSCUDA_HOST_DEVICE inline long long plan_elements(int batch, int workgroups) {
     return plan_first_sequence_at(batch) + workgroups;
 }
+// Size of a plan buffer that fits whatever device builds the plan: a call cuts its list into at
+// most one range per compute unit (the host clamps the count it asks the device for to
+// PLAN_MAX_WORKGROUPS), or runs one workgroup per sequence.
+constexpr int PLAN_MAX_WORKGROUPS = 1024;
+DSCUDA_HOST_DEVICE inline long long plan_elements_bound(int batch) {
+    return plan_elements(batch, batch > PLAN_MAX_WORKGROUPS ? batch : PLAN_MAX_WORKGROUPS);
+}
 
 // The caller's workspace holds batch * heads * splits * (rank + 2) floats.  A
 // range that holds only part of a sequence leaves its unnormalised result there:

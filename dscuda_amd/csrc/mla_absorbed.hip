@@ -757,30 +757,23 @@ void raise_lds_limit(Kernel kernel, int bytes) {
 constexpr long long LARGE_INPUT_BYTES = 64LL << 20;   // per batch element, against 32 MB of L2 and 256 MB behind it
 constexpr int INTERVAL_TILES = 256;                   // 18 MB of rows
 
-// DSCUDA_AMD_KEY_INTERVAL_TILES in the environment (read once per process) forces the interval cut with that many
-// row tiles per interval at any size the slots allow: the cut can then be exercised at sizes a test can check.
+// mla_absorbed_backward_set_key_interval_tiles (> 0) forces the interval cut with that many row tiles per interval at
+// any size the slots allow; 0 gives the choice back to the dispatch below.
+std::atomic<int> forced_key_interval_tiles{0};
+
 int forced_interval_tiles() {
-    static const int forced = [] {
-        const char* text = std::getenv("DSCUDA_AMD_KEY_INTERVAL_TILES");
-        const long value = text ? std::strtol(text, nullptr, 10) : 0;
-        return value > 0 && value < (1 << 24) ? (int)value : 0;
-    }();
-    return forced;
+    return forced_key_interval_tiles.load(std::memory_order_relaxed);
 }
 
 int device_compute_units() {
-    static thread_local int device_of = -1;
-    static thread_local int units = 0;
-    int device = 0;
-    HIP_CHECK(hipGetDevice(&device));
-    if (device != device_of) {
-        HIP_CHECK(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
-        device_of = device;
-    }
-    return units;
+    return hip_common::compute_units_of_current_device();
 }
 
 }  // namespace
+
+void mla_absorbed_backward_set_key_interval_tiles(int tiles) {
+    forced_key_interval_tiles.store(tiles > 0 && tiles < (1 << 24) ? tiles : 0, std::memory_order_relaxed);
+}
 
 void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query_rope_gradient,
                                     bf16_t* kv_latent_gradient, bf16_t* key_rope_gradient,
@@ -797,12 +790,11 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
         reinterpret_cast<uintptr_t>(query_rope_gradient) % 16 != 0) {
         throw std::invalid_argument("MLA backward: the query gradients must be aligned to 16 bytes");
     }
-    static thread_local bool prepared = false;
-    if (!prepared) {
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] {
         raise_lds_limit(mla_absorbed_query_gradient_kernel, QueryGradLayout::LDS_BYTES);
         raise_lds_limit(mla_absorbed_key_gradient_kernel, KeyGradLayout::LDS_BYTES);
-        prepared = true;
-    }
+    });
     // scratch memory until the last launch: delta in the rope query gradients, partial key gradients in the latent ones
     float* delta = reinterpret_cast<float*>(query_rope_gradient);
     float* partial_slots = reinterpret_cast<float*>(query_latent_gradient);

@@ -1084,21 +1084,18 @@ void allow_large_lds(Kernel kernel) {
                                   LDS_BYTES));
 }
 
+// The count decides how many ranges a call's work list is cut into, so it is clamped to the bound
+// the plan size below is computed for.
 int compute_units() {
-    static thread_local int cached = 0;
-    if (cached == 0) {
-        int device = 0;
-        HIP_CHECK(hipGetDevice(&device));
-        HIP_CHECK(hipDeviceGetAttribute(&cached, hipDeviceAttributeMultiprocessorCount, device));
-    }
-    return cached;
+    return std::min(std::max(hip_common::compute_units_of_current_device(), 1), index_math::PLAN_MAX_WORKGROUPS);
 }
 
 }  // namespace
 
-std::size_t mla_decode_plan_elements(int batch_size, int heads, int splits) {
-    const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
-    return static_cast<std::size_t>(layout.plan_ints);
+std::size_t mla_decode_plan_elements(int batch_size, int /*heads*/, int /*splits*/) {
+    // Pure arithmetic, no device needed (as the reference's workspace size, kernels/attention/mla/sm89.cu:539-541):
+    // room for the plan of any device this library runs on.
+    return static_cast<std::size_t>(index_math::plan_elements_bound(batch_size));
 }
 
 void mla_decode_plan_dispatch(int* plan, const int* cache_lengths, int batch_size, int heads, int splits,
@@ -1116,11 +1113,8 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) {
         throw std::invalid_argument("MLA decode requires a workspace aligned to 16 bytes");
     }
-    static thread_local bool prepared = false;
-    if (!prepared) {
-        allow_large_lds(mla_decode_split_kernel);
-        prepared = true;
-    }
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] { allow_large_lds(mla_decode_split_kernel); });
     // How the caller's B*H*splits*(C+2) floats are used: index_math::decode_layout.
     const index_math::DecodeLayout layout = index_math::decode_layout(batch_size, heads, splits, compute_units(), ROWS, RANK);
     int own_workgroups = 0;
@@ -1153,11 +1147,8 @@ void mla_decode_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query, 
 void mla_absorbed_forward_dispatch(bf16_t* output, float* logsumexp, const bf16_t* query_latent,
                                    const bf16_t* query_rope, const bf16_t* kv_latent, const bf16_t* key_rope,
                                    int batch_size, int sequence_length, int heads, float scale, hipStream_t stream) {
-    static thread_local bool prepared = false;
-    if (!prepared) {
-        allow_large_lds(mla_absorbed_forward_kernel);
-        prepared = true;
-    }
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] { allow_large_lds(mla_absorbed_forward_kernel); });
     const long long rows = (long long)sequence_length * heads;
     const long long row_blocks = (rows + ROWS - 1) / ROWS;
     if (row_blocks * batch_size > 0x7fffffffLL) {

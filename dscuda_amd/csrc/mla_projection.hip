@@ -259,15 +259,7 @@ void check(bool condition, const char* message) {
 }
 
 int compute_units() {
-    static thread_local int device_of = -1;
-    static thread_local int units = 0;
-    int device = 0;
-    HIP_CHECK(hipGetDevice(&device));
-    if (device != device_of) {
-        HIP_CHECK(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
-        device_of = device;
-    }
-    return units;
+    return hip_common::compute_units_of_current_device();
 }
 
 // One staging of a head's weight should serve as many tokens as possible while the grid still covers the chip
@@ -310,12 +302,11 @@ void mla_absorb_query_dispatch(bf16_t* query_latent, const bf16_t* query_nope, c
     const Strides strides = {query_nope_token_stride, query_nope_head_stride, query_latent_token_stride,
                              query_latent_head_stride, weight_head_stride};
     validate(query_latent, query_nope, weight, tokens, heads, strides, HEAD, RANK);
-    static thread_local bool prepared = false;
-    if (!prepared) {
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(mla_absorb_query_kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-        prepared = true;
-    }
+    });
     launch(mla_absorb_query_kernel, query_latent, query_nope, weight, tokens, heads, strides, stream);
 }
 
@@ -326,12 +317,11 @@ void mla_unabsorb_output_dispatch(bf16_t* output, const bf16_t* output_latent, c
     const Strides strides = {output_latent_token_stride, output_latent_head_stride, output_token_stride,
                              output_head_stride, weight_head_stride};
     validate(output, output_latent, weight, tokens, heads, strides, RANK, HEAD);
-    static thread_local bool prepared = false;
-    if (!prepared) {
+    static hip_common::OncePerDevice prepared;
+    prepared.run([] {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(mla_unabsorb_output_kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-        prepared = true;
-    }
+    });
     launch(mla_unabsorb_output_kernel, output, output_latent, weight, tokens, heads, strides, stream);
 }
 

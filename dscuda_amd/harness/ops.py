@@ -45,6 +45,8 @@ class _Mla:
         self.prefill_backward = bind(lib, "dscuda_mla_prefill_backward", [P] * 10 + [I] * 5 + [F, P])
         self.prefill_workspace = bind(
             lib, "dscuda_mla_prefill_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
+        self.prefill_workspace_limit = bind(lib, "dscuda_mla_prefill_backward_set_workspace_limit", [ctypes.c_size_t], None)
+        self.key_interval_tiles = bind(lib, "dscuda_mla_backward_set_key_interval_tiles", [I], None)
 
 
 class _Flash:
@@ -54,6 +56,7 @@ class _Flash:
         self.forward = bind(lib, "dscuda_flash_forward", [P] * 5 + [I] * 5 + [F, P])
         self.backward = bind(lib, "dscuda_flash_backward", [P] * 10 + [I] * 5 + [F, P])
         self.backward_workspace = bind(lib, "dscuda_flash_backward_workspace_elements", [I] * 5, ctypes.c_size_t)
+        self.backward_workspace_limit = bind(lib, "dscuda_flash_backward_set_workspace_limit", [ctypes.c_size_t], None)
 
 
 _mla = None
@@ -102,6 +105,16 @@ def mla_prefill_forward(query, key, value, scale, out=None, lse=None):
 def mla_prefill_backward_workspace_elements(batch, seq, heads, dqk, dv):
     """fp32 elements of the per-head backward's workspace (dscuda_mla_prefill_backward_workspace_elements)."""
     return mla_library().prefill_workspace(batch, seq, heads, dqk, dv)
+
+
+def mla_prefill_backward_set_workspace_limit(limit_bytes: int) -> None:
+    """Process-wide bound on the dS blocks of one chunk of (batch, head) pairs; 0 restores the built-in 3 GiB."""
+    mla_library().prefill_workspace_limit(int(limit_bytes))
+
+
+def mla_backward_set_key_interval_tiles(tiles: int) -> None:
+    """Force the interval cut of the absorbed backward's key-gradient pass (0: the library's own choice)."""
+    mla_library().key_interval_tiles(int(tiles))
 
 
 def mla_prefill_backward_workspace(batch, seq, heads, dqk, dv, device="cuda"):

@@ -102,15 +102,20 @@ def run_family(family: str, args) -> str | None:
     import torch
     workloads = catalogue.select(family, args.suite, args.test, args.operation)
     rows, samples = [], []
+    # A profiler run of the library alone binds no PyTorch expression: nothing but the library's kernels runs in
+    # the process, and no autograd worker thread is ever started in it (see `finish`).
+    library_only = args.profile and args.backend == "custom"
     for workload in workloads:
-        bound = catalogue.bind(workload, args.with_reference)
+        bound = catalogue.bind(workload, args.with_reference and not library_only)
         if args.test and bound.expected is None:
             raise RuntimeError(f"{family}: {workload.label}: a correctness test needs a PyTorch result to compare with")
-        check_once(bound, only_custom=args.test)
+        check_once(bound, only_custom=args.test or library_only)
         if args.test:
+            del bound
             continue
         if args.profile:
             profile_once(bound, args.backend)
+            del bound
             continue
         try:
             timings = replay.time_backends(bound.backends, args.settings, bound.verify)
@@ -131,9 +136,42 @@ def run_family(family: str, args) -> str | None:
     return tables.write(args.output, family, rows, samples, environment)
 
 
+def finish(profile: bool) -> None:
+    """Orderly end of a run: nothing of this process is left in flight or alive on the device side before the
+    interpreter starts taking itself apart.
+
+    One run of ``mla_prefill --test`` ended, after all results were printed and with every check passed, in
+    ``terminate called without an active exception`` (abort at interpreter exit); runs of the same command before and
+    after did not.  That message is the C++ runtime's for std::terminate() reached with no exception in flight: a
+    joinable std::thread destroyed, or a thread unwound by force through a noexcept frame, which is what CPython 3.10
+    does (pthread_exit) to a non-Python thread that asks for the GIL while the interpreter finalises.  This library
+    starts no threads and registers no exit handlers; the process that aborted had, unlike the runs of the other
+    families' ``--test`` that day, used PyTorch's autograd worker thread within milliseconds of its exit (the last
+    workload of that family is a backward check whose expected gradients come from ``torch.autograd.grad``).  The
+    cause has not been shown beyond that, so the exit is made as quiet as this module can make it: references
+    dropped and collected, the device idle and its cached blocks returned, output flushed; then a timed run leaves
+    through ``common.leave`` (no exit-time teardown at all), while a profiler run, whose tool writes its trace from
+    an exit handler, takes the ordinary exit, having started no autograd thread when only the library is profiled.
+    ``faulthandler`` is armed in ``main`` so that an abort, should one come again, names the threads alive in it."""
+    import gc
+
+    import torch
+    gc.collect()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    sys.stdout.flush()
+    sys.stderr.flush()
+    if not profile:
+        from dscuda_amd.harness import common
+        common.leave()
+
+
 def main(argv=None):
     parser, args = parse(argv)
+    import faulthandler
+
     import torch
+    faulthandler.enable()
     if not torch.cuda.is_available():
         sys.exit("dscuda_amd.harness.run needs a GPU")
     torch.manual_seed(2026)
@@ -151,10 +189,10 @@ def main(argv=None):
                     parser.error("No matching operations.")
                 continue
             print(text, end="")
+    torch.cuda.current_stream().wait_stream(side)
+    del side
     return args
 
 
 if __name__ == "__main__":
-    if not main().profile:   # a profiler around the process needs the ordinary exit
-        from dscuda_amd.harness import common
-        common.leave()
+    finish(main().profile)

@@ -42,6 +42,11 @@ std::size_t flash_attention_backward_workspace_elements(
     int key_value_heads,
     int head_size);
 
+// Replaces, for the whole process, the 3 GiB that the dS blocks of one chunk of (batch,
+// key/value head) pairs may take (0 restores it): set it before asking for the workspace
+// size and leave it unchanged until the backward call has been issued.
+void flash_attention_backward_set_workspace_limit(std::size_t bytes);
+
 // Recompute-based backward of flash_attention_forward_cuda from the saved BF16 output and
 // FP32 logsumexp; it has no counterpart in the reference (whose flash attention is forward
 // only, include/flash_attention.h:12-24).  dQ [B,T,Hq,D], dK and dV [B,T,Hkv,D] are
@@ -84,6 +89,8 @@ int dscuda_flash_forward(  // flash_attention_bridge.cu:17-30
 // additive (no counterpart in the reference): see dscuda::flash_attention_backward_cuda above
 std::size_t dscuda_flash_backward_workspace_elements(
     int batch, int sequence, int query_heads, int key_value_heads, int dimension);
+
+void dscuda_flash_backward_set_workspace_limit(std::size_t bytes);
 
 int dscuda_flash_backward(
     __hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,

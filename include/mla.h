@@ -107,6 +107,18 @@ void mla_decode_forward_cuda(
     float scale,
     hipStream_t stream = nullptr);
 
+// ---- additive: a tuning knob of mla_compressed_attention_backward_cuda (no counterpart in
+// the reference) -----------------------------------------------------------------------
+//
+// The key-gradient pass cuts its (key block, row tile) visits in one of two ways: into
+// equal ranges, or -- when the query and dO rows of a batch element outgrow the caches --
+// into (interval of row tiles, key block) items so that the workgroups running at one time
+// walk the same rows.  tiles > 0 forces the second cut with that many 32-row tiles per
+// interval at any size (as far as the partial-result slots inside dq_latent allow); 0, the
+// default, leaves the choice to the library.  Process-wide; the results do not depend on it
+// beyond the order of fp32 summation.
+void mla_backward_set_key_interval_tiles(int tiles);
+
 // ---- additive: a decode plan that outlives one call (no counterpart in the reference's
 // kernels; the pattern of FlashMLA's get_mla_metadata, reference/python/flashmla.py:41-63) --
 //
@@ -119,7 +131,10 @@ void mla_decode_forward_cuda(
 //     mla_decode_plan_cuda(plan, lengths, B, H, C, splits, stream)
 //     for each layer: mla_decode_forward_planned_cuda(..., workspace, plan, ...)
 // The plan depends on the lengths, B, H and splits (all must be the same in the
-// calls that use it) and on the device's compute-unit count, and on nothing else.
+// calls that use it) and on the compute-unit count of the device that built it, and
+// on nothing else.  mla_decode_plan_elements is plain arithmetic on its arguments
+// (no device is asked, so it can be called on a host without a GPU): room for the
+// plan of any device, 0 for arguments that admit no plan.
 // The calls only read it: any number of them may share one plan, in any order and
 // on any streams (each with a workspace of its own).
 std::size_t mla_decode_plan_elements(
@@ -221,6 +236,13 @@ std::size_t mla_prefill_backward_workspace_elements(
     int heads,
     int qk_head_size,
     int v_head_size);
+
+// Replaces, for the whole process, the 3 GiB that the dS blocks of one chunk of
+// (batch, head) pairs may take (0 restores it): a caller short of memory trades
+// more launches for a smaller workspace.  Set it before asking for the workspace
+// size and leave it unchanged until the backward call that uses that workspace has
+// been issued.  No counterpart in the reference.
+void mla_prefill_backward_set_workspace_limit(std::size_t bytes);
 
 // Recompute-based backward of mla_prefill_forward_cuda from the saved BF16
 // output and FP32 logsumexp.  dQ/dK [B,S,H,d_qk] and dV [B,S,H,d_v] are
@@ -369,6 +391,10 @@ int dscuda_mla_prefill_forward(
 
 std::size_t dscuda_mla_prefill_backward_workspace_elements(
     int batch, int sequence, int heads, int qk_head_size, int v_head_size);
+
+// additive (no counterpart in the reference): tuning knobs, see the dscuda:: functions of the same names above
+void dscuda_mla_prefill_backward_set_workspace_limit(std::size_t bytes);
+void dscuda_mla_backward_set_key_interval_tiles(int tiles);
 
 int dscuda_mla_prefill_backward(
     __hip_bfloat16* dquery, __hip_bfloat16* dkey, __hip_bfloat16* dvalue,

@@ -22,7 +22,9 @@ the headline configurations has no counterpart in the reference; its oracle
 is textbook causal attention with ``d_v != d_qk`` in the same style.  The
 two per-head projections either side of absorbed attention are likewise
 outside the reference (``reference/python/sources.json:2``); their oracle is
-one einsum each.
+one einsum each.  Rotary embedding is left to the caller by the reference as
+well (same line); ``apply_rope`` states DeepSeek-V3's convention as a complex
+multiplication.
 
 How each function is pinned (see ``tests/test_oracle_pins.py``):
 
@@ -46,6 +48,13 @@ mla_decode             SDPA with a length mask; equals row T-1 of the
                        causal prefill when len == T; closed form of
                        ``benchmark_mla_decode.cu:42-48``
 pack_cache             closed form (identity table, zero padding)
+apply_rope             closed forms: the unit pair (1, 0) at position p becomes
+                       (cos, sin) of p * theta^(-2i/R); position 0 is the
+                       identity; R = 2 leaves the single angle p; rotations
+                       compose (p then q == p + q); relative-position
+                       property of the rotated dot product; a half-split
+                       pairing, a reversed direction and a -i/R exponent
+                       each fail those checks
 absorb_query,          fp64 triple-loop brute force; the identity absorption
 unabsorb_output        rests on: scores and outputs of per-head attention
                        over k_nope = latent W_UK^T, v = latent W_UV^T equal
@@ -257,3 +266,18 @@ def unabsorb_output(output_latent, w_uv):
     """out[..., h, d] = sum_c output_latent[..., h, c] * w_uv[h, d, c] in fp32: the step after absorbed attention
     (the latent output times the last 128 rows per head of wkv_b, same source)."""
     return torch.einsum("...hc,hdc->...hd", _compute(output_latent), _compute(w_uv))
+
+
+def apply_rope(x, theta=10000.0, start=0):
+    """Rotary position embedding of the last dimension of x [B, S, H, R], positions start .. start + S - 1, in the
+    convention of DeepSeek-V3's ``apply_rotary_emb``: consecutive columns (2i, 2i + 1) are the real and imaginary
+    part of one complex number, multiplied by ``exp(1j * position * theta ** (-2i / R))``.  The reference leaves this
+    step to its caller (reference/python/sources.json:2), so the convention is this build's choice; it is stated here
+    through complex arithmetic in fp64, independently of the real-arithmetic formulation the workloads are generated
+    with.  Returns fp64."""
+    batch, seq, heads, width = x.shape
+    pairs = torch.view_as_complex(x.double().reshape(batch, seq, heads, width // 2, 2).contiguous())
+    frequency = float(theta) ** (-2.0 * torch.arange(width // 2, dtype=torch.float64) / width)
+    position = torch.arange(start, start + seq, dtype=torch.float64)
+    rotation = torch.polar(torch.ones(seq, width // 2, dtype=torch.float64), position[:, None] * frequency[None, :])
+    return torch.view_as_real(pairs * rotation[None, :, None, :]).reshape(batch, seq, heads, width)

@@ -54,6 +54,41 @@ def test_workspace_elements_match_the_reference_formula():
     assert prefill(0, 65, 3, 192, 128) == 0
 
 
+def test_size_queries_need_no_device():
+    """Every size query is arithmetic on its integer arguments (benchmarks/bindings/mla_bridge.cu:53-56 is): on a host
+    without a GPU it returns, in a process of its own so that an exception let through the C boundary shows up as a
+    failed status here instead of ending the test run."""
+    import subprocess
+    import sys
+    script = """
+import ctypes, sys
+from dscuda_amd.harness.common import I, bind, library
+mla, flash = library("mla"), library("flash_attention")
+size_t = ctypes.c_size_t
+plan = bind(mla, "dscuda_mla_decode_plan_elements", [I] * 4, size_t)
+assert plan(2, 3, 8, 512) == 5 + 2 + 1 + 1024, plan(2, 3, 8, 512)        # header, prefix, one entry per range
+assert plan(64, 128, 8, 512) == 5 + 64 + 1 + 1024
+assert plan(3500, 128, 8, 512) == 5 + 3500 + 1 + 3500                    # one workgroup per sequence at most
+assert plan(2, 3, 8, 256) == 0 and plan(0, 3, 8, 512) == 0 and plan(2, 3, 0, 512) == 0
+assert bind(mla, "dscuda_mla_workspace_elements", [I] * 4, size_t)(2, 3, 8, 512) == 2 * 3 * 8 * 514
+prefill = bind(mla, "dscuda_mla_prefill_backward_workspace_elements", [I] * 5, size_t)
+assert prefill(2, 65, 3, 192, 128) == 2 * 3 * (2 * 128 + 2 * 4096) and prefill(1, -4, 3, 192, 128) == 0
+backward = bind(flash, "dscuda_flash_backward_workspace_elements", [I] * 5, size_t)
+assert backward(1, 128, 4, 2, 64) > 0
+assert backward(1, 128, 4, 3, 64) == 0 and backward(1, 128, 4, 0, 64) == 0 and backward(1, 128, 4, 2, 96) == 0
+limit = bind(mla, "dscuda_mla_prefill_backward_set_workspace_limit", [size_t], None)
+limit(3 * 16384)                                                        # room for three dS blocks: one pair at a time
+assert prefill(2, 65, 3, 192, 128) == 2 * 3 * 2 * 128 + 2 * 4096
+limit(0)
+assert prefill(2, 65, 3, 192, 128) == 2 * 3 * (2 * 128 + 2 * 4096)
+bind(mla, "dscuda_mla_backward_set_key_interval_tiles", [I], None)(7)
+bind(flash, "dscuda_flash_backward_set_workspace_limit", [size_t], None)(0)
+print("size queries ok")
+"""
+    result = subprocess.run([sys.executable, "-c", script], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert result.returncode == 0 and "size queries ok" in result.stdout, result.stdout + result.stderr
+
+
 def _status_and_message(lib, prefix, status):
     with pytest.raises(RuntimeError) as info:
         checked(lib, prefix, status)

@@ -4,11 +4,6 @@ C-ABI.  As in the reference harness (benchmarks/mla.py:68,113-117) the
 backward is fed the oracle's own bf16-rounded O and fp32 LSE, so forward and
 backward are tested independently."""
 
-import os
-import subprocess
-import sys
-from pathlib import Path
-
 import pytest
 import torch
 
@@ -98,11 +93,15 @@ def test_backward_workload_3(cuda):
 def test_absorbed_backward(cuda, batch, tokens, heads):
     """Shapes of benchmarks/mla.py:34-45; dO = 0.2 * N(0,1) as at :108; saved O (bf16) and LSE
     come from the oracle forward as at :68,113-117."""
-    ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
-    g = torch.Generator().manual_seed(77)
     # dLatent sums over all heads: with 128 of them dO is scaled down so that the sums stay where half a bf16 ulp
     # (the rounding of the result itself) is below the tolerance
-    dout = (torch.randn(batch, tokens, heads, 512, generator=g) * (0.2 if heads <= 32 else 0.05)).bfloat16()
+    _absorbed_case(cuda, batch, tokens, heads, seed=77, dout_factor=0.2 if heads <= 32 else 0.05)
+
+
+def _absorbed_case(cuda, batch, tokens, heads, seed, dout_factor):
+    ql, qr, c, kr, scale = configs.mla_absorbed_inputs(batch, tokens, heads)
+    g = torch.Generator().manual_seed(seed)
+    dout = (torch.randn(batch, tokens, heads, 512, generator=g) * dout_factor).bfloat16()
     mask = oracle.causal_mask(tokens)
     out, lse = oracle.mla_forward(ql, qr, c, kr, scale, mask)
     announce("mla_backward", dict(B=batch, T=tokens, H=heads))
@@ -142,16 +141,21 @@ def test_absorbed_backward_closed_form_constant_fill(cuda):
     (1, 300, 3, 0.5, 1),      # a budget below one pair still runs, one pair at a time
 ])
 def test_backward_in_chunks_of_pairs(cuda, batch, seq, heads, budget_pairs, expected_chunk):
-    """The dS workspace is bounded: with a budget that holds only some (batch, head) pairs the two gradient passes run
+    """The dS workspace is bounded: with a limit that holds only some (batch, head) pairs the two gradient passes run
     chunk after chunk over one set of dS blocks, and the workspace the library asks for shrinks accordingly."""
     key_blocks, tiles = (seq + 127) // 128, (seq + 63) // 64
-    pair_bytes = sum(tiles - 2 * kb for kb in range(key_blocks)) * 16384
-    environment = dict(os.environ, DSCUDA_AMD_DS_BUDGET_BYTES=str(int(budget_pairs * pair_bytes)))
-    root = Path(__file__).resolve().parents[1]
-    result = subprocess.run([sys.executable, "-m", "tests.backward_chunk_case", str(batch), str(seq), str(heads),
-                             str(expected_chunk)], cwd=root, env=environment, capture_output=True, text=True, timeout=300)
-    assert result.returncode == 0, result.stdout[-2000:] + result.stderr[-4000:]
-    assert "chunked backward ok" in result.stdout
+    blocks = sum(tiles - 2 * kb for kb in range(key_blocks))
+    limit = int(budget_pairs * blocks * 16384)
+    ops.mla_prefill_backward_set_workspace_limit(limit)
+    try:
+        statistics = batch * heads * tiles * 128
+        elements = ops.mla_prefill_backward_workspace_elements(batch, seq, heads, 192, 128)
+        assert elements == statistics + expected_chunk * blocks * 4096, (elements, statistics, expected_chunk, blocks)
+        assert expected_chunk * blocks * 16384 <= limit or expected_chunk == 1
+        _backward_case(cuda, batch, seq, heads, 128, 64, 128, seed=31)
+    finally:
+        ops.mla_prefill_backward_set_workspace_limit(0)
+    assert ops.mla_prefill_backward_workspace_elements(batch, seq, heads, 192, 128) == statistics + batch * heads * blocks * 4096
 
 
 @pytest.mark.parametrize("batch,tokens,heads,interval_tiles", [
@@ -162,13 +166,12 @@ def test_backward_in_chunks_of_pairs(cuda, batch, seq, heads, budget_pairs, expe
 ])
 def test_absorbed_backward_interval_cut(cuda, batch, tokens, heads, interval_tiles):
     """The cut of the key gradients for inputs that outgrow the caches (items of one interval of row tiles and one
-    key block, dealt to the XCDs), forced at sizes the oracle can check."""
-    environment = dict(os.environ, DSCUDA_AMD_KEY_INTERVAL_TILES=str(interval_tiles))
-    root = Path(__file__).resolve().parents[1]
-    result = subprocess.run([sys.executable, "-m", "tests.absorbed_interval_case", str(batch), str(tokens), str(heads)],
-                            cwd=root, env=environment, capture_output=True, text=True, timeout=300)
-    assert result.returncode == 0, result.stdout[-2000:] + result.stderr[-4000:]
-    assert "interval cut ok" in result.stdout
+    key block), forced at sizes the oracle can check."""
+    ops.mla_backward_set_key_interval_tiles(interval_tiles)
+    try:
+        _absorbed_case(cuda, batch, tokens, heads, seed=78, dout_factor=0.2 if heads <= 32 else 0.05)
+    finally:
+        ops.mla_backward_set_key_interval_tiles(0)
 
 
 def test_backward_workspace_is_bounded(cuda):

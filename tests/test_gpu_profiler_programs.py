@@ -18,7 +18,6 @@ CASES = [
     ("benchmark_mla_prefill", (1, 1024, 8, 192, 128, "--operation", "both")),
     ("benchmark_flash_attention", (2, 256, 8, 128)),
     ("benchmark_flash_attention", (1, 512, 8, 64)),
-    ("hbm_read_probe", (64, 3)),
 ]
 
 

@@ -1,35 +1,32 @@
-"""The rotary-embedding kernel (dscuda_rope_apply) against the host formulation every workload of this repository
-is generated with (dscuda_amd/harness/configs.py apply_rope: interleaved pairs, fp64 angles, fp32 sine / cosine,
-unfused fp32 arithmetic): the same roundings in the same order, so the results are compared bit for bit apart from
-the rare element whose sine or cosine rounds differently on the device (at most one in ten thousand, off by one
-bf16 step, or by less than 1e-5 where the two products of a rotation cancel)."""
+"""The rotary-embedding kernel (dscuda_rope_apply) against the oracle's statement of the convention (complex
+multiplication in fp64, pinned by closed forms in tests/test_oracle_pins.py), rounded to bf16.  The kernel computes
+in fp32 (fp32 sine / cosine of an fp64-exact angle, unfused products), so its result differs from the correctly
+rounded one only where fp32 rounding moves a value across a bf16 rounding boundary: a small fraction of the
+elements, each off by one bf16 step, or by less than 1e-5 where the two products of a rotation cancel."""
 
 import pytest
 import torch
 
-from dscuda_amd.harness import configs, ops
+from dscuda_amd.harness import ops
+from oracle import attention_oracle as oracle
 from tests.parity import announce
 
 pytestmark = pytest.mark.gpu
 
 
 def _expected(x, offset, size, theta=10000.0, start=None):
-    out = x.float().clone()
-    batch, seq = x.shape[:2]
-    for b in range(batch):
+    out = x.double().clone()
+    for b in range(x.shape[0]):
         first = 0 if start is None else int(start[b])
-        # apply_rope rotates positions 0..S-1: a longer run is rotated and its tail taken for a start position
-        padded = torch.zeros(1, first + seq, x.shape[2], size)
-        padded[:, first:] = out[b:b + 1, :, :, offset:offset + size]
-        out[b:b + 1, :, :, offset:offset + size] = configs.apply_rope(padded, theta)[:, first:]
-    return out.bfloat16()
+        out[b:b + 1, :, :, offset:offset + size] = oracle.apply_rope(x[b:b + 1, :, :, offset:offset + size], theta, first)
+    return out.float().bfloat16()
 
 
 def _compare(got, expected):
     got, expected = got.cpu(), expected
     different = (got.view(torch.int16) != expected.view(torch.int16))
     fraction = different.float().mean().item()
-    assert fraction <= 1e-4, f"{fraction:.2e} of the elements differ"
+    assert fraction <= 3e-4, f"{fraction:.2e} of the elements differ"
     if different.any():
         # ... and then by one bf16 step, or by next to nothing in absolute terms where the two products cancel
         a, b = got[different].float(), expected[different].float()
@@ -44,7 +41,7 @@ def _compare(got, expected):
     ((2, 50, 5, 40), 8, 32),           # another width: 16 pairs, four groups of lanes
     ((1, 7, 2, 8), 2, 4),
 ])
-def test_rope_matches_the_host_formulation(cuda, shape, offset, size):
+def test_rope_matches_the_oracle(cuda, shape, offset, size):
     announce("rope", dict(shape=shape, offset=offset, size=size))
     g = torch.Generator().manual_seed(77)
     x = (torch.randn(shape, generator=g) * 0.5).bfloat16()

@@ -339,3 +339,81 @@ def test_projections_brute_force_and_absorption_identity():
     out_heads = torch.einsum("hts,shd->thd", p, v)
     out_absorbed = oracle.unabsorb_output(torch.einsum("hts,sc->thc", p, latent), w_uv)
     assert (out_heads - out_absorbed).abs().max() < 1e-9
+
+
+# ---- rotary embedding ----------------------------------------------------------------------------------------
+
+def _rope_variant(x, theta, pairing="interleaved", direction=1.0, exponent=2.0):
+    """Real-arithmetic RoPE with one knob per plausible mistake: how columns pair up, which way the pair turns,
+    and the frequency exponent."""
+    _, seq, _, width = x.shape
+    half = width // 2
+    frequency = theta ** (-exponent * torch.arange(half, dtype=torch.float64) / width)
+    angle = direction * torch.arange(seq, dtype=torch.float64)[:, None] * frequency[None]
+    cos, sin = angle.cos()[None, :, None], angle.sin()[None, :, None]
+    x = x.double()
+    out = torch.empty_like(x)
+    if pairing == "interleaved":
+        a, b = x[..., 0::2], x[..., 1::2]
+        out[..., 0::2], out[..., 1::2] = a * cos - b * sin, a * sin + b * cos
+    else:   # first half with second half
+        a, b = x[..., :half], x[..., half:]
+        out[..., :half], out[..., half:] = a * cos - b * sin, a * sin + b * cos
+    return out
+
+
+def test_rope_closed_forms():
+    theta, width, seq = 10000.0, 64, 300
+    # (1, 0) in every pair at position p -> (cos, sin) of p * theta^(-2i/R), written out with math.cos / math.sin
+    unit = torch.zeros(1, seq, 1, width)
+    unit[..., 0::2] = 1.0
+    rotated = oracle.apply_rope(unit, theta)
+    for p in (0, 1, 7, 299):
+        for i in (0, 1, 5, 31):
+            angle = p * theta ** (-2.0 * i / width)
+            assert abs(rotated[0, p, 0, 2 * i].item() - math.cos(angle)) < 1e-12
+            assert abs(rotated[0, p, 0, 2 * i + 1].item() - math.sin(angle)) < 1e-12
+    # (0, 1) -> (-sin, cos): the pair turns counter-clockwise
+    unit = torch.zeros(1, seq, 1, width)
+    unit[..., 1::2] = 1.0
+    rotated = oracle.apply_rope(unit, theta)
+    angle = 7 * theta ** (-2.0 * 5 / width)
+    assert abs(rotated[0, 7, 0, 10].item() + math.sin(angle)) < 1e-12 and abs(rotated[0, 7, 0, 11].item() - math.cos(angle)) < 1e-12
+    # position 0 is the identity; R = 2 leaves one pair turning by exactly p radians whatever theta is
+    x = torch.randn(2, 5, 3, width, generator=torch.Generator().manual_seed(5), dtype=torch.float64)
+    assert torch.equal(oracle.apply_rope(x, theta)[:, 0], x[:, 0])
+    pair = torch.tensor([0.3, -1.1], dtype=torch.float64).expand(1, 9, 1, 2)
+    for any_theta in (10000.0, 3.0):
+        turned = oracle.apply_rope(pair, any_theta)
+        for p in range(9):
+            assert abs(turned[0, p, 0, 0].item() - (0.3 * math.cos(p) + 1.1 * math.sin(p))) < 1e-12
+            assert abs(turned[0, p, 0, 1].item() - (0.3 * math.sin(p) - 1.1 * math.cos(p))) < 1e-12
+
+
+def test_rope_composes_and_depends_on_relative_position_only():
+    theta, width = 10000.0, 64
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(1, 40, 2, width, generator=g, dtype=torch.float64)
+    k = torch.randn(1, 40, 2, width, generator=g, dtype=torch.float64)
+    # start position s: the same as rotating a longer run and taking its tail
+    shifted = oracle.apply_rope(q, theta, start=11)
+    padded = torch.cat([torch.zeros(1, 11, 2, width, dtype=torch.float64), q], 1)
+    torch.testing.assert_close(shifted, oracle.apply_rope(padded, theta)[:, 11:], atol=1e-12, rtol=0)
+    # <rope(q, m), rope(k, n)> depends on m - n only
+    rq, rk = oracle.apply_rope(q, theta), oracle.apply_rope(k, theta)
+    rq5, rk5 = oracle.apply_rope(q, theta, start=5), oracle.apply_rope(k, theta, start=5)
+    torch.testing.assert_close(torch.einsum("bmhd,bnhd->bhmn", rq, rk), torch.einsum("bmhd,bnhd->bhmn", rq5, rk5),
+                               atol=1e-10, rtol=0)
+
+
+def test_rope_workload_formulation_matches_the_oracle_and_mistakes_do_not():
+    from dscuda_amd.harness import configs
+    theta, width = 10000.0, 64
+    x = torch.randn(2, 257, 3, width, generator=torch.Generator().manual_seed(7)) * 0.5
+    expected = oracle.apply_rope(x, theta)
+    # the formulation every workload is generated with (fp32 sine / cosine, fp32 products)
+    torch.testing.assert_close(configs.apply_rope(x, theta).double(), expected, atol=2e-6, rtol=0)
+    torch.testing.assert_close(_rope_variant(x, theta), expected, atol=1e-12, rtol=0)
+    # each plausible mistake is far outside that
+    for mistake in (dict(pairing="halves"), dict(direction=-1.0), dict(exponent=1.0)):
+        assert (_rope_variant(x, theta, **mistake) - expected).abs().max() > 0.1, mistake

@@ -63,3 +63,41 @@ def test_static_workspace_decode_rejects_sizes_beyond_its_capacity(cuda):
                           configs.c_float(192 ** -0.5), 3, out, lse)
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()
+
+
+def test_static_workspace_decode_allocates_nothing_and_replays_from_a_graph(cuda):
+    """Device memory in use is the same before and after warm calls (the driver's own count, which sees allocations
+    of any library in the process), and the call, captured into a graph after one eager call, replays bit-equal to
+    the workspace entry point on fresh buffer contents, with eager work between the replays."""
+    scale = configs.c_float(192 ** -0.5)
+    batch, tokens, heads, splits = 6, 1500, 128, 8
+    query, cache, paged, table, lengths = _inputs(batch, tokens, heads, 105)
+    static = [x.to(cuda) for x in (query, paged, table, lengths)]
+    out = torch.empty(batch, 1, heads, 512, device=cuda, dtype=torch.bfloat16)
+    lse = torch.empty(batch, heads, 1, device=cuda, dtype=torch.float32)
+    announce("mla_decode_static: no allocation", dict(B=batch, KV=tokens, H=heads, splits=splits))
+    ops.mla_decode_static(*static, scale, splits, out, lse)      # first call on the device: symbol address, attributes
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before = torch.cuda.memory_reserved()
+    for _ in range(3):
+        ops.mla_decode_static(*static, scale, splits, out, lse)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before and torch.cuda.memory_reserved() == reserved_before
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.mla_decode_static(*static, scale, splits, out, lse)
+    for seed in (106, 107):
+        fresh = _inputs(batch, tokens, heads, seed)
+        for target, source in zip(static, (fresh[0], fresh[2], fresh[3], fresh[4])):
+            target.copy_(source)
+        out.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed_out, replayed_lse = out.clone(), lse.clone()
+        expected_out, expected_lse = ops.mla_decode(*static, scale, splits=splits)    # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(replayed_out, expected_out) and torch.equal(replayed_lse, expected_lse)
