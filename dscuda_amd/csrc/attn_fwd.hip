@@ -377,6 +377,15 @@ struct PingPong {
     static constexpr int V_SLOTS = 4;
     static constexpr int RING = 8;
     static constexpr int CLUSTERS = 8;
+    // Output rows leave through LDS, half a row (64 columns, one 128-byte line) at a time: 32 rows of
+    // 128 + 16 bytes per wave, for the four waves of one group (the two groups store in different phases).
+    static constexpr int O_HALF_COLUMNS = 64;
+    static constexpr int O_PITCH = O_HALF_COLUMNS * 2 + 16;
+    static constexpr int O_WAVE_BYTES = 32 * O_PITCH;
+    static constexpr int O_BYTES = 4 * O_WAVE_BYTES;
+    // Where the loads that only warm the cache for the next item's queries put their data: 256 bytes per wave.
+    static constexpr int WARM_BYTES = 8 * 256;
+    static constexpr int EXTRA_BYTES = O_BYTES + WARM_BYTES;
 };
 
 using index_math::forward_item;
@@ -395,6 +404,9 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
     constexpr int SPAN = (C::K_ROW % 256 == 0) ? 16 : 8;   // chunk positions the K swizzle permutes
     constexpr int KLOW = SPAN / 2;                          // k-steps with distinct swizzled addresses
     constexpr int V_RING = PingPong::K_SLOTS * C::K_BYTES;  // byte offset of the V slots
+    constexpr int O_STAGE = V_RING + PingPong::V_SLOTS * C::V_BYTES;   // byte offset of the output staging rows
+    constexpr int WARM_AT = O_STAGE + PingPong::O_BYTES;
+    static_assert(DV % PingPong::O_HALF_COLUMNS == 0, "output rows leave in halves of 64 columns");
     constexpr int RING = PingPong::RING;
     constexpr int PV_MFMAS = 4 * DBLOCKS;
     constexpr int QK_MFMAS = 2 * KSTEPS;
@@ -523,6 +535,22 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
             }
             qf[ks] = __builtin_bit_cast(bf16x8, bits);
         }
+    };
+
+    // The query rows of an item are read once, from memory, and a wave cannot ask for them before its registers
+    // are free, one phase before it needs them.  One tile earlier it therefore touches every 128-byte line of
+    // those rows with loads whose data nobody reads (they land in a scratch line of LDS), so that the real loads
+    // find the lines in the L2.  Two instructions: lines 0 and 1 of the lane's row, then line 2.
+    auto warm_queries = [&](const ForwardItem& next) {
+        const int fresh = fresh_lane_id();
+        const int row_index = min(next.query_block * C::BM + 32 * wave + fresh % 32, S - 1);
+        const int b = next.batch_head / query_heads;
+        const int h = next.batch_head % query_heads;
+        const unsigned char* row = reinterpret_cast<const unsigned char*>(
+            query + ((size_t)b * S * query_heads + h) * DQK + (size_t)row_index * q_stride);
+        const unsigned scratch = lds_base + WARM_AT + wave * 256;
+        direct_load_4(row + 128 * (fresh / 32), scratch);
+        direct_load_4(row + (DQK * 2 > 256 ? 256 : 128 * (fresh / 32)), scratch);
     };
 
     ForwardItem item, next_item;
@@ -655,8 +683,9 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
         };
         // Y(tile): O += V^T P, and with FULL the next S.  The first RING fragments
         // are read before the barrier that separates X from Y.
-        auto phase_y = [&](auto full_tag) {
+        auto phase_y = [&](auto full_tag, auto warming_tag) {
             constexpr bool FULL = decltype(full_tag)::value;
+            constexpr bool WARMING = decltype(warming_tag)::value;   // two warming loads follow this tile's requests
             constexpr int COUNT = FULL ? PV_MFMAS + QK_MFMAS : PV_MFMAS;
             const int k_slot1 = k_slot == 2 ? 0 : k_slot + 1;
             const unsigned char* k_tile = lds + k_slot1 * C::K_BYTES;           // K(tile + 1)
@@ -682,49 +711,74 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_setprio(0);
-            wait_vector_memory<0>();   // this wave's requests of X(tile)
+            wait_vector_memory<WARMING ? 2 : 0>();   // this wave's requests of X(tile); warming loads may take their time
             workgroup_barrier();
             k_slot = k_slot1;
             v_slot = (v_slot + 1) & 3;
         };
 
-        for (int tile = 0; tile + 1 < tiles; ++tile) {
+        for (int tile = 0; tile + 2 < tiles; ++tile) {
             phase_x(tile);
-            phase_y(std::true_type{});
+            phase_y(std::true_type{}, std::false_type{});
         }
-        // Last tile: the query registers are free from here on, the next item's
-        // queries load while this tile finishes.
-        phase_x(tiles - 1);
-        const float total = half_wave_sum(row_sum);
-        const float lse_value = row_max * scale + __logf(total);
-        const int store_row = q_row;
-        const int store_batch_head = item.batch_head;
+        // The tile before the last (kept apart from the loop, whose instructions stay what they are): behind its
+        // requests go the loads that warm the cache for the next item's queries.
+        phase_x(tiles - 2);
+        warm_queries(has_next ? next_item : item);
+        phase_y(std::true_type{}, std::true_type{});
+        // Last tile: its scores exist already, so the query registers are free: the next item's queries load
+        // while this tile finishes.
         if (has_next) {
             load_queries(next_item);
         }
-        phase_y(std::false_type{});
+        phase_x(tiles - 1);
+        phase_y(std::false_type{}, std::false_type{});
 
-        // ---- epilogue: normalise and store straight from the accumulators.  A
-        // lane holds 4 consecutive d_v of one query per (d, i4): 8-byte stores.
+        // ---- epilogue: normalise, round, and store rows and logsumexp.  A lane holds, per column block, four
+        // runs of four columns of one query; the rows go through this wave's staging rows in LDS, 64 columns
+        // at a time, so that every store instruction writes eight whole 128-byte lines.  Only this wave touches
+        // its staging rows; the two groups come through here in different phases and share them.
         {
+            const int fresh = fresh_lane_id();   // nothing of the address arithmetic below is carried through the tile loop
+            const int row = fresh % 32;
+            const int half_wave = fresh / 32;
+            const float total = half_wave_sum(row_sum);
             const float inverse = 1.0f / total;
-            const int b = store_batch_head / query_heads;
-            const int h = store_batch_head % query_heads;
-            if (store_row < S) {
-                if (g == 0) {
-                    logsumexp[((size_t)b * query_heads + h) * S + store_row] = lse_value;
-                }
-                bf16_t* o_row = output + ((size_t)b * S * query_heads + h) * DV + (size_t)store_row * o_stride;
+            const int b = item.batch_head / query_heads;
+            const int h = item.batch_head % query_heads;
+            if (half_wave == 0 && wave_q0 + row < S) {
+                logsumexp[((size_t)b * query_heads + h) * S + wave_q0 + row] = row_max * scale + __logf(total);
+            }
+            bf16_t* o_head = output + ((size_t)b * S * query_heads + h) * DV;
+            unsigned char* o_lds = lds + O_STAGE + (wave % 4) * PingPong::O_WAVE_BYTES;
+            constexpr int HALVES = DV / PingPong::O_HALF_COLUMNS;
+            constexpr int HALF_BLOCKS = PingPong::O_HALF_COLUMNS / 32;
 #pragma unroll
-                for (int d = 0; d < DBLOCKS; ++d) {
+            for (int half = 0; half < HALVES; ++half) {
+#pragma unroll
+                for (int db = 0; db < HALF_BLOCKS; ++db) {
+                    const int d = half * HALF_BLOCKS + db;
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
                         u32x2 packed;
                         packed.x = pack_bf16(o_acc[d][4 * i4 + 0] * inverse, o_acc[d][4 * i4 + 1] * inverse);
                         packed.y = pack_bf16(o_acc[d][4 * i4 + 2] * inverse, o_acc[d][4 * i4 + 3] * inverse);
-                        *reinterpret_cast<u32x2*>(o_row + 32 * d + 8 * i4 + 4 * g) = packed;
+                        *reinterpret_cast<u32x2*>(o_lds + row * PingPong::O_PITCH + 2 * (32 * db + 8 * i4 + 4 * half_wave)) = packed;
                     }
                 }
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
+                __builtin_amdgcn_wave_barrier();
+                // 32 rows x 128 bytes: eight lanes per row, eight rows per pass
+#pragma unroll
+                for (int pass = 0; pass < 4; ++pass) {
+                    const int r = 8 * pass + fresh / 8;
+                    const u32x4 bits = *reinterpret_cast<const u32x4*>(o_lds + r * PingPong::O_PITCH + 16 * (fresh % 8));
+                    if (wave_q0 + r < S) {
+                        *reinterpret_cast<u32x4*>(o_head + (size_t)(wave_q0 + r) * o_stride +
+                                                  half * PingPong::O_HALF_COLUMNS + 8 * (fresh % 8)) = bits;
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();   // the reads above precede the next half's writes
             }
         }
         if (!has_next) {
@@ -772,8 +826,8 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
                              const bf16_t* value, int batch_size, int sequence_length, int query_heads,
                              int key_value_heads, float scale, hipStream_t stream) {
     using C = FwdConfig<DQK, DV, 8>;
-    constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES;
-    static_assert(LDS_BYTES <= 160 * 1024, "the tile slots must fit the LDS");
+    constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES + PingPong::EXTRA_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "the tile slots, the output staging rows and the warming scratch must fit the LDS");
     const int query_blocks = (sequence_length + C::BM - 1) / C::BM;
     const long long batch_heads = (long long)batch_size * query_heads;
     if (batch_heads * query_blocks > 0x7fffffffLL) {
