@@ -383,9 +383,6 @@ struct PingPong {
     static constexpr int O_PITCH = O_HALF_COLUMNS * 2 + 16;
     static constexpr int O_WAVE_BYTES = 32 * O_PITCH;
     static constexpr int O_BYTES = 4 * O_WAVE_BYTES;
-    // Where the loads that only warm the cache for the next item's queries put their data: 256 bytes per wave.
-    static constexpr int WARM_BYTES = 8 * 256;
-    static constexpr int EXTRA_BYTES = O_BYTES + WARM_BYTES;
 };
 
 using index_math::forward_item;
@@ -405,7 +402,6 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
     constexpr int KLOW = SPAN / 2;                          // k-steps with distinct swizzled addresses
     constexpr int V_RING = PingPong::K_SLOTS * C::K_BYTES;  // byte offset of the V slots
     constexpr int O_STAGE = V_RING + PingPong::V_SLOTS * C::V_BYTES;   // byte offset of the output staging rows
-    constexpr int WARM_AT = O_STAGE + PingPong::O_BYTES;
     static_assert(DV % PingPong::O_HALF_COLUMNS == 0, "output rows leave in halves of 64 columns");
     constexpr int RING = PingPong::RING;
     constexpr int PV_MFMAS = 4 * DBLOCKS;
@@ -535,22 +531,6 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
             }
             qf[ks] = __builtin_bit_cast(bf16x8, bits);
         }
-    };
-
-    // The query rows of an item are read once, from memory, and a wave cannot ask for them before its registers
-    // are free, one phase before it needs them.  One tile earlier it therefore touches every 128-byte line of
-    // those rows with loads whose data nobody reads (they land in a scratch line of LDS), so that the real loads
-    // find the lines in the L2.  Two instructions: lines 0 and 1 of the lane's row, then line 2.
-    auto warm_queries = [&](const ForwardItem& next) {
-        const int fresh = fresh_lane_id();
-        const int row_index = min(next.query_block * C::BM + 32 * wave + fresh % 32, S - 1);
-        const int b = next.batch_head / query_heads;
-        const int h = next.batch_head % query_heads;
-        const unsigned char* row = reinterpret_cast<const unsigned char*>(
-            query + ((size_t)b * S * query_heads + h) * DQK + (size_t)row_index * q_stride);
-        const unsigned scratch = lds_base + WARM_AT + wave * 256;
-        direct_load_4(row + 128 * (fresh / 32), scratch);
-        direct_load_4(row + (DQK * 2 > 256 ? 256 : 128 * (fresh / 32)), scratch);
     };
 
     ForwardItem item, next_item;
@@ -683,9 +663,8 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
         };
         // Y(tile): O += V^T P, and with FULL the next S.  The first RING fragments
         // are read before the barrier that separates X from Y.
-        auto phase_y = [&](auto full_tag, auto warming_tag) {
+        auto phase_y = [&](auto full_tag) {
             constexpr bool FULL = decltype(full_tag)::value;
-            constexpr bool WARMING = decltype(warming_tag)::value;   // two warming loads follow this tile's requests
             constexpr int COUNT = FULL ? PV_MFMAS + QK_MFMAS : PV_MFMAS;
             const int k_slot1 = k_slot == 2 ? 0 : k_slot + 1;
             const unsigned char* k_tile = lds + k_slot1 * C::K_BYTES;           // K(tile + 1)
@@ -711,28 +690,23 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_setprio(0);
-            wait_vector_memory<WARMING ? 2 : 0>();   // this wave's requests of X(tile); warming loads may take their time
+            wait_vector_memory<0>();   // this wave's requests of X(tile)
             workgroup_barrier();
             k_slot = k_slot1;
             v_slot = (v_slot + 1) & 3;
         };
 
-        for (int tile = 0; tile + 2 < tiles; ++tile) {
+        for (int tile = 0; tile + 1 < tiles; ++tile) {
             phase_x(tile);
-            phase_y(std::true_type{}, std::false_type{});
+            phase_y(std::true_type{});
         }
-        // The tile before the last (kept apart from the loop, whose instructions stay what they are): behind its
-        // requests go the loads that warm the cache for the next item's queries.
-        phase_x(tiles - 2);
-        warm_queries(has_next ? next_item : item);
-        phase_y(std::true_type{}, std::true_type{});
         // Last tile: its scores exist already, so the query registers are free: the next item's queries load
         // while this tile finishes.
         if (has_next) {
             load_queries(next_item);
         }
         phase_x(tiles - 1);
-        phase_y(std::false_type{}, std::false_type{});
+        phase_y(std::false_type{});
 
         // ---- epilogue: normalise, round, and store rows and logsumexp.  A lane holds, per column block, four
         // runs of four columns of one query; the rows go through this wave's staging rows in LDS, 64 columns
@@ -826,8 +800,8 @@ void launch_forward_pingpong(bf16_t* output, float* logsumexp, const bf16_t* que
                              const bf16_t* value, int batch_size, int sequence_length, int query_heads,
                              int key_value_heads, float scale, hipStream_t stream) {
     using C = FwdConfig<DQK, DV, 8>;
-    constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES + PingPong::EXTRA_BYTES;
-    static_assert(LDS_BYTES <= 160 * 1024, "the tile slots, the output staging rows and the warming scratch must fit the LDS");
+    constexpr int LDS_BYTES = PingPong::K_SLOTS * C::K_BYTES + PingPong::V_SLOTS * C::V_BYTES + PingPong::O_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "the tile slots and the output staging rows must fit the LDS");
     const int query_blocks = (sequence_length + C::BM - 1) / C::BM;
     const long long batch_heads = (long long)batch_size * query_heads;
     if (batch_heads * query_blocks > 0x7fffffffLL) {

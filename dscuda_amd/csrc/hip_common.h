@@ -159,15 +159,6 @@ __device__ __forceinline__ void direct_load_16(const void* source, unsigned lds_
                  : "memory", "m0");
 }
 
-// Four bytes per lane (256 bytes of LDS per wave instruction): used where only the side effect matters, the
-// cache line a later load will find closer than memory.
-__device__ __forceinline__ void direct_load_4(const void* source, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
-                 :
-                 : "v"(source), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
-}
-
 // source = uniform 64-bit base + per-lane 32-bit byte offset; lds_base wave-uniform
 __device__ __forceinline__ void direct_load_16_offset(const void* uniform_base, unsigned byte_offset, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
