@@ -696,6 +696,7 @@ struct QueryGradConfig {
     static constexpr int D_BLOCKS = DQK / 64;            // 32-column blocks per wave
     static_assert(LDS_BYTES <= 160 * 1024, "stages must fit the LDS");
     static_assert(4 * D_BLOCKS * 2 * 16 * 64 * 4 <= LDS_BYTES, "the final sums must fit the LDS");
+    static_assert(2 * QTILE * (2 * DQK + 16) <= LDS_BYTES, "the staged gradient rows must fit the LDS");
 };
 
 // dQ^T (d x queries) = sum over keys of K^T (d x keys) dS^T (keys x queries).
@@ -877,38 +878,55 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
             }
         }
         __syncthreads();
-        if (key_half == 1) {
-            return;
-        }
+        if (key_half == 0) {
 #pragma unroll
-        for (int d = 0; d < C::D_BLOCKS; ++d) {
+            for (int d = 0; d < C::D_BLOCKS; ++d) {
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
+                for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) dq_acc[d][qb][i] += area[((d * 2 + qb) * 16 + i) * 64];
+                    for (int i = 0; i < 16; ++i) dq_acc[d][qb][i] += area[((d * 2 + qb) * 16 + i) * 64];
+                }
             }
         }
     }
 
-    // ---- epilogue: lane holds query lq and columns 32*block + 8*(i/4) + 4*g + i%4
-    if (2 * jb + tile_of_wave < query_tiles) {
+    // ---- epilogue.  A lane holds query lq and columns 32*block + 8*(i/4) + 4*g + i%4 of its wave's column
+    // blocks: stored from there, every instruction would touch 32 rows with 8 bytes each.  The rows are put
+    // together in LDS instead (both column halves of a query tile side by side) and leave as whole rows,
+    // 24 lanes of 16 bytes per row.
+    __syncthreads();   // every wave has taken its sums out of the area the rows are staged in
+    constexpr int ROW_PITCH = 2 * DQK + 16;
+    if (key_half == 0) {
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+            unsigned char* row = lds + (size_t)(tile_of_wave * QTILE + 32 * qb + lq) * ROW_PITCH;
+#pragma unroll
+            for (int d = 0; d < C::D_BLOCKS; ++d) {
+                const int column0 = 32 * (2 * d + column_half);
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    u32x2 packed;
+                    packed.x = pack_bf16(dq_acc[d][qb][4 * i4 + 0] * scale, dq_acc[d][qb][4 * i4 + 1] * scale);
+                    packed.y = pack_bf16(dq_acc[d][qb][4 * i4 + 2] * scale, dq_acc[d][qb][4 * i4 + 3] * scale);
+                    *reinterpret_cast<u32x2*>(row + 2 * (column0 + 8 * i4 + 4 * g)) = packed;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    {
+        constexpr int ROW_CHUNKS = DQK / 8;                      // 16-byte pieces of a row
+        constexpr int PIECES = 2 * QTILE * ROW_CHUNKS;           // of the workgroup's two query tiles
         bf16_t* dq_base = query_gradient + ((size_t)b * S * heads + h) * DQK;
         const size_t q_stride = (size_t)heads * DQK;
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-            const int q_row = (2 * jb + tile_of_wave) * QTILE + 32 * qb + lq;
+        for (int piece = tid; piece < PIECES; piece += DQ_THREADS) {
+            const int r = piece / ROW_CHUNKS;                    // row of the staged 128
+            const int chunk = piece % ROW_CHUNKS;
+            const int q_row = 2 * jb * QTILE + r;
             if (q_row < S) {
-#pragma unroll
-                for (int d = 0; d < C::D_BLOCKS; ++d) {
-                    const int column0 = 32 * (2 * d + column_half);
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) {
-                        u32x2 packed;
-                        packed.x = pack_bf16(dq_acc[d][qb][4 * i4 + 0] * scale, dq_acc[d][qb][4 * i4 + 1] * scale);
-                        packed.y = pack_bf16(dq_acc[d][qb][4 * i4 + 2] * scale, dq_acc[d][qb][4 * i4 + 3] * scale);
-                        *reinterpret_cast<u32x2*>(dq_base + (size_t)q_row * q_stride + column0 + 8 * i4 + 4 * g) = packed;
-                    }
-                }
+                const u32x4 bits = *reinterpret_cast<const u32x4*>(lds + (size_t)r * ROW_PITCH + 16 * chunk);
+                *reinterpret_cast<u32x4*>(dq_base + (size_t)q_row * q_stride + 8 * chunk) = bits;
             }
         }
     }
