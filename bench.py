@@ -42,7 +42,7 @@ def profiled_figures(stem, kernel_prefix):
         line = line.strip()
         if line.startswith(kernel_prefix) and " :: " in line:
             fields = dict(part.strip().split(" = ") for part in line.split(" :: ", 1)[1].split(" ; "))
-            nbytes = float(fields["hbm_bytes"])
+            nbytes = float(fields.get("fabric_bytes", fields.get("hbm_bytes", "nan")))
             return (None if nbytes != nbytes else nbytes), float(fields["time_us"])
     return None, None
 
@@ -203,7 +203,7 @@ def main():
                                "0.5*N(0,1) seed 1, RoPE theta=10000, scale 1/sqrt(192)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic,
-                     "traffic_source": "profiles/mla_prefill_forward_S4096_H128.md (rocprofv3 FETCH_SIZE + WRITE_SIZE)",
+                     "traffic_source": "profiles/mla_prefill_forward_S4096_H128.md (rocprofv3 FETCH_SIZE + WRITE_SIZE: bytes between the L2s and the fabric, an upper bound of the HBM bytes since the Infinity Cache serves part of them)",
                      "kernel": "attention_forward_pingpong_kernel<192,128>", "kernel_ms": kernel_ms,
                      "profiled_kernel_ms": None if profiled_us is None else profiled_us / 1000.0,
                      "flops_per_launch": flops},

@@ -61,14 +61,14 @@ def measure(device, event_time_ms, q, k, v, scale, out, lse, steps=40, warmup=15
     lv, ldo = draw((1, long_seq, heads, dv), 0.5), draw((1, long_seq, heads, dv), 1.0)
     lout = torch.empty(1, long_seq, heads, dv, device=device, dtype=torch.bfloat16)
     llse = torch.empty(1, heads, long_seq, device=device, dtype=torch.float32)
-    ms, _ = event_time_ms(lambda: ops.mla_prefill_forward(lq, lk, lv, scale, lout, llse), 3, 1)
+    ms, _ = event_time_ms(lambda: ops.mla_prefill_forward(lq, lk, lv, scale, lout, llse), 12, 3)
     flops = configs.forward_flops(1, heads, long_seq, dqk, dv)
     results["mla_forward_S16384_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
                                           "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,
                                           "data": "synthetic, GPU generator"}
     grads = (torch.empty_like(lq), torch.empty_like(lk), torch.empty_like(lv))
     workspace = ops.mla_prefill_backward_workspace(1, long_seq, heads, dqk, dv, device)
-    ms, _ = event_time_ms(lambda: ops.mla_prefill_backward(ldo, lout, llse, lq, lk, lv, scale, workspace, grads), 3, 1)
+    ms, _ = event_time_ms(lambda: ops.mla_prefill_backward(ldo, lout, llse, lq, lk, lv, scale, workspace, grads), 10, 2)
     flops = configs.backward_flops(1, heads, long_seq, dqk, dv)
     results["mla_backward_S16384_H128"] = {"ms": ms, "tflops": flops / ms / 1e9,
                                            "frac_of_bf16_peak": flops / ms / 1e9 / PEAK_BF16_TFLOPS, "flops": flops,

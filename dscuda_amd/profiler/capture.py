@@ -6,22 +6,32 @@ and ``scripts/extract_ncu.py`` (the per-kernel duration / DRAM traffic /
 throughput / registers / spills table, ``extract_ncu.py:193-326``), on rocprofv3:
 
     python -m dscuda_amd.profiler.capture {metric|mla|flash_attention} [quick|full] [profile|extract]
-        [--out DIR] [--profiles DIR] [--only STEM] [--passes time,fetch,write,mfma[,waits]]
+        [--out DIR] [--profiles DIR] [--only STEM] [--passes time,fetch,write,mfma,cache,waits,lds]
+        [--no-gate] [--commit HASH]
 
-``profile`` runs every case of the family once per pass, each pass a rocprofv3
-process of its own (a kernel trace, or one ``--pmc`` group that fits the
-hardware's counter blocks), raw CSV under ``--out``; then extracts.  ``extract``
-only rebuilds the tables from raw output that is already there.  The tables go
-to ``--profiles`` as one ``<stem>.md`` per case plus ``capture_<family>.md``.
+``profile`` first runs the family's GPU correctness tests (the reference gates
+its captures on its tests the same way, ``scripts/profile.sh:109-113``;
+``--no-gate`` skips that), then runs every case of the family once per pass,
+each pass a rocprofv3 process of its own (a kernel trace, or one ``--pmc``
+group that fits the hardware's counter blocks), raw CSV under ``--out``; then
+extracts.  ``extract`` only rebuilds the tables from raw output that is already
+there.  The tables go to ``--profiles`` as one ``<stem>.md`` per case plus
+``capture_<family>.md`` and ``<family>_environment.md`` (GPU, ROCm, compiler,
+commit: the counterpart of ``scripts/profile.sh:129-141``).
 
 What a row holds, per kernel of a case:
 
 * launches and duration: mean over the second half of the launches of the
   timing pass (the chip's clock needs some tens of back-to-back launches to
   settle, so the first launches are reported separately);
-* HBM bytes read / written per launch: ``FETCH_SIZE`` / ``WRITE_SIZE`` (KiB per
-  dispatch) times the factor the same counter shows for a plain device copy
-  of known size (the ``copy`` case of the metric family);
+* bytes the L2 caches fetched from / wrote to the fabric per launch:
+  ``FETCH_SIZE`` / ``WRITE_SIZE`` (KiB per dispatch) times the factor the same
+  counter shows for a plain device copy of known size (the ``copy`` case of
+  the metric family).  These are L2 misses and write-backs: the Infinity Cache
+  may serve them, so they bound the HBM bytes from above;
+* L2 hit rate ``TCC_HIT_sum / (TCC_HIT_sum + TCC_MISS_sum)`` (the reference's
+  table carries L1 / L2 hit rates, ``scripts/extract_ncu.py:227-231``) and the
+  read requests the L2s sent on (``TCC_EA0_RDREQ_sum``);
 * matrix-pipe utilisation ``SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / XCDS *
   SIMDS)`` and the shader clock ``GRBM_GUI_ACTIVE / XCDS / duration`` of the
   counter pass, LDS bank-conflict cycles;
@@ -61,8 +71,16 @@ PASSES = {
     "lds": ["--pmc", "SQ_INSTS_LDS_LOAD", "SQ_INSTS_LDS_LOAD_BANDWIDTH", "SQ_LDS_IDX_ACTIVE", "SQ_LDS_DATA_FIFO_FULL",
             "SQ_LDS_CMD_FIFO_FULL", "SQ_INST_LEVEL_LDS", "SQ_INSTS_MFMA", "SQ_BUSY_CYCLES"],
 }
-EXTRA_PASSES = ("waits", "lds")   # reported counter by counter below the table
-DEFAULT_PASSES = ("time", "fetch", "write", "mfma")
+PASSES["cache"] = ["--pmc", "TCC_HIT_sum", "TCC_MISS_sum", "TCC_EA0_RDREQ_sum"]
+EXTRA_PASSES = ("waits", "lds", "cache")   # reported counter by counter below the table; a failing one is skipped
+DEFAULT_PASSES = ("time", "fetch", "write", "mfma", "cache", "waits", "lds")
+
+# GPU correctness tests that must pass before a family is captured
+GATES = {
+    "metric": ["tests/test_gpu_forward.py", "tests/test_gpu_backward.py", "tests/test_gpu_decode.py"],
+    "mla": ["tests/test_gpu_decode.py", "tests/test_gpu_backward.py", "tests/test_gpu_profiler_programs.py"],
+    "flash_attention": ["tests/test_gpu_forward.py", "tests/test_gpu_profiler_programs.py"],
+}
 
 Case = collections.namedtuple("Case", "stem label command counter_command kernels")
 
@@ -151,7 +169,61 @@ def run_pass(case, pass_name, out, limit):
                             capture_output=True, text=True)
     (directory / "log.txt").write_text(result.stdout[-4000:] + "\n--- stderr ---\n" + result.stderr[-4000:])
     if result.returncode != 0:
-        raise RuntimeError(f"{case.stem}/{pass_name}: rocprofv3 exited with {result.returncode}; see {directory / 'log.txt'}")
+        message = f"{case.stem}/{pass_name}: rocprofv3 exited with {result.returncode}; see {directory / 'log.txt'}"
+        if pass_name in EXTRA_PASSES:
+            print(f"[capture] skipped: {message}", flush=True)   # a counter this rocprofv3 does not know
+            return
+        raise RuntimeError(message)
+
+
+def run_gate(family):
+    """The family's GPU tests, as the reference runs its own before a capture."""
+    command = [sys.executable, "-u", "-m", "pytest", *GATES[family], "-m", "gpu", "-x", "-q", "--timeout", "300",
+               "--timeout-method", "thread"]
+    print("[capture] gate: " + shlex.join(command), flush=True)
+    result = subprocess.run(command, cwd=ROOT, capture_output=True, text=True)
+    tail = (result.stdout + result.stderr).strip().splitlines()[-1:]
+    print("[capture] gate: " + " ".join(tail), flush=True)
+    if result.returncode != 0:
+        raise RuntimeError("the correctness gate failed; nothing was captured\n" + result.stdout[-3000:] + result.stderr[-2000:])
+
+
+def _first_line(command):
+    try:
+        result = subprocess.run(command, capture_output=True, text=True, timeout=60)
+    except (OSError, subprocess.TimeoutExpired):
+        return "unavailable"
+    lines = [line.strip() for line in (result.stdout + result.stderr).splitlines() if line.strip()]
+    return lines[0] if lines else "unavailable"
+
+
+def write_environment(family, suite, profiles, commit, gate):
+    """What the capture ran on: `<family>_environment.md`."""
+    gpu = "unavailable"
+    try:
+        result = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=60)
+        names = [line.split(":", 1)[1].strip() for line in result.stdout.splitlines() if "Marketing Name" in line]
+        chips = [line.split(":", 1)[1].strip() for line in result.stdout.splitlines() if line.strip().startswith("Name:") and "gfx" in line]
+        gpu = "; ".join(dict.fromkeys(name for name in names if "Instinct" in name or "MI" in name)) or "unavailable"
+        if chips:
+            gpu += " (" + ", ".join(dict.fromkeys(chips)) + ")"
+    except (OSError, subprocess.TimeoutExpired):
+        pass
+    version_file = Path("/opt/rocm/.info/version")
+    rocm = version_file.read_text().strip() if version_file.exists() else "unavailable"
+    hipcc = [line for line in [_first_line(["/opt/rocm/bin/hipcc", "--version"])]][0]
+    rocprof = _first_line(["rocprofv3", "--version"])
+    try:
+        import torch
+        framework = f"{torch.__version__} (HIP {torch.version.hip})"
+    except Exception:   # noqa: BLE001 -- the standalone programs need no PyTorch
+        framework = "unavailable"
+    lines = [f"# capture environment: family `{family}`, suite `{suite}`", "",
+             f"- GPU: {gpu}", f"- ROCm: {rocm}", f"- compiler: {hipcc}", f"- profiler: {rocprof}",
+             f"- PyTorch (device memory and streams of the Python cases): {framework}",
+             f"- commit: {commit or 'not given (--commit)'}",
+             f"- correctness gate before the capture: {gate}", ""]
+    (profiles / f"{family}_environment.md").write_text("\n".join(lines))
 
 
 # ---- extraction ---------------------------------------------------------------------------------------------
@@ -231,7 +303,8 @@ def extract_case(case, out, factors):
         durations = entry["durations"]
         row = {"kernel": kernel, "launches": len(durations), "first_us": mean(durations[:5]), "time_us": settled(durations),
                "vgpr": entry["vgpr"], "scratch": entry["scratch"], "lds": entry["lds"],
-               "read_mb": float("nan"), "write_mb": float("nan"), "mfma_pct": float("nan"), "clock_ghz": float("nan"),
+               "read_mb": float("nan"), "write_mb": float("nan"), "l2_hit_pct": float("nan"), "mfma_pct": float("nan"),
+               "clock_ghz": float("nan"),
                "bank_conflict": float("nan"), "counter_us": float("nan")}
         if kernel in fetch and "FETCH_SIZE" in fetch[kernel]:
             row["read_mb"] = settled(fetch[kernel]["FETCH_SIZE"]) * factors[0] * 1024 / 1e6
@@ -248,6 +321,11 @@ def extract_case(case, out, factors):
                     row["mfma_pct"] = 100.0 * settled(counters["SQ_VALU_MFMA_BUSY_CYCLES"]) / (cycles * SIMDS)
             if "SQ_LDS_BANK_CONFLICT" in counters:
                 row["bank_conflict"] = settled(counters["SQ_LDS_BANK_CONFLICT"])
+        cache, _ = read_counters(directory / "cache", case.kernels)
+        if kernel in cache and "TCC_HIT_sum" in cache[kernel] and "TCC_MISS_sum" in cache[kernel]:
+            hits, misses = settled(cache[kernel]["TCC_HIT_sum"]), settled(cache[kernel]["TCC_MISS_sum"])
+            if hits + misses > 0:
+                row["l2_hit_pct"] = 100.0 * hits / (hits + misses)
         row["more"] = collections.OrderedDict()
         for pass_name in EXTRA_PASSES:
             table, _ = read_counters(directory / pass_name, case.kernels)
@@ -258,8 +336,8 @@ def extract_case(case, out, factors):
 
 
 COLUMNS = [("kernel", "kernel", "{}"), ("launches", "launches", "{:d}"), ("first_us", "first 5 us", "{:.1f}"),
-           ("time_us", "settled us", "{:.1f}"), ("read_mb", "HBM read MB", "{:.1f}"), ("write_mb", "HBM write MB", "{:.1f}"),
-           ("mfma_pct", "MFMA busy %", "{:.1f}"), ("clock_ghz", "clock GHz", "{:.2f}"),
+           ("time_us", "settled us", "{:.1f}"), ("read_mb", "L2 fetch MB", "{:.1f}"), ("write_mb", "L2 write-back MB", "{:.1f}"),
+           ("l2_hit_pct", "L2 hit %", "{:.1f}"), ("mfma_pct", "MFMA busy %", "{:.1f}"), ("clock_ghz", "clock GHz", "{:.2f}"),
            ("counter_us", "us in counter pass", "{:.1f}"), ("bank_conflict", "LDS bank conflict cycles", "{:.0f}"),
            ("vgpr", "registers/lane", "{:d}"), ("scratch", "scratch B/lane", "{:d}"),
            ("lds", "static LDS B", "{:d}")]
@@ -308,7 +386,9 @@ def write_case(case, rows, out, profiles, factors):
         if recorded.exists():
             lines.append(f"- {pass_name}: `{portable(recorded.read_text().strip(), out)}`")
     lines += ["", f"Counter calibration from the 1 GiB copy: FETCH_SIZE x {factors[0]:.3f}, WRITE_SIZE x {factors[1]:.3f}.",
-              "Durations are the mean of the second half of the launches of the timing pass.", ""]
+              "Durations are the mean of the second half of the launches of the timing pass.",
+              "L2 fetch / write-back: what the L2 caches exchanged with the fabric (Infinity Cache or HBM behind it): an upper",
+              "bound of the HBM bytes.", ""]
     lines += markdown_table(rows)
     if any(row.get("more") for row in rows):
         lines += ["", "Further counters, mean per launch over the second half of the launches (summed over the chip as "
@@ -319,7 +399,7 @@ def write_case(case, rows, out, profiles, factors):
     lines += ["", "Machine-readable (bytes per launch from the two traffic columns, microseconds from the settled column):", ""]
     for row in rows:
         total = (row["read_mb"] + row["write_mb"]) * 1e6
-        lines.append(f"    {row['kernel']} :: time_us = {row['time_us']:.3f} ; hbm_bytes = "
+        lines.append(f"    {row['kernel']} :: time_us = {row['time_us']:.3f} ; fabric_bytes = "
                      f"{'nan' if total != total else format(total, '.0f')}")
     (profiles / f"{case.stem}.md").write_text("\n".join(lines) + "\n")
 
@@ -336,8 +416,8 @@ def write_overview(family, suite, cases, results, profiles):
         total = sum(row["time_us"] for row in rows)
         read = sum(row["read_mb"] for row in rows)
         wrote = sum(row["write_mb"] for row in rows)
-        lines += ["", f"total: {len(rows)} kernels, {total:.1f} us, HBM read {cell('{:.1f}', read)} MB, "
-                      f"written {cell('{:.1f}', wrote)} MB", ""]
+        lines += ["", f"total: {len(rows)} kernels, {total:.1f} us, L2 fetch {cell('{:.1f}', read)} MB, "
+                      f"write-back {cell('{:.1f}', wrote)} MB", ""]
     (profiles / f"capture_{family}.md").write_text("\n".join(lines) + "\n")
 
 
@@ -351,6 +431,8 @@ def main(argv=None):
     parser.add_argument("--only", action="append", default=[], help="case stems to run (default: all)")
     parser.add_argument("--passes", default=",".join(DEFAULT_PASSES))
     parser.add_argument("--limit", type=int, default=240, help="seconds before a pass is killed")
+    parser.add_argument("--no-gate", action="store_true", help="do not run the family's GPU tests before the capture")
+    parser.add_argument("--commit", default=os.environ.get("DSCUDA_AMD_COMMIT", ""), help="recorded in the environment file")
     args = parser.parse_args(argv)
 
     passes = [name for name in args.passes.split(",") if name]
@@ -361,7 +443,13 @@ def main(argv=None):
     if args.only:
         cases = [case for case in cases if case.stem in args.only or case.stem == "copy_1GiB"]
     out = args.out.resolve()
+    args.profiles.mkdir(parents=True, exist_ok=True)
     if args.mode == "profile":
+        gate = "skipped (--no-gate)"
+        if not args.no_gate:
+            run_gate(args.family)
+            gate = "passed: " + " ".join(GATES[args.family])
+        write_environment(args.family, args.suite, args.profiles, args.commit, gate)
         for case in cases:
             for name in passes:
                 run_pass(case, name, out, args.limit)

@@ -78,7 +78,7 @@ def test_extraction_on_synthetic_rocprof_output(tmp_path):
     assert abs(row["mfma_pct"] - 50.0) < 1e-6 and abs(row["clock_ghz"] - 2.0) < 1e-6
     assert (row["vgpr"], row["scratch"], row["lds"]) == (438, 0, 155648)   # VGPR_Count is in units of two
     text = (profiles / f"{stem}.md").read_text()
-    assert "attention_forward_pingpong_kernel<192, 128> :: time_us = 640.000 ; hbm_bytes = 1228800000" in text
+    assert "attention_forward_pingpong_kernel<192, 128> :: time_us = 640.000 ; fabric_bytes = 1228800000" in text
     assert (profiles / "capture_metric.md").is_file()
 
 
