@@ -407,7 +407,7 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
     constexpr int PV_MFMAS = 4 * DBLOCKS;
     constexpr int QK_MFMAS = 2 * KSTEPS;
     constexpr int REQUESTS = C::K_LOADS_PER_WAVE + C::V_LOADS_PER_WAVE;
-    static_assert(REQUESTS <= 6, "X has six places for tile requests");
+    static_assert(REQUESTS <= 5, "X issues five tile requests");
     static_assert(PV_MFMAS >= RING, "the fragments read ahead in X must all belong to V");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -592,7 +592,7 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
             }
         }
 
-        // X(tile): softmax with the requests for stream tile + 2 spread through it.
+        // X(tile): the requests for stream tile + 2, then the softmax.
         // A wave whose rows all lie before this tile runs it like any other: the
         // mask turns its scores into zeros, and the phases are barrier-locked, so
         // skipping would not end the tile sooner.  (Branching around the
@@ -611,7 +611,12 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                     request_part(request_k, request_v, request_key0, k_slot2, v_slot2, part);
                 }
             };
+            // all of this wave's requests first: they have the whole phase and the next to arrive
             request_next(0);
+            request_next(1);
+            request_next(2);
+            request_next(3);
+            request_next(4);
             if (key0 + BN - 1 > wave_q0) {  // tile reaches past this wave's first row
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) {
@@ -644,7 +649,6 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                     for (int i = 0; i < 16; ++i) o_acc[d][i] *= alpha;
                 }
             }
-            request_next(1);
             const float offset = row_max * c;
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
@@ -658,7 +662,6 @@ __global__ __launch_bounds__(512) void attention_forward_pingpong_kernel(
                     packed[j] = pack_bf16(p0, p1);
                 }
                 pf[n] = __builtin_bit_cast(bf16x8, packed);
-                request_next(2 + n);
             }
         };
         // Y(tile): O += V^T P, and with FULL the next S.  The first RING fragments

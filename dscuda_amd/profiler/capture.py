@@ -202,11 +202,17 @@ def write_environment(family, suite, profiles, commit, gate):
     gpu = "unavailable"
     try:
         result = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=60)
-        names = [line.split(":", 1)[1].strip() for line in result.stdout.splitlines() if "Marketing Name" in line]
-        chips = [line.split(":", 1)[1].strip() for line in result.stdout.splitlines() if line.strip().startswith("Name:") and "gfx" in line]
-        gpu = "; ".join(dict.fromkeys(name for name in names if "Instinct" in name or "MI" in name)) or "unavailable"
-        if chips:
-            gpu += " (" + ", ".join(dict.fromkeys(chips)) + ")"
+        # one block per agent: "Name:", "Marketing Name:", ..., "Device Type:"
+        found, name, marketing = [], "", ""
+        for line in result.stdout.splitlines():
+            text = line.strip()
+            if text.startswith("Name:"):
+                name = text.split(":", 1)[1].strip()
+            elif text.startswith("Marketing Name:"):
+                marketing = text.split(":", 1)[1].strip()
+            elif text.startswith("Device Type:") and "GPU" in text:
+                found.append(f"{marketing or 'unnamed'} ({name})")
+        gpu = "; ".join(dict.fromkeys(found)) or "unavailable"
     except (OSError, subprocess.TimeoutExpired):
         pass
     version_file = Path("/opt/rocm/.info/version")
