@@ -103,6 +103,10 @@ struct TileRequestMath {
 //                           of a 16-row step -- the order a C-layout register block
 //                           carries; block = TR*m + i lies TR*64*m bytes further
 //                           (transposed_constant)
+//   quadrant(i, lane)       for the 16x16x32 products: row lane%16, chunk (4i + lane/16) ^ f(row):
+//                           the operand whose contraction index is the tile column, 32 columns
+//                           per step; step s = TR*m + i lies TR*64*m bytes further, 16 rows down
+//                           16*ROW_BYTES (quadrant_constant; f repeats after 16 rows)
 template <int ROW_BYTES>
 struct TileReadMath {
     static constexpr int SPAN = (ROW_BYTES % 256 == 0) ? 16 : 8;
@@ -120,6 +124,13 @@ struct TileReadMath {
         const int low = 2 * ((lane / 16) % 2) + (s % 4) / 2;
         const int row = 4 * g + s / 4 + 8 * h;
         return row * ROW_BYTES + 16 * ((4 * i + low) ^ tile_swizzle<ROW_BYTES>(row)) + 8 * (s % 2);
+    }
+    DSCUDA_HOST_DEVICE static unsigned quadrant(int i, int lane) {
+        const int row = lane % 16;
+        return row * ROW_BYTES + 16 * ((4 * i + lane / 16) ^ tile_swizzle<ROW_BYTES>(row));
+    }
+    DSCUDA_HOST_DEVICE static constexpr int quadrant_constant(int row0, int s) {
+        return row0 * ROW_BYTES + (s / TR) * (TR * 64);
     }
     DSCUDA_HOST_DEVICE static constexpr int natural_constant(int row0, int ks) {
         return row0 * ROW_BYTES + (ks / NAT) * (NAT * 32);
@@ -321,6 +332,16 @@ DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int he
     cut.row_tiles = (int)(((long long)sequence_length * heads + 31) / 32);
     cut.intervals = (cut.row_tiles + length - 1) / length;
     return cut;
+}
+
+// Workgroups are handed to the chip's `clusters` L2 domains in turn (workgroup w runs in domain w % clusters), and
+// the ones resident at any time have neighbouring numbers.  To let the workgroups that share an L2 walk
+// neighbouring entries of a list of `count` entries, domain d takes the d-th of `clusters` contiguous stretches of
+// the list (lengths differ by at most one) and its workgroups, in launch order, the entries of that stretch in order.
+DSCUDA_HOST_DEVICE inline long long entry_of_workgroup(long long workgroup, long long count, int clusters) {
+    const long long domain = workgroup % clusters;
+    const long long stretch = count / clusters, longer = count % clusters;
+    return domain * stretch + (domain < longer ? domain : longer) + workgroup / clusters;
 }
 
 constexpr long long KEY_PARTIAL_BYTES = 32LL * 576 * 4;   // one slot: [32 keys][576] fp32

@@ -58,11 +58,16 @@ constexpr int ROPE = 64;
 constexpr int WIDTH = RANK + ROPE;
 constexpr int TILE = 32;
 constexpr int THREADS = 256;
+constexpr int L2_DOMAINS = 8;   // the chip's XCDs: workgroup w of a launch runs on XCD w % 8
 
+// A [32][D] LDS tile of bf16, row-major without padding: 16-byte chunk c of row r sits at position
+// c ^ tile_swizzle(r), which spreads both the 16-byte reads down a column and the transposing reads over the banks.
 template <int D>
 struct Tile32 {
-    static constexpr int PITCH = 2 * D + 16;                // row-major, rows 16 bytes apart modulo 256
-    static constexpr int BYTES = TILE * PITCH;
+    static constexpr int ROW = 2 * D;
+    static constexpr int BYTES = TILE * ROW;
+    using Read = index_math::TileReadMath<ROW>;
+    static constexpr int PARTS = Read::TR;   // per-lane address parts a fragment read chooses from
 };
 
 // One thread's share of a [32][D_PART] tile in registers: 16-byte pieces of rows.
@@ -98,40 +103,39 @@ __device__ __forceinline__ void place_tile(const TileShare<D_PART>& share, unsig
         const int piece = tid + p * THREADS;
         if (piece >= S::PIECES) break;
         const int row = piece / (D_PART / 8);
-        const int column = column0 + 8 * (piece % (D_PART / 8));
-        *reinterpret_cast<u32x4*>(tile + row * Tile32<D>::PITCH + 2 * column) = share.r[p];
+        const int chunk = column0 / 8 + piece % (D_PART / 8);
+        *reinterpret_cast<u32x4*>(tile + row * Tile32<D>::ROW +
+                                  16 * (chunk ^ index_math::tile_swizzle<Tile32<D>::ROW>(row))) = share.r[p];
     }
-}
-
-// Operand with the tile's column as the contraction index: row lane%32, k-step ks.
-template <int D>
-__device__ __forceinline__ bf16x8 natural_fragment(const unsigned char* tile, int row, int ks, int g) {
-    return *reinterpret_cast<const bf16x8*>(tile + row * Tile32<D>::PITCH + 32 * ks + 16 * g);
 }
 
 // Operand with the tile's row as the contraction index, through transposing reads (ds_read_b64_tr_b16): in a
 // block of 16 lanes, lane s points at row 4*g + s/4 (+8 for the second read), columns 4*(s%4)..+3 of the block's
-// 16 columns, and receives the four rows' values of column s.  The lane ends up with column lane%32 of the
-// 32-column block at `column0` and tile rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}, the order in which the
-// accumulators of the score products hold rows.
+// 16 columns, and receives the four rows' values of column s.  The lane ends up with column lane%32 of a
+// 32-column block and tile rows {16n + 4g .. +3, 16n + 8 + 4g .. +3}, the order in which the accumulators of the
+// score products hold rows.  `low` / `high`: the lane's addresses of the two reads inside the tile's first 16
+// rows (TransposedAt), `offset` what is the same for all lanes.
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4* transposing_read_pointer;
 
-template <int D>
-__device__ __forceinline__ int transposed_lane_offset(int lane) {
-    const int g = lane / 32;
-    const int s = lane % 16;
-    const int half = (lane / 16) % 2;
-    return (4 * g + s / 4) * Tile32<D>::PITCH + 32 * half + 8 * (s % 4);
-}
-
-template <int D>
-__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* tile, int lane_offset, int column0, int n) {
-    const unsigned char* at = tile + lane_offset + n * 16 * Tile32<D>::PITCH + 2 * column0;
-    const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)at);
-    const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(at + 8 * Tile32<D>::PITCH));
+__device__ __forceinline__ bf16x8 transposed_fragment(const unsigned char* tile, int low_at, int high_at, int offset) {
+    const s16x4 low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(tile + low_at + offset));
+    const s16x4 high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((transposing_read_pointer)(tile + high_at + offset));
     return __builtin_bit_cast(bf16x8, __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7));
 }
+
+// The lane's addresses for column block b: part b % PARTS, plus (b / PARTS) * 64 * PARTS bytes.
+template <int D>
+struct TransposedAt {
+    int low[Tile32<D>::PARTS], high[Tile32<D>::PARTS];
+    __device__ __forceinline__ TransposedAt(int lane, int extra_bytes) {
+#pragma unroll
+        for (int i = 0; i < Tile32<D>::PARTS; ++i) {
+            low[i] = (int)Tile32<D>::Read::transposed(0, i, lane) + extra_bytes;
+            high[i] = (int)Tile32<D>::Read::transposed(1, i, lane) + extra_bytes;
+        }
+    }
+};
 
 __device__ __forceinline__ void clear(f32x16& value) {
 #pragma unroll
@@ -188,10 +192,23 @@ __device__ __forceinline__ bf16x8 exchange_fragment(const unsigned char* exchang
     return __builtin_bit_cast(bf16x8, u32x4{low.x, low.y, high.x, high.y});
 }
 
-// Operand of the 16x16x32 products out of a row-major tile: row `row` (of the wave's 16), k-step s of 32 columns.
+// Operand of the 16x16x32 products out of a tile: row 16*half + lane%16, k-step s of 32 columns: part s % PARTS
+// of the lane's addresses, plus (s / PARTS) * 64 * PARTS bytes.
 template <int D>
-__device__ __forceinline__ bf16x8 quadrant_fragment(const unsigned char* tile, int row, int s, int quad) {
-    return *reinterpret_cast<const bf16x8*>(tile + row * Tile32<D>::PITCH + 64 * s + 16 * quad);
+struct QuadrantAt {
+    int at[Tile32<D>::PARTS];
+    __device__ __forceinline__ QuadrantAt(int lane, int half) {
+#pragma unroll
+        for (int i = 0; i < Tile32<D>::PARTS; ++i) {
+            at[i] = (int)Tile32<D>::Read::quadrant(i, lane) + half * 16 * Tile32<D>::ROW;
+        }
+    }
+};
+
+template <int S, int D>
+__device__ __forceinline__ bf16x8 quadrant_fragment(const unsigned char* tile, const QuadrantAt<D>& lane_at) {
+    constexpr int PARTS = Tile32<D>::PARTS;
+    return *reinterpret_cast<const bf16x8*>(tile + lane_at.at[S % PARTS] + (S / PARTS) * 64 * PARTS);
 }
 
 // The same operand straight from memory: 32 columns per step, latent part first, then the rope part.
@@ -242,7 +259,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_row_statistics_kernel(
 
 // What the gradient formulas need of one row besides its vectors.
 struct RowStatistics {
-    float lse2;    // lse * log2(e)
+    float lse;     // as loaded: whoever multiplies it (by log2(e)) waits for the load, so that is left to the user
     float delta;
     int token;     // -1: no such row, it sees no key
 };
@@ -255,7 +272,7 @@ __device__ __forceinline__ RowStatistics fetch_row_statistics(const float* delta
     if (row < rows) {
         const int token = (int)(row / heads);
         const int head = (int)(row % heads);
-        statistics.lse2 = lse_batch[(size_t)head * sequence_length + token] * LOG2E;
+        statistics.lse = lse_batch[(size_t)head * sequence_length + token];
         statistics.delta = delta[(batch_row0 + row) * DELTA_STRIDE];
         statistics.token = token;
     }
@@ -286,6 +303,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x;
+    __builtin_assume(tid >= 0 && tid < THREADS);   // lets the per-piece bounds of the tile shares fold away
     const int wave = tid / 64;
     const int lane = tid % 64;
     const int lq = lane % 32;
@@ -330,10 +348,17 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
     fetch_quadrant_operand(dof, output_gradient + own * RANK, nullptr, own_valid, quad);
     const RowStatistics statistics = fetch_row_statistics(delta_of_rows, logsumexp + (size_t)batch * heads * T,
                                                           batch_row0, own_row, rows, heads, T);
-    const float row_lse2 = statistics.lse2;
+    const float row_lse2 = statistics.lse * LOG2E;
     const float row_delta = statistics.delta;
     const int row_token = statistics.token;
-    const int transposed_at = transposed_lane_offset<WIDTH>(lane);
+    const QuadrantAt<WIDTH> key_rows(lane, key_half);
+    // the wave's column blocks of the key tile: wave + 4*J for J < 4 and, last, 16 + wave % 2 (for waves 2 and 3 a
+    // duplicate that is never stored) -- all of parity wave % 2, two blocks share 128 bytes of a row
+    using KeyRead = Tile32<WIDTH>::Read;
+    const int key_columns_low = (int)KeyRead::transposed(0, wave % 2, lane) + 128 * (wave / 2);
+    const int key_columns_high = (int)KeyRead::transposed(1, wave % 2, lane) + 128 * (wave / 2);
+    const int last_columns_low = (int)KeyRead::transposed(0, wave % 2, lane) + 128 * 8;
+    const int last_columns_high = (int)KeyRead::transposed(1, wave % 2, lane) + 128 * 8;
     unsigned char* exchange = lds + L::EXCHANGE;
     const long long row = row0 + lq;   // the row whose gradient this lane ends up with
     const bool valid = row < rows;
@@ -365,7 +390,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
         f32x4 s_acc = {0.f, 0.f, 0.f, 0.f}, dp_acc = {0.f, 0.f, 0.f, 0.f};
         bf16x8 ring[AHEAD];
         auto key_fragment = [&](auto tag) {
-            return quadrant_fragment<WIDTH>(keys, 16 * key_half + l16, decltype(tag)::value, quad);
+            return quadrant_fragment<decltype(tag)::value>(keys, key_rows);
         };
         fill_ring(ring, key_fragment);
         fragment_stream<Q_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
@@ -380,8 +405,12 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
         auto column_fragment = [&](auto tag) {
             constexpr int J = decltype(tag)::value / 2;
             constexpr int N = decltype(tag)::value % 2;
-            const int block = min(wave + 4 * J, BLOCKS - 1);   // the clamped duplicate is never stored
-            return transposed_fragment<WIDTH>(keys, transposed_at, 32 * block, N);
+            constexpr int ROWS_DOWN = N * 16 * Tile32<WIDTH>::ROW;
+            if constexpr (J < 4) {
+                return transposed_fragment(keys, key_columns_low, key_columns_high, ROWS_DOWN + 256 * J);
+            } else {
+                return transposed_fragment(keys, last_columns_low, last_columns_high, ROWS_DOWN);
+            }
         };
         fill_ring(ring, column_fragment);
 
@@ -432,12 +461,14 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
 // ---- key gradients -------------------------------------------------------------
 
 struct KeyGradLayout {
-    static constexpr int Q_ROWS = 0;                                  // [32 rows][576]
-    static constexpr int DO_ROWS = Q_ROWS + Tile32<WIDTH>::BYTES;     // [32 rows][512]
-    static constexpr int STATS = DO_ROWS + Tile32<RANK>::BYTES;
+    static constexpr int Q_LATENT = 0;                                   // [32 rows][512]
+    static constexpr int DO_ROWS = Q_LATENT + Tile32<RANK>::BYTES;       // [32 rows][512]
+    static constexpr int Q_ROPE = DO_ROWS + Tile32<RANK>::BYTES;         // [32 rows][64]
+    static constexpr int STATS = Q_ROPE + Tile32<ROPE>::BYTES;
     static constexpr int BUFFER_BYTES = STATS + 3 * TILE * 4;
-    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;                 // the tile being multiplied and the next one
-    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_BYTES;   // P and dS
+    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;                    // the tile in use and the one arriving
+    static constexpr int EXCHANGE_PAIR = 2 * EXCHANGE_BYTES;             // P and dS of one tile
+    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_PAIR;       // of the tile being scored and the one before
 };
 
 constexpr int PARTIAL_FLOATS = TILE * WIDTH;   // one slot of partial key gradients: [32 keys][576] fp32
@@ -446,22 +477,45 @@ static_assert(PARTIAL_FLOATS * 4 == index_math::KEY_PARTIAL_BYTES, "slot size");
 // `interval_length` > 0: workgroup w takes item w of the interval cut (index_math.h), slot w.  Otherwise `ranges` > 0:
 // workgroup w walks range w of the list of visits; 0: workgroup w walks all visits of key block w (numbered through
 // the batch elements) and writes the gradients itself.
-__global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
+//
+// The four waves have two roles.  Waves 0 and 1 form the scores of a row tile: each takes 16 rows against all
+// 32 keys (the keys as register operands, every row fragment read from LDS feeds both key halves), applies the
+// softmax gradient and leaves P and dS in an exchange tile.  Waves 2 and 3 hold the gradient sums, nine column
+// blocks each (eight latent, one rope), and multiply the exchange tiles of the row tile BEFORE into them while the
+// next scores are formed: the two roles load the matrix pipes of their SIMDs equally (68 products of 16x16x32
+// against 34 of 32x32x16) and run side by side, where one wave doing both in turn would leave its pipe idle
+// during every LDS round trip.
+//
+// The gradient waves keep the column fragments of that earlier tile in registers: while a step's products consume
+// them one by one, each is replaced by the same fragment of the tile being scored, for the next step.  So only one
+// tile is read from LDS at a time, the other buffer is free for the whole step, and the rows of the next tile go
+// straight from memory into it (global_load_lds, issued at the start of the step, awaited at its end): no registers,
+// no LDS write instructions and no separate phase for them, and a step has one barrier.
+//
+// The walk is compiled once per role (SCORES), the kernel branches into one of the two: the key operands of the
+// score waves and the sums and fragments of the gradient waves then share the register file.  Both roles pass the
+// same barriers in the same order.
+template <bool SCORES>
+__device__ __forceinline__ void key_gradient_walk(
     bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
     const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
     const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
     const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int batch_size, int sequence_length,
     int heads, int ranges, int interval_length, float scale) {
     using L = KeyGradLayout;
+    using Wide = Tile32<RANK>;             // the latent query rows and the dO rows
+    using Narrow = Tile32<ROPE>;           // the rope query rows
     constexpr int Q_STEPS = WIDTH / 32;    // 18
     constexpr int O_STEPS = RANK / 32;     // 16
     constexpr int AHEAD = 6;
+    constexpr int LATENT_BLOCKS = 8;       // per gradient wave
+    constexpr int PER_STEP = 2 * LATENT_BLOCKS + 1;   // column fragments per 16-row step of a gradient wave
+    constexpr int ROWS_PER_WAVE = TILE / 4;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* p_exchange = lds + L::EXCHANGE;
-    unsigned char* ds_exchange = p_exchange + EXCHANGE_BYTES;
 
     const int tid = threadIdx.x;
+    __builtin_assume(tid >= 0 && tid < THREADS);
     const int wave = tid / 64;
     const int lane = tid % 64;
     const int lq = lane % 32;
@@ -469,23 +523,38 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     const int T = sequence_length;
     const long long rows = (long long)T * heads;
     const float c = scale * LOG2E;
-    const int q_transposed_at = transposed_lane_offset<WIDTH>(lane);
-    const int do_transposed_at = transposed_lane_offset<RANK>(lane);
-    const int row_half = wave / 2;
-    const int key_half = wave % 2;
+    const int half = wave % 2;             // score waves: rows 16*half .. +15; gradient waves: column blocks 8*half .. +7, 16 + half
     const int l16 = lane % 16;
     const int quad = lane / 16;
+    const QuadrantAt<RANK> wide_quadrant(lane, half);
+    const QuadrantAt<ROPE> narrow_quadrant(lane, half);
+    const TransposedAt<RANK> wide_columns(lane, 512 * half);
+    const int rope_columns_low = (int)Narrow::Read::transposed(0, half, lane);
+    const int rope_columns_high = (int)Narrow::Read::transposed(1, half, lane);
+
+    // Requests: the wave brings rows 8*wave .. +7 of the two wide tiles (an instruction fills one row: lane l
+    // fetches the chunk that belongs at position l) and instruction `wave` of the narrow tile (eight rows of eight chunks).
+    const unsigned lds_base = lds_offset_of(lds);
+    unsigned wide_part[ROWS_PER_WAVE];
+#pragma unroll
+    for (int j = 0; j < ROWS_PER_WAVE; ++j) {
+        wide_part[j] = 16u * (unsigned)(lane ^ index_math::tile_swizzle<Wide::ROW>(ROWS_PER_WAVE * wave + j));
+    }
+    const int narrow_row = ROWS_PER_WAVE * wave + lane / 8;
+    const unsigned narrow_part = 16u * (unsigned)((lane % 8) ^ index_math::tile_swizzle<Narrow::ROW>(narrow_row));
 
     const index_math::KeyVisits visits = index_math::key_visits(T, heads);
     const long long per_batch = visits.per_batch();
     const long long total = per_batch * batch_size;
     long long position, range_end;
+    long long item = 0;
     if (interval_length > 0) {
         const index_math::KeyIntervals cut = index_math::key_intervals(T, heads, interval_length);
         const long long items = cut.items();
-        const int batch = (int)(blockIdx.x / items);
+        item = blockIdx.x;
+        const int batch = (int)(item / items);
         int interval, key_block;
-        cut.locate(blockIdx.x - batch * items, interval, key_block);
+        cut.locate(item - batch * items, interval, key_block);
         const int first = max(interval * interval_length, visits.first_tile(key_block));
         position = batch * per_batch + visits.before(key_block) + (first - visits.first_tile(key_block));
         range_end = position + (cut.end_of(interval) - first);
@@ -511,7 +580,6 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
         const bool whole = within == block_begin && segment_end == block_end;
 
         const int k0 = key_block * TILE;
-        const int key = k0 + lq;
         const long long batch_row0 = (long long)batch * rows;
         const bf16_t* ql = query_latent + batch_row0 * RANK;
         const bf16_t* qr = query_rope + batch_row0 * ROPE;
@@ -520,173 +588,227 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
         const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
         const float* lse_batch = logsumexp + (size_t)batch * heads * T;
 
-        // this wave's quadrant of the score tile: rows 16*row_half .. +15 x keys 16*key_half .. +15.  Its keys as
-        // B operands (column = key l16); the value operand is the latent part
-        bf16x8 kf[Q_STEPS];
-        {
-            const int own_key = k0 + 16 * key_half + l16;
-            const size_t k = own_key < T ? own_key : 0;
-            fetch_quadrant_operand(kf, latent + k * RANK, rope + k * ROPE, own_key < T, quad);
+        // score waves: the keys as B operands (column = key 16*kh + l16); the value operand is the latent part
+        bf16x8 kf[2][Q_STEPS];
+        if constexpr (SCORES) {
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                const int own_key = k0 + 16 * kh + l16;
+                const size_t k = own_key < T ? own_key : 0;
+                fetch_quadrant_operand(kf[kh], latent + k * RANK, rope + k * ROPE, own_key < T, quad);
+            }
         }
 
-        f32x16 latent_acc[4], rope_acc;   // column blocks 4*wave + j of the latent, block wave%2 of the rope part
+        // gradient waves: column blocks 8*half + j of the latent part, block half of the rope part; and the column
+        // fragments of the tile before the one in LDS (zero before the first: its products add nothing)
+        f32x16 latent_acc[LATENT_BLOCKS], rope_acc;
+        bf16x8 held[2 * PER_STEP];
+        if constexpr (!SCORES) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) clear(latent_acc[j]);
-        clear(rope_acc);
+            for (int j = 0; j < LATENT_BLOCKS; ++j) clear(latent_acc[j]);
+            clear(rope_acc);
+#pragma unroll
+            for (int f = 0; f < 2 * PER_STEP; ++f) held[f] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+        }
 
-        TileShare<RANK> q_share, do_share;
-        TileShare<ROPE> rope_share;
+        // Rows of a tile past the last row of the batch element repeat that row: their token is -1, which sees no
+        // key, so their P and dS are zero whatever the rows hold.
         RowStatistics statistics = {0.f, 0.f, -1};
-        auto fetch_rows = [&](int tile) {
+        auto request_rows = [&](int tile, int parity) {
             const long long row0 = (long long)tile * TILE;
-            const int valid_rows = (int)min(rows - row0, (long long)TILE);
-            fetch_tile(q_share, ql + row0 * RANK, valid_rows, tid);
-            fetch_tile(rope_share, qr + row0 * ROPE, valid_rows, tid);
-            fetch_tile(do_share, dout + row0 * RANK, valid_rows, tid);
+            const int last_valid = (int)min(rows - row0, (long long)TILE) - 1;
+            const unsigned buffer = lds_base + parity * L::BUFFER_BYTES;
+            const bf16_t* ql_tile = ql + row0 * RANK;
+            const bf16_t* do_tile = dout + row0 * RANK;
+#pragma unroll
+            for (int j = 0; j < ROWS_PER_WAVE; ++j) {
+                const int row = ROWS_PER_WAVE * wave + j;
+                const unsigned source = wide_part[j] + (unsigned)(min(row, last_valid) * Wide::ROW);
+                direct_load_16_offset(ql_tile, source, buffer + L::Q_LATENT + row * Wide::ROW);
+                direct_load_16_offset(do_tile, source, buffer + L::DO_ROWS + row * Wide::ROW);
+            }
+            direct_load_16_offset(qr + row0 * ROPE, narrow_part + (unsigned)(min(narrow_row, last_valid) * Narrow::ROW),
+                                  buffer + L::Q_ROPE + ROWS_PER_WAVE * wave * Narrow::ROW);
             if (tid < TILE) {
                 statistics = fetch_row_statistics(delta_of_rows, lse_batch, batch_row0, row0 + tid, rows, heads, T);
             }
         };
-        auto place_rows = [&](int tile) {
-            unsigned char* buffer = lds + ((tile - first_tile) & 1) * L::BUFFER_BYTES;
-            place_tile<WIDTH>(q_share, buffer + L::Q_ROWS, 0, tid);
-            place_tile<WIDTH>(rope_share, buffer + L::Q_ROWS, RANK, tid);
-            place_tile<RANK>(do_share, buffer + L::DO_ROWS, 0, tid);
+        // after the wave's requests have arrived
+        auto place_statistics = [&](int parity) {
             if (tid < TILE) {
-                float* lse2 = reinterpret_cast<float*>(buffer + L::STATS);
-                lse2[tid] = statistics.lse2;
+                float* lse2 = reinterpret_cast<float*>(lds + parity * L::BUFFER_BYTES + L::STATS);
+                lse2[tid] = statistics.lse * LOG2E;
                 lse2[TILE + tid] = statistics.delta;
                 reinterpret_cast<int*>(lse2)[2 * TILE + tid] = statistics.token;
             }
         };
-        // Tile t is multiplied out of one buffer while tile t + 1 goes from registers into the other and tile
-        // t + 2 is on its way from memory: a fetch has a whole step to arrive, and a step has one barrier.
-        // (A second register set, for a fetch two steps ahead, was tried: the compiler waits for all
-        // outstanding loads before the first use of any, so the depth is lost, and the kernel spills.)
-        fetch_rows(first_tile);
-        __syncthreads();   // the previous segment has been read
-        place_rows(first_tile);
-        if (first_tile + 1 < end_tile) fetch_rows(first_tile + 1);
 
-        for (int tile = first_tile; tile < end_tile; ++tile) {
-            const unsigned char* buffer = lds + ((tile - first_tile) & 1) * L::BUFFER_BYTES;
-            const unsigned char* q_rows = buffer + L::Q_ROWS;
+        // scores of one tile: (rows x keys) quadrants of 16 x 16, lane holds key 16*kh + l16 and rows 4*quad .. +3 of
+        // the wave's 16; the score and dP products take turns, every row fragment serves both key halves
+        auto score_tile = [&](const unsigned char* buffer, unsigned char* exchange) {
+            const unsigned char* q_latent = buffer + L::Q_LATENT;
+            const unsigned char* q_rope = buffer + L::Q_ROPE;
             const unsigned char* do_rows = buffer + L::DO_ROWS;
             const float* lse2 = reinterpret_cast<const float*>(buffer + L::STATS);
             const float* delta = lse2 + TILE;
             const int* token_of = reinterpret_cast<const int*>(delta + TILE);
-            __syncthreads();   // this tile is in place, the other buffer has been read
-            if (tile + 1 < end_tile) {
-                place_rows(tile + 1);
-                if (tile + 2 < end_tile) fetch_rows(tile + 2);
-            }
-
-            // (rows x keys) quadrant: lane holds key l16 and rows 4*quad .. +3 of the wave's halves; the score and dP
-            // products take turns
-            f32x4 s_acc = {0.f, 0.f, 0.f, 0.f}, dp_acc = {0.f, 0.f, 0.f, 0.f};
+            f32x4 s_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            f32x4 dp_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
             bf16x8 ring[AHEAD];
             auto row_fragment = [&](auto tag) {
                 constexpr int I = decltype(tag)::value;
                 if constexpr (I >= 2 * O_STEPS) {
-                    return quadrant_fragment<WIDTH>(q_rows, 16 * row_half + l16, I - O_STEPS, quad);
+                    return quadrant_fragment<I - 2 * O_STEPS>(q_rope, narrow_quadrant);
                 } else if constexpr (I % 2 == 0) {
-                    return quadrant_fragment<WIDTH>(q_rows, 16 * row_half + l16, I / 2, quad);
+                    return quadrant_fragment<I / 2>(q_latent, wide_quadrant);
                 } else {
-                    return quadrant_fragment<RANK>(do_rows, 16 * row_half + l16, I / 2, quad);
+                    return quadrant_fragment<I / 2>(do_rows, wide_quadrant);
                 }
             };
             fill_ring(ring, row_fragment);
             fragment_stream<Q_STEPS + O_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
                 constexpr int I = decltype(tag)::value;
-                if constexpr (I >= 2 * O_STEPS) {
-                    s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I - O_STEPS], s_acc, 0, 0, 0);
-                } else if constexpr (I % 2 == 0) {
-                    s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I / 2], s_acc, 0, 0, 0);
-                } else {
-                    dp_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[I / 2], dp_acc, 0, 0, 0);
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh) {
+                    if constexpr (I >= 2 * O_STEPS) {
+                        s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I - O_STEPS], s_acc[kh], 0, 0, 0);
+                    } else if constexpr (I % 2 == 0) {
+                        s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], s_acc[kh], 0, 0, 0);
+                    } else {
+                        dp_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], dp_acc[kh], 0, 0, 0);
+                    }
                 }
             });
-
-            // per 16-row step n: (q columns, dO columns) of the wave's four latent blocks, then its rope block; the
-            // first fragments are on their way during the softmax
-            auto column_fragment = [&](auto tag) {
-                constexpr int N = decltype(tag)::value / 9;
-                constexpr int F = decltype(tag)::value % 9;
-                if constexpr (F == 8) {
-                    return transposed_fragment<WIDTH>(q_rows, q_transposed_at, RANK + 32 * (wave % 2), N);
-                } else if constexpr (F % 2 == 0) {
-                    return transposed_fragment<WIDTH>(q_rows, q_transposed_at, 32 * (4 * wave + F / 2), N);
-                } else {
-                    return transposed_fragment<RANK>(do_rows, do_transposed_at, 32 * (4 * wave + F / 2), N);
-                }
-            };
-            fill_ring(ring, column_fragment);
-
-            {
-                const int local = 16 * row_half + 4 * quad;
-                const int own_key = k0 + 16 * key_half + l16;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
-                const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
-                const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+            const int local = 16 * half + 4 * quad;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
+            const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
+            const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                const int own_key = k0 + 16 * kh + l16;
                 float p[4], ds[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -lse4[i]));
+                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[kh][i], c, -lse4[i]));
                     if (own_key > (int)token4[i]) probability = 0.f;
                     p[i] = probability;
-                    ds[i] = probability * (dp_acc[i] - delta4[i]) * scale;
+                    ds[i] = probability * (dp_acc[kh][i] - delta4[i]) * scale;
                 }
-                exchange_store(p_exchange, 16 * key_half + l16, local, p);     // [key][row]
-                exchange_store(ds_exchange, 16 * key_half + l16, local, ds);
+                exchange_store(exchange, 16 * kh + l16, local, p);     // [key][row]
+                exchange_store(exchange + EXCHANGE_BYTES, 16 * kh + l16, local, ds);
             }
-            __syncthreads();   // the four quadrants are in place
+        };
+
+        // One step of a gradient wave: the held fragments (tile t - 1) meet P and dS of that tile, and each gives way
+        // to the same fragment of tile t in `buffer`.  Per 16-row step n: the query columns of the wave's eight
+        // latent blocks (with dS), its rope block (with dS), the dO columns of the latent blocks (with P):
+        // neighbouring products go to different accumulators.
+        auto add_tile = [&](const unsigned char* buffer, const unsigned char* exchange, bool any) {
+            const unsigned char* q_latent = buffer + L::Q_LATENT;
+            const unsigned char* q_rope = buffer + L::Q_ROPE;
+            const unsigned char* do_rows = buffer + L::DO_ROWS;
             bf16x8 pf[2], dsf[2];
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                pf[n] = exchange_fragment(p_exchange, lq, g, n);
-                dsf[n] = exchange_fragment(ds_exchange, lq, g, n);
-            }
-            fragment_stream<18>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
-                constexpr int N = decltype(tag)::value / 9;
-                constexpr int F = decltype(tag)::value % 9;
-                if constexpr (F == 8) {
-                    rope_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], fragment, rope_acc, 0, 0, 0);
-                } else if constexpr (F % 2 == 0) {
-                    latent_acc[F / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], fragment, latent_acc[F / 2], 0, 0, 0);
-                } else {
-                    latent_acc[F / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[N], fragment, latent_acc[F / 2], 0, 0, 0);
+                pf[n] = dsf[n] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+                if (any) {
+                    pf[n] = exchange_fragment(exchange, lq, g, n);
+                    dsf[n] = exchange_fragment(exchange + EXCHANGE_BYTES, lq, g, n);
                 }
+            }
+            static_for<0, 2 * PER_STEP>([&](auto tag) {
+                constexpr int I = decltype(tag)::value;
+                constexpr int N = I / PER_STEP;
+                constexpr int F = I % PER_STEP;
+                if constexpr (F < LATENT_BLOCKS) {
+                    latent_acc[F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], held[I], latent_acc[F], 0, 0, 0);
+                    held[I] = transposed_fragment(q_latent, wide_columns.low[F % 4], wide_columns.high[F % 4],
+                                                  N * 16 * Wide::ROW + 256 * (F / 4));
+                } else if constexpr (F == LATENT_BLOCKS) {
+                    rope_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[N], held[I], rope_acc, 0, 0, 0);
+                    held[I] = transposed_fragment(q_rope, rope_columns_low, rope_columns_high, N * 16 * Narrow::ROW);
+                } else {
+                    constexpr int J = F - LATENT_BLOCKS - 1;
+                    latent_acc[J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[N], held[I], latent_acc[J], 0, 0, 0);
+                    held[I] = transposed_fragment(do_rows, wide_columns.low[J % 4], wide_columns.high[J % 4],
+                                                  N * 16 * Wide::ROW + 256 * (J / 4));
+                }
+                __builtin_amdgcn_sched_barrier(0);
             });
+        };
+
+        // Step t: tile t is in buffer t % 2 (scored there, and picked up by the gradient waves for step t + 1), tile
+        // t + 1 arrives in the other buffer.  One more step after the last tile lets the gradient waves catch up.
+        // Every step ends with a barrier behind all LDS reads, so the buffers are free when a segment begins.
+        request_rows(first_tile, 0);
+        wait_vector_memory<0>();
+        place_statistics(0);
+        workgroup_barrier();
+
+        for (int tile = first_tile; tile <= end_tile; ++tile) {
+            const int parity = (tile - first_tile) & 1;
+            const bool more = tile + 1 < end_tile;
+            if (more) request_rows(tile + 1, parity ^ 1);
+            if constexpr (SCORES) {
+                if (tile < end_tile) {
+                    score_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + parity * L::EXCHANGE_PAIR);
+                }
+            } else {
+                add_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + (parity ^ 1) * L::EXCHANGE_PAIR,
+                         tile > first_tile);
+            }
+            wait_vector_memory<0>();
+            if (more) place_statistics(parity ^ 1);
+            workgroup_barrier();   // tile t has been read, P and dS of it and tile t + 1 are in place
         }
 
-        // lane holds column (block, lq) and keys k0 + 8*(i/4) + 4*g + i%4
-        if (whole) {
+        // gradient waves: lane holds column (block, lq) and keys k0 + 8*(i/4) + 4*g + i%4
+        if constexpr (!SCORES) {
+            if (whole) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int k = k0 + 8 * (i / 4) + 4 * g + i % 4;
-                if (k < T) {
-                    __bf16* latent_row = reinterpret_cast<__bf16*>(kv_latent_gradient) + ((size_t)batch * T + k) * RANK;
+                for (int i = 0; i < 16; ++i) {
+                    const int k = k0 + 8 * (i / 4) + 4 * g + i % 4;
+                    if (k < T) {
+                        __bf16* latent_row = reinterpret_cast<__bf16*>(kv_latent_gradient) + ((size_t)batch * T + k) * RANK;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) latent_row[32 * (4 * wave + j) + lq] = (__bf16)latent_acc[j][i];
-                    if (wave < 2) {
+                        for (int j = 0; j < LATENT_BLOCKS; ++j) {
+                            latent_row[32 * (LATENT_BLOCKS * half + j) + lq] = (__bf16)latent_acc[j][i];
+                        }
                         __bf16* rope_row = reinterpret_cast<__bf16*>(key_rope_gradient) + ((size_t)batch * T + k) * ROPE;
-                        rope_row[32 * wave + lq] = (__bf16)rope_acc[i];
+                        rope_row[32 * half + lq] = (__bf16)rope_acc[i];
                     }
                 }
-            }
-        } else {
-            const long long slot_number =
-                interval_length > 0 ? (long long)blockIdx.x : (long long)blockIdx.x + (long long)batch * visits.key_blocks + key_block;
-            float* slot = partial_slots + slot_number * PARTIAL_FLOATS;
+            } else {
+                const long long slot_number =
+                    interval_length > 0 ? item : (long long)blockIdx.x + (long long)batch * visits.key_blocks + key_block;
+                float* slot = partial_slots + slot_number * PARTIAL_FLOATS;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float* slot_row = slot + (8 * (i / 4) + 4 * g + i % 4) * WIDTH;
+                for (int i = 0; i < 16; ++i) {
+                    float* slot_row = slot + (8 * (i / 4) + 4 * g + i % 4) * WIDTH;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) slot_row[32 * (4 * wave + j) + lq] = latent_acc[j][i];
-                if (wave < 2) slot_row[RANK + 32 * wave + lq] = rope_acc[i];
+                    for (int j = 0; j < LATENT_BLOCKS; ++j) slot_row[32 * (LATENT_BLOCKS * half + j) + lq] = latent_acc[j][i];
+                    slot_row[RANK + 32 * half + lq] = rope_acc[i];
+                }
             }
         }
         position = batch * per_batch + segment_end;
+    }
+}
+
+__global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
+    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
+    const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
+    const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
+    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int batch_size, int sequence_length,
+    int heads, int ranges, int interval_length, float scale) {
+    if (threadIdx.x < THREADS / 2) {
+        key_gradient_walk<true>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient,
+                                logsumexp, query_latent, query_rope, kv_latent, key_rope, batch_size, sequence_length,
+                                heads, ranges, interval_length, scale);
+    } else {
+        key_gradient_walk<false>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient,
+                                 logsumexp, query_latent, query_rope, kv_latent, key_rope, batch_size, sequence_length,
+                                 heads, ranges, interval_length, scale);
     }
 }
 

@@ -138,6 +138,18 @@ void check_fragment_reads() {
             }
         }
     }
+    // quadrant (16x16x32 operand layout: lane l holds row l % 16 and contraction indices 8 * (l / 16) + j of a
+    // 32-column step): operand row = tile row ROW0 + l % 16, first column 32 * S + 8 * (l / 16)
+    for (int row0 : {0, 16, 32, 48}) {
+        for (int step = 0; step < COLUMNS / 32; ++step) {
+            for (int lane = 0; lane < 64; ++lane) {
+                int row, column;
+                locate<ROW_BYTES>(Math::quadrant(step % Math::TR, lane) + Math::quadrant_constant(row0, step), row, column);
+                EXPECT(row == row0 + lane % 16 && column == 32 * step + 8 * (lane / 16),
+                       "quadrant ROW_BYTES %d row0 %d step %d lane %d -> row %d column %d", ROW_BYTES, row0, step, lane, row, column);
+            }
+        }
+    }
     // transposed: operand row = tile column 32 * BLOCK + l % 32, contraction index j -> tile row
     // ROW0 + {4g .. 4g+3, 8+4g .. 8+4g+3}[j], g = l / 32 (two reads, h = 0 for j < 4, h = 1 for j >= 4)
     for (int row0 : {0, 16, 32, 48}) {
@@ -160,6 +172,27 @@ void check_fragment_reads() {
                                block, h, lane, e, row, column);
                     }
                 }
+            }
+        }
+    }
+}
+
+// ---- list entries of workgroups: a bijection; the workgroups of one L2 domain take a contiguous stretch in order
+void check_entries_of_workgroups() {
+    for (int clusters : {1, 8}) {
+        for (long long count : {1LL, 2LL, 7LL, 8LL, 9LL, 63LL, 64LL, 255LL, 4160LL, 4163LL}) {
+            std::vector<int> taken(count, 0);
+            for (long long workgroup = 0; workgroup < count; ++workgroup) {
+                const long long entry = entry_of_workgroup(workgroup, count, clusters);
+                EXPECT(entry >= 0 && entry < count, "clusters %d count %lld workgroup %lld -> %lld", clusters, count, workgroup, entry);
+                if (entry >= 0 && entry < count) ++taken[entry];
+                if (workgroup >= clusters) {
+                    EXPECT(entry == entry_of_workgroup(workgroup - clusters, count, clusters) + 1,
+                           "clusters %d count %lld workgroup %lld: the domain's entries are not consecutive", clusters, count, workgroup);
+                }
+            }
+            for (long long entry = 0; entry < count; ++entry) {
+                EXPECT(taken[entry] == 1, "clusters %d count %lld: entry %lld taken %d times", clusters, count, entry, taken[entry]);
             }
         }
     }
@@ -493,6 +526,7 @@ int main() {
     check_swizzle<128>();
     check_swizzle<256>();
     check_swizzle<384>();
+    check_swizzle<1024>();
     check_swizzle<1152>();
     check_requests<384, 4>();
     check_requests<256, 4>();
@@ -503,6 +537,9 @@ int main() {
     check_fragment_reads<128>();
     check_fragment_reads<256>();
     check_fragment_reads<384>();
+    check_fragment_reads<1024>();
+    check_fragment_reads<1152>();
+    check_entries_of_workgroups();
     check_ds_blocks();
     check_forward_items();
     check_decode_loads<16>();
