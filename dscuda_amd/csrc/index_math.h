@@ -334,16 +334,6 @@ DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int he
     return cut;
 }
 
-// Workgroups are handed to the chip's `clusters` L2 domains in turn (workgroup w runs in domain w % clusters), and
-// the ones resident at any time have neighbouring numbers.  To let the workgroups that share an L2 walk
-// neighbouring entries of a list of `count` entries, domain d takes the d-th of `clusters` contiguous stretches of
-// the list (lengths differ by at most one) and its workgroups, in launch order, the entries of that stretch in order.
-DSCUDA_HOST_DEVICE inline long long entry_of_workgroup(long long workgroup, long long count, int clusters) {
-    const long long domain = workgroup % clusters;
-    const long long stretch = count / clusters, longer = count % clusters;
-    return domain * stretch + (domain < longer ? domain : longer) + workgroup / clusters;
-}
-
 constexpr long long KEY_PARTIAL_BYTES = 32LL * 576 * 4;   // one slot: [32 keys][576] fp32
 
 // How many ranges the list is cut into when `scratch_bytes` are there for the slots: one per compute unit if the

@@ -58,7 +58,6 @@ constexpr int ROPE = 64;
 constexpr int WIDTH = RANK + ROPE;
 constexpr int TILE = 32;
 constexpr int THREADS = 256;
-constexpr int L2_DOMAINS = 8;   // the chip's XCDs: workgroup w of a launch runs on XCD w % 8
 
 // A [32][D] LDS tile of bf16, row-major without padding: 16-byte chunk c of row r sits at position
 // c ^ tile_swizzle(r), which spreads both the 16-byte reads down a column and the transposing reads over the banks.
@@ -281,180 +280,270 @@ __device__ __forceinline__ RowStatistics fetch_row_statistics(const float* delta
 
 // ---- query gradients -----------------------------------------------------------
 
+constexpr int QUERY_THREADS = 512;
+constexpr int QUERY_ROWS = 64;   // rows of one workgroup: every key tile it fetches serves two row tiles
+
 struct QueryGradLayout {
-    static constexpr int BUFFER_BYTES = Tile32<WIDTH>::BYTES;  // [32 keys][576]
-    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;          // the tile being multiplied and the next one
-    static constexpr int LDS_BYTES = EXCHANGE + EXCHANGE_BYTES;
+    static constexpr int K_LATENT = 0;                                    // [32 keys][512]
+    static constexpr int K_ROPE = K_LATENT + Tile32<RANK>::BYTES;         // [32 keys][64]
+    static constexpr int BUFFER_BYTES = K_ROPE + Tile32<ROPE>::BYTES;
+    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;                     // the tile in use and the one arriving
+    static constexpr int EXCHANGE_PAIR = 2 * EXCHANGE_BYTES;              // dS of the two row tiles against one key tile
+    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_PAIR;        // of the key tile being scored and the one before
 };
 
-__global__ __launch_bounds__(THREADS) void mla_absorbed_query_gradient_kernel(
+// Eight waves, two per SIMD, in two roles (the design of the key-gradient kernel below, turned round: here the rows
+// stay and the key tiles pass).  Waves 0..3 form the scores: wave w holds rows 16*w .. +15 of the workgroup's 64
+// as register operands (query and dO row), multiplies every key fragment it reads from LDS into the score and the
+// dP product, applies the softmax gradient and leaves dS in the exchange tile of its row tile.  Waves 4..7 hold
+// the sums: wave 4 + v row tile v / 2, eight latent column blocks and one rope block (halves v % 2); they keep the
+// transposed fragments of the key tile BEFORE in registers, multiply them with that tile's dS while the next
+// scores are formed, and replace each by the same fragment of the tile being scored.  So one key tile is read at
+// a time, the other buffer is free during the whole step and the next tile goes straight from memory into it
+// (global_load_lds, requested from inside the product streams, awaited before the step's one barrier).  Each SIMD
+// carries a score wave (68 products of 16x16x32) and a gradient wave (18 of 32x32x16).
+// The walk is compiled once per role so that the roles share the register file.
+template <bool SCORES>
+__device__ __forceinline__ void query_gradient_walk(
     bf16_t* query_latent_gradient, bf16_t* query_rope_gradient, const float* delta_of_rows,
     const bf16_t* __restrict__ output_gradient, const float* __restrict__ logsumexp,
     const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
     const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
     int row_blocks, float scale) {
     using L = QueryGradLayout;
-    constexpr int BLOCKS = WIDTH / 32;                 // 18 column blocks of dQ
-    constexpr int OWN = (BLOCKS + 3) / 4;              // at most 5 per wave
-    constexpr int QK_STEPS = WIDTH / 16;               // 36
-    constexpr int V_STEPS = RANK / 16;                 // 32
+    using Wide = Tile32<RANK>;
+    using Narrow = Tile32<ROPE>;
+    constexpr int Q_STEPS = WIDTH / 32;   // 18
+    constexpr int O_STEPS = RANK / 32;    // 16
     constexpr int AHEAD = 6;
+    constexpr int LATENT_BLOCKS = 8;      // per gradient wave
+    constexpr int BLOCKS = LATENT_BLOCKS + 1;
+    constexpr int ROWS_PER_WAVE = TILE / 8;   // key rows of the wide tile a wave requests
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x;
-    __builtin_assume(tid >= 0 && tid < THREADS);   // lets the per-piece bounds of the tile shares fold away
+    __builtin_assume(tid >= 0 && tid < QUERY_THREADS);
     const int wave = tid / 64;
     const int lane = tid % 64;
     const int lq = lane % 32;
     const int g = lane / 32;
+    const int l16 = lane % 16;
+    const int quad = lane / 16;
     const int T = sequence_length;
 
     const int batch = blockIdx.x / row_blocks;
     const int row_block = row_blocks - 1 - blockIdx.x % row_blocks;   // latest rows (most keys) first
     const long long rows = (long long)T * heads;
-    const long long row0 = (long long)row_block * TILE;
+    const long long row0 = (long long)row_block * QUERY_ROWS;
     const long long batch_row0 = (long long)batch * rows;
     const bf16_t* latent = kv_latent + (size_t)batch * T * RANK;
     const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
 
-    TileShare<RANK> latent_share;
-    TileShare<ROPE> rope_share;
-    auto fetch_keys = [&](int tile) {
-        const int key0 = tile * TILE;
-        fetch_tile(latent_share, latent + (size_t)key0 * RANK, T - key0, tid);
-        fetch_tile(rope_share, rope + (size_t)key0 * ROPE, T - key0, tid);
-    };
-    auto place_keys = [&](int tile) {
-        unsigned char* keys = lds + (tile & 1) * L::BUFFER_BYTES;
-        place_tile<WIDTH>(latent_share, keys, 0, tid);
-        place_tile<WIDTH>(rope_share, keys, RANK, tid);
-    };
-    fetch_keys(0);
-
-    // this wave's quadrant of the score tile: keys 16*key_half .. +15 x rows 16*row_half .. +15.  Its rows as B
-    // operands (column = row l16): the query row and its dO row
-    constexpr int Q_STEPS = WIDTH / 32;   // 18
-    constexpr int O_STEPS = RANK / 32;    // 16
-    const int key_half = wave / 2;
-    const int row_half = wave % 2;
-    const int l16 = lane % 16;
-    const int quad = lane / 16;
-    const long long own_row = row0 + 16 * row_half + l16;
-    const bool own_valid = own_row < rows;
-    const size_t own = batch_row0 + (own_valid ? own_row : 0);
-    bf16x8 qf[Q_STEPS], dof[O_STEPS];
-    fetch_quadrant_operand(qf, query_latent + own * RANK, query_rope + own * ROPE, own_valid, quad);
-    fetch_quadrant_operand(dof, output_gradient + own * RANK, nullptr, own_valid, quad);
-    const RowStatistics statistics = fetch_row_statistics(delta_of_rows, logsumexp + (size_t)batch * heads * T,
-                                                          batch_row0, own_row, rows, heads, T);
-    const float row_lse2 = statistics.lse * LOG2E;
-    const float row_delta = statistics.delta;
-    const int row_token = statistics.token;
-    const QuadrantAt<WIDTH> key_rows(lane, key_half);
-    // the wave's column blocks of the key tile: wave + 4*J for J < 4 and, last, 16 + wave % 2 (for waves 2 and 3 a
-    // duplicate that is never stored) -- all of parity wave % 2, two blocks share 128 bytes of a row
-    using KeyRead = Tile32<WIDTH>::Read;
-    const int key_columns_low = (int)KeyRead::transposed(0, wave % 2, lane) + 128 * (wave / 2);
-    const int key_columns_high = (int)KeyRead::transposed(1, wave % 2, lane) + 128 * (wave / 2);
-    const int last_columns_low = (int)KeyRead::transposed(0, wave % 2, lane) + 128 * 8;
-    const int last_columns_high = (int)KeyRead::transposed(1, wave % 2, lane) + 128 * 8;
-    unsigned char* exchange = lds + L::EXCHANGE;
-    const long long row = row0 + lq;   // the row whose gradient this lane ends up with
-    const bool valid = row < rows;
-
-    const long long last_row = min(rows, row0 + TILE) - 1;
+    const long long last_row = min(rows, row0 + QUERY_ROWS) - 1;
     const int visible = (int)(last_row / heads) + 1;
     const int tiles = (visible + TILE - 1) / TILE;
     const float c = scale * LOG2E;
 
-    f32x16 dq_acc[OWN];
+    // Requests of a key tile: the wave brings key rows 4*wave .. +3 of the wide tile (an instruction fills one row:
+    // lane l fetches the chunk that belongs at position l), waves 0..3 also instruction `wave` of the narrow tile
+    // (eight rows of eight chunks).  Keys past the last one repeat it: every row's token is below them, so their
+    // dS is zero whatever they hold.
+    const unsigned lds_base = lds_offset_of(lds);
+    unsigned wide_part[ROWS_PER_WAVE];
 #pragma unroll
-    for (int j = 0; j < OWN; ++j) clear(dq_acc[j]);
-
-    // Tile t is multiplied out of buffer t % 2 while tile t + 1 goes from registers into the other buffer and
-    // tile t + 2 is on its way from memory: a fetch has a whole step to arrive, and a step has one barrier.
-    place_keys(0);
-    if (tiles > 1) fetch_keys(1);
-    for (int tile = 0; tile < tiles; ++tile) {
+    for (int j = 0; j < ROWS_PER_WAVE; ++j) {
+        wide_part[j] = 16u * (unsigned)(lane ^ index_math::tile_swizzle<Wide::ROW>(ROWS_PER_WAVE * wave + j));
+    }
+    const int narrow_row = 8 * (wave % 4) + lane / 8;
+    const unsigned narrow_part = 16u * (unsigned)((lane % 8) ^ index_math::tile_swizzle<Narrow::ROW>(narrow_row));
+    constexpr int REQUESTS = ROWS_PER_WAVE + 1;
+    struct {
+        const bf16_t* latent;
+        const bf16_t* rope;
+        int last_valid;
+        unsigned buffer;
+    } arriving;
+    auto begin_requests = [&](int tile, int parity) {
         const int key0 = tile * TILE;
-        const unsigned char* keys = lds + (tile & 1) * L::BUFFER_BYTES;
-        __syncthreads();   // this tile is in place, the other buffer has been read
-        if (tile + 1 < tiles) {
-            place_keys(tile + 1);
-            if (tile + 2 < tiles) fetch_keys(tile + 2);
+        arriving.latent = latent + (size_t)key0 * RANK;
+        arriving.rope = rope + (size_t)key0 * ROPE;
+        arriving.last_valid = min(T - key0, TILE) - 1;
+        arriving.buffer = lds_base + parity * L::BUFFER_BYTES;
+    };
+    auto request = [&](auto tag) {
+        constexpr int R = decltype(tag)::value;
+        if constexpr (R < ROWS_PER_WAVE) {
+            const int row = ROWS_PER_WAVE * wave + R;
+            direct_load_16_offset(arriving.latent, wide_part[R] + (unsigned)(min(row, arriving.last_valid) * Wide::ROW),
+                                  arriving.buffer + L::K_LATENT + row * Wide::ROW);
+        } else if constexpr (R == ROWS_PER_WAVE) {
+            if constexpr (SCORES) {
+                direct_load_16_offset(arriving.rope, narrow_part + (unsigned)(min(narrow_row, arriving.last_valid) * Narrow::ROW),
+                                      arriving.buffer + L::K_ROPE + 8 * wave * Narrow::ROW);
+            }
         }
+    };
 
-        // (keys x rows) quadrant: lane holds row l16 and keys 4*quad .. +3 of the wave's halves.  A key fragment of
-        // the latent part serves the score product and the dP product.
-        f32x4 s_acc = {0.f, 0.f, 0.f, 0.f}, dp_acc = {0.f, 0.f, 0.f, 0.f};
+    // score waves: rows 16*wave .. +15 as B operands (column = row l16): the query row and its dO row
+    bf16x8 qf[Q_STEPS], dof[O_STEPS];
+    float row_lse2 = 0.f, row_delta = 0.f;
+    int row_token = -1;
+    const QuadrantAt<RANK> wide_quadrant(lane, 0);
+    const QuadrantAt<ROPE> narrow_quadrant(lane, 0);
+    if constexpr (SCORES) {
+        const long long own_row = row0 + 16 * wave + l16;
+        const bool own_valid = own_row < rows;
+        const size_t own = batch_row0 + (own_valid ? own_row : 0);
+        fetch_quadrant_operand(qf, query_latent + own * RANK, query_rope + own * ROPE, own_valid, quad);
+        fetch_quadrant_operand(dof, output_gradient + own * RANK, nullptr, own_valid, quad);
+        const RowStatistics statistics = fetch_row_statistics(delta_of_rows, logsumexp + (size_t)batch * heads * T,
+                                                              batch_row0, own_row, rows, heads, T);
+        row_lse2 = statistics.lse * LOG2E;
+        row_delta = statistics.delta;
+        row_token = statistics.token;
+    }
+
+    // gradient waves: row tile `row_tile` of the two, latent column blocks 8*half .. +7 and rope block half
+    const int row_tile = (wave % 4) / 2;
+    const int half = wave % 2;
+    const TransposedAt<RANK> wide_columns(lane, 512 * half);
+    const int rope_columns_low = (int)Narrow::Read::transposed(0, half, lane);
+    const int rope_columns_high = (int)Narrow::Read::transposed(1, half, lane);
+    f32x16 dq_acc[BLOCKS];
+    bf16x8 held[2 * BLOCKS];   // the column fragments of the key tile before the one in LDS (zero before the first)
+    if constexpr (!SCORES) {
+#pragma unroll
+        for (int j = 0; j < BLOCKS; ++j) clear(dq_acc[j]);
+#pragma unroll
+        for (int f = 0; f < 2 * BLOCKS; ++f) held[f] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+    }
+
+    // (keys x rows) quadrants of 16 x 16, lane holds row l16 and keys 4*quad .. +3 of each key half.  A key fragment
+    // of the latent part serves the score product and the dP product.
+    auto score_tile = [&](const unsigned char* buffer, unsigned char* exchange, int key0) {
+        const unsigned char* k_latent = buffer + L::K_LATENT;
+        const unsigned char* k_rope = buffer + L::K_ROPE;
+        f32x4 s_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        f32x4 dp_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
         bf16x8 ring[AHEAD];
         auto key_fragment = [&](auto tag) {
-            return quadrant_fragment<decltype(tag)::value>(keys, key_rows);
+            constexpr int S = decltype(tag)::value / 2;
+            constexpr int KH = decltype(tag)::value % 2;
+            if constexpr (S < O_STEPS) {
+                return quadrant_fragment<S>(k_latent + KH * 16 * Wide::ROW, wide_quadrant);
+            } else {
+                return quadrant_fragment<S - O_STEPS>(k_rope + KH * 16 * Narrow::ROW, narrow_quadrant);
+            }
         };
         fill_ring(ring, key_fragment);
-        fragment_stream<Q_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
-            constexpr int S = decltype(tag)::value;
-            s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, qf[S], s_acc, 0, 0, 0);
+        fragment_stream<2 * Q_STEPS>(ring, key_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int I = decltype(tag)::value;
+            constexpr int S = I / 2;
+            constexpr int KH = I % 2;
+            s_acc[KH] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, qf[S], s_acc[KH], 0, 0, 0);
             if constexpr (S < O_STEPS) {
-                dp_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, dof[S], dp_acc, 0, 0, 0);
+                dp_acc[KH] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, dof[S], dp_acc[KH], 0, 0, 0);
             }
+            if constexpr (I % 7 == 0) request(std::integral_constant<int, I / 7>{});
         });
-
-        // dQ^T += K^T dS^T for this wave's column blocks; the first fragments are on their way during the softmax
-        auto column_fragment = [&](auto tag) {
-            constexpr int J = decltype(tag)::value / 2;
-            constexpr int N = decltype(tag)::value % 2;
-            constexpr int ROWS_DOWN = N * 16 * Tile32<WIDTH>::ROW;
-            if constexpr (J < 4) {
-                return transposed_fragment(keys, key_columns_low, key_columns_high, ROWS_DOWN + 256 * J);
-            } else {
-                return transposed_fragment(keys, last_columns_low, last_columns_high, ROWS_DOWN);
-            }
-        };
-        fill_ring(ring, column_fragment);
-
-        {
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
             float ds[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int k = key0 + 16 * key_half + 4 * quad + i;
-                float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[i], c, -row_lse2));
+                const int k = key0 + 16 * kh + 4 * quad + i;
+                float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[kh][i], c, -row_lse2));
                 if (k > row_token) probability = 0.f;
-                ds[i] = probability * (dp_acc[i] - row_delta) * scale;
+                ds[i] = probability * (dp_acc[kh][i] - row_delta) * scale;
             }
-            exchange_store(exchange, 16 * row_half + l16, 16 * key_half + 4 * quad, ds);   // [row][key]
+            exchange_store(exchange, 16 * (wave % 2) + l16, 16 * kh + 4 * quad, ds);   // [row][key]
         }
-        __syncthreads();   // the four quadrants are in place
+    };
+
+    // dQ^T += K^T dS^T: the held fragments (key tile t - 1) meet dS of that tile, and each gives way to the same
+    // fragment of tile t in `buffer`
+    auto add_tile = [&](const unsigned char* buffer, const unsigned char* exchange, bool any) {
+        const unsigned char* k_latent = buffer + L::K_LATENT;
+        const unsigned char* k_rope = buffer + L::K_ROPE;
         bf16x8 dsf[2];
 #pragma unroll
-        for (int n = 0; n < 2; ++n) dsf[n] = exchange_fragment(exchange, lq, g, n);
-        fragment_stream<2 * OWN>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
-            constexpr int J = decltype(tag)::value / 2;
-            constexpr int N = decltype(tag)::value % 2;
-            dq_acc[J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, dsf[N], dq_acc[J], 0, 0, 0);
+        for (int n = 0; n < 2; ++n) {
+            dsf[n] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+            if (any) dsf[n] = exchange_fragment(exchange, lq, g, n);
+        }
+        static_for<0, 2 * BLOCKS>([&](auto tag) {
+            constexpr int I = decltype(tag)::value;
+            constexpr int N = I / BLOCKS;
+            constexpr int F = I % BLOCKS;
+            dq_acc[F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(held[I], dsf[N], dq_acc[F], 0, 0, 0);
+            if constexpr (F < LATENT_BLOCKS) {
+                held[I] = transposed_fragment(k_latent, wide_columns.low[F % 4], wide_columns.high[F % 4],
+                                              N * 16 * Wide::ROW + 256 * (F / 4));
+            } else {
+                held[I] = transposed_fragment(k_rope, rope_columns_low, rope_columns_high, N * 16 * Narrow::ROW);
+            }
+            if constexpr (I % 4 == 0) request(std::integral_constant<int, I / 4>{});
+            __builtin_amdgcn_sched_barrier(0);
         });
+    };
+
+    // Step t: key tile t is in buffer t % 2 (scored there, and picked up by the gradient waves for step t + 1), tile
+    // t + 1 arrives in the other buffer; past the last tile the last one is requested again, into a buffer nobody
+    // reads, which keeps the streams free of branches.  One more step lets the gradient waves catch up.
+    begin_requests(0, 0);
+    static_for<0, REQUESTS>(request);
+    wait_vector_memory<0>();
+    workgroup_barrier();
+    for (int tile = 0; tile <= tiles; ++tile) {
+        const int parity = tile & 1;
+        begin_requests(tile + 1 < tiles ? tile + 1 : tiles - 1, parity ^ 1);
+        if constexpr (SCORES) {
+            if (tile < tiles) {
+                score_tile(lds + parity * L::BUFFER_BYTES,
+                           lds + L::EXCHANGE + parity * L::EXCHANGE_PAIR + (wave / 2) * EXCHANGE_BYTES, tile * TILE);
+            }
+        } else {
+            add_tile(lds + parity * L::BUFFER_BYTES,
+                     lds + L::EXCHANGE + (parity ^ 1) * L::EXCHANGE_PAIR + row_tile * EXCHANGE_BYTES, tile > 0);
+        }
+        wait_vector_memory<0>();
+        workgroup_barrier();   // tile t has been read, its dS and tile t + 1 are in place
     }
 
-    // lane holds row lq and columns 32*block + 8*(i/4) + 4*g + i%4
-    if (valid) {
+    // gradient waves: lane holds row lq of the row tile and columns 32*block + 8*(i/4) + 4*g + i%4
+    if constexpr (!SCORES) {
+        const long long row = row0 + TILE * row_tile + lq;
+        if (row < rows) {
 #pragma unroll
-        for (int j = 0; j < OWN; ++j) {
-            const int block = wave + 4 * j;
-            if (block < BLOCKS) {
+            for (int j = 0; j < BLOCKS; ++j) {
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     u32x2 packed;
                     packed.x = pack_bf16(dq_acc[j][4 * i4 + 0], dq_acc[j][4 * i4 + 1]);
                     packed.y = pack_bf16(dq_acc[j][4 * i4 + 2], dq_acc[j][4 * i4 + 3]);
-                    const int column = 32 * block + 8 * i4 + 4 * g;
-                    bf16_t* destination = column < RANK
-                        ? query_latent_gradient + (batch_row0 + row) * RANK + column
-                        : query_rope_gradient + (batch_row0 + row) * ROPE + (column - RANK);
+                    bf16_t* destination = j < LATENT_BLOCKS
+                        ? query_latent_gradient + (batch_row0 + row) * RANK + 32 * (LATENT_BLOCKS * half + j) + 8 * i4 + 4 * g
+                        : query_rope_gradient + (batch_row0 + row) * ROPE + 32 * half + 8 * i4 + 4 * g;
                     *reinterpret_cast<u32x2*>(destination) = packed;
                 }
             }
         }
+    }
+}
+
+__global__ __launch_bounds__(QUERY_THREADS) void mla_absorbed_query_gradient_kernel(
+    bf16_t* query_latent_gradient, bf16_t* query_rope_gradient, const float* delta_of_rows,
+    const bf16_t* __restrict__ output_gradient, const float* __restrict__ logsumexp,
+    const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
+    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
+    int row_blocks, float scale) {
+    if (threadIdx.x < QUERY_THREADS / 2) {
+        query_gradient_walk<true>(query_latent_gradient, query_rope_gradient, delta_of_rows, output_gradient, logsumexp,
+                                  query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, row_blocks, scale);
+    } else {
+        query_gradient_walk<false>(query_latent_gradient, query_rope_gradient, delta_of_rows, output_gradient, logsumexp,
+                                   query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, row_blocks, scale);
     }
 }
 
@@ -612,34 +701,71 @@ __device__ __forceinline__ void key_gradient_walk(
         }
 
         // Rows of a tile past the last row of the batch element repeat that row: their token is -1, which sees no
-        // key, so their P and dS are zero whatever the rows hold.
+        // key, so their P and dS are zero whatever the rows hold.  The wave's REQUESTS requests of a tile are issued
+        // one by one from inside the product streams (issued in one go they fill the queue of the memory pipe and
+        // the wave stands still until it drains); past the last tile of the segment the last tile is requested again,
+        // into a buffer nobody reads, which keeps the streams free of branches.
+        constexpr int REQUESTS = 2 * ROWS_PER_WAVE + 1;
+        struct {
+            const bf16_t* latent;
+            const bf16_t* gradient;
+            const bf16_t* rope;
+            int last_valid;
+            unsigned buffer;
+        } arriving;
         RowStatistics statistics = {0.f, 0.f, -1};
-        auto request_rows = [&](int tile, int parity) {
+        auto begin_requests = [&](int tile, int parity) {
             const long long row0 = (long long)tile * TILE;
-            const int last_valid = (int)min(rows - row0, (long long)TILE) - 1;
-            const unsigned buffer = lds_base + parity * L::BUFFER_BYTES;
-            const bf16_t* ql_tile = ql + row0 * RANK;
-            const bf16_t* do_tile = dout + row0 * RANK;
-#pragma unroll
-            for (int j = 0; j < ROWS_PER_WAVE; ++j) {
-                const int row = ROWS_PER_WAVE * wave + j;
-                const unsigned source = wide_part[j] + (unsigned)(min(row, last_valid) * Wide::ROW);
-                direct_load_16_offset(ql_tile, source, buffer + L::Q_LATENT + row * Wide::ROW);
-                direct_load_16_offset(do_tile, source, buffer + L::DO_ROWS + row * Wide::ROW);
+            arriving.latent = ql + row0 * RANK;
+            arriving.gradient = dout + row0 * RANK;
+            arriving.rope = qr + row0 * ROPE;
+            arriving.last_valid = (int)min(rows - row0, (long long)TILE) - 1;
+            arriving.buffer = lds_base + parity * L::BUFFER_BYTES;
+            // the statistics of its rows: one lane per row, in a gradient wave (the score waves have more to do)
+            if (tid >= 2 * 64 && tid < 2 * 64 + TILE) {
+                const int r = tid - 2 * 64;
+                statistics = {0.f, 0.f, -1};
+                if (r <= arriving.last_valid) {
+                    // rows fit 31 bits as a rule: 32-bit division is a fraction of the 64-bit one
+                    int token, head;
+                    if (rows <= 0x7fffffffLL) {
+                        const unsigned row = (unsigned)row0 + (unsigned)r;
+                        token = (int)(row / (unsigned)heads);
+                        head = (int)(row % (unsigned)heads);
+                    } else {
+                        token = (int)((row0 + r) / heads);
+                        head = (int)((row0 + r) % heads);
+                    }
+                    statistics.lse = lse_batch[(size_t)head * T + token];
+                    statistics.delta = delta_of_rows[(batch_row0 + row0 + r) * DELTA_STRIDE];
+                    statistics.token = token;
+                }
             }
-            direct_load_16_offset(qr + row0 * ROPE, narrow_part + (unsigned)(min(narrow_row, last_valid) * Narrow::ROW),
-                                  buffer + L::Q_ROPE + ROWS_PER_WAVE * wave * Narrow::ROW);
-            if (tid < TILE) {
-                statistics = fetch_row_statistics(delta_of_rows, lse_batch, batch_row0, row0 + tid, rows, heads, T);
+        };
+        auto request = [&](auto tag) {
+            constexpr int R = decltype(tag)::value;
+            if constexpr (R < 2 * ROWS_PER_WAVE) {
+                constexpr int J = R / 2;
+                const int row = ROWS_PER_WAVE * wave + J;
+                const unsigned source = wide_part[J] + (unsigned)(min(row, arriving.last_valid) * Wide::ROW);
+                if constexpr (R % 2 == 0) {
+                    direct_load_16_offset(arriving.latent, source, arriving.buffer + L::Q_LATENT + row * Wide::ROW);
+                } else {
+                    direct_load_16_offset(arriving.gradient, source, arriving.buffer + L::DO_ROWS + row * Wide::ROW);
+                }
+            } else if constexpr (R == 2 * ROWS_PER_WAVE) {
+                direct_load_16_offset(arriving.rope, narrow_part + (unsigned)(min(narrow_row, arriving.last_valid) * Narrow::ROW),
+                                      arriving.buffer + L::Q_ROPE + ROWS_PER_WAVE * wave * Narrow::ROW);
             }
         };
         // after the wave's requests have arrived
         auto place_statistics = [&](int parity) {
-            if (tid < TILE) {
+            if (tid >= 2 * 64 && tid < 2 * 64 + TILE) {
+                const int r = tid - 2 * 64;
                 float* lse2 = reinterpret_cast<float*>(lds + parity * L::BUFFER_BYTES + L::STATS);
-                lse2[tid] = statistics.lse * LOG2E;
-                lse2[TILE + tid] = statistics.delta;
-                reinterpret_cast<int*>(lse2)[2 * TILE + tid] = statistics.token;
+                lse2[r] = statistics.lse * LOG2E;
+                lse2[TILE + r] = statistics.delta;
+                reinterpret_cast<int*>(lse2)[2 * TILE + r] = statistics.token;
             }
         };
 
@@ -678,6 +804,7 @@ __device__ __forceinline__ void key_gradient_walk(
                         dp_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], dp_acc[kh], 0, 0, 0);
                     }
                 }
+                if constexpr (I % 2 == 0) request(std::integral_constant<int, I / 2>{});
             });
             const int local = 16 * half + 4 * quad;
             const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
@@ -733,6 +860,7 @@ __device__ __forceinline__ void key_gradient_walk(
                     held[I] = transposed_fragment(do_rows, wide_columns.low[J % 4], wide_columns.high[J % 4],
                                                   N * 16 * Wide::ROW + 256 * (J / 4));
                 }
+                if constexpr (I % 2 == 0) request(std::integral_constant<int, I / 2>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
@@ -740,7 +868,8 @@ __device__ __forceinline__ void key_gradient_walk(
         // Step t: tile t is in buffer t % 2 (scored there, and picked up by the gradient waves for step t + 1), tile
         // t + 1 arrives in the other buffer.  One more step after the last tile lets the gradient waves catch up.
         // Every step ends with a barrier behind all LDS reads, so the buffers are free when a segment begins.
-        request_rows(first_tile, 0);
+        begin_requests(first_tile, 0);
+        static_for<0, REQUESTS>(request);
         wait_vector_memory<0>();
         place_statistics(0);
         workgroup_barrier();
@@ -748,7 +877,7 @@ __device__ __forceinline__ void key_gradient_walk(
         for (int tile = first_tile; tile <= end_tile; ++tile) {
             const int parity = (tile - first_tile) & 1;
             const bool more = tile + 1 < end_tile;
-            if (more) request_rows(tile + 1, parity ^ 1);
+            begin_requests(more ? tile + 1 : end_tile - 1, parity ^ 1);
             if constexpr (SCORES) {
                 if (tile < end_tile) {
                     score_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + parity * L::EXCHANGE_PAIR);
@@ -758,7 +887,7 @@ __device__ __forceinline__ void key_gradient_walk(
                          tile > first_tile);
             }
             wait_vector_memory<0>();
-            if (more) place_statistics(parity ^ 1);
+            place_statistics(parity ^ 1);
             workgroup_barrier();   // tile t has been read, P and dS of it and tile t + 1 are in place
         }
 
@@ -959,10 +1088,11 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
                            batch_size, (int)ranges, interval_length);
         HIP_CHECK(hipGetLastError());
     }
-    hipLaunchKernelGGL(mla_absorbed_query_gradient_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS),
+    const long long query_blocks = (rows + QUERY_ROWS - 1) / QUERY_ROWS;
+    hipLaunchKernelGGL(mla_absorbed_query_gradient_kernel, dim3((unsigned)(query_blocks * batch_size)), dim3(QUERY_THREADS),
                        QueryGradLayout::LDS_BYTES, stream, query_latent_gradient, query_rope_gradient, delta,
                        output_gradient, logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length, heads,
-                       (int)row_blocks, scale);
+                       (int)query_blocks, scale);
     HIP_CHECK(hipGetLastError());
 }
 

@@ -177,27 +177,6 @@ void check_fragment_reads() {
     }
 }
 
-// ---- list entries of workgroups: a bijection; the workgroups of one L2 domain take a contiguous stretch in order
-void check_entries_of_workgroups() {
-    for (int clusters : {1, 8}) {
-        for (long long count : {1LL, 2LL, 7LL, 8LL, 9LL, 63LL, 64LL, 255LL, 4160LL, 4163LL}) {
-            std::vector<int> taken(count, 0);
-            for (long long workgroup = 0; workgroup < count; ++workgroup) {
-                const long long entry = entry_of_workgroup(workgroup, count, clusters);
-                EXPECT(entry >= 0 && entry < count, "clusters %d count %lld workgroup %lld -> %lld", clusters, count, workgroup, entry);
-                if (entry >= 0 && entry < count) ++taken[entry];
-                if (workgroup >= clusters) {
-                    EXPECT(entry == entry_of_workgroup(workgroup - clusters, count, clusters) + 1,
-                           "clusters %d count %lld workgroup %lld: the domain's entries are not consecutive", clusters, count, workgroup);
-                }
-            }
-            for (long long entry = 0; entry < count; ++entry) {
-                EXPECT(taken[entry] == 1, "clusters %d count %lld: entry %lld taken %d times", clusters, count, entry, taken[entry]);
-            }
-        }
-    }
-}
-
 // ---- dS blocks: key-block-major enumeration of the causal (key block, query tile) pairs, without gaps
 void check_ds_blocks() {
     for (int sequence = 1; sequence <= 4200; sequence += (sequence < 600 ? 1 : 97)) {
@@ -539,7 +518,6 @@ int main() {
     check_fragment_reads<384>();
     check_fragment_reads<1024>();
     check_fragment_reads<1152>();
-    check_entries_of_workgroups();
     check_ds_blocks();
     check_forward_items();
     check_decode_loads<16>();
