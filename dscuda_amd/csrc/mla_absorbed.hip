@@ -296,9 +296,10 @@ struct QueryGradLayout {
 // stay and the key tiles pass).  Waves 0..3 form the scores: wave w holds rows 16*w .. +15 of the workgroup's 64
 // as register operands (query and dO row), multiplies every key fragment it reads from LDS into the score and the
 // dP product, applies the softmax gradient and leaves dS in the exchange tile of its row tile.  Waves 4..7 hold
-// the sums: wave 4 + v row tile v / 2, eight latent column blocks and one rope block (halves v % 2); they keep the
-// transposed fragments of the key tile BEFORE in registers, multiply them with that tile's dS while the next
-// scores are formed, and replace each by the same fragment of the tile being scored.  So one key tile is read at
+// the sums: wave 4 + v the latent column blocks 4*v .. +3 of BOTH row tiles (a key fragment read once serves two
+// products) and rope block v % 2 of row tile v / 2; they keep the transposed fragments of the key tile BEFORE in
+// registers, multiply them with that tile's dS while the next scores are formed, and replace each by the same
+// fragment of the tile being scored.  So one key tile is read at
 // a time, the other buffer is free during the whole step and the next tile goes straight from memory into it
 // (global_load_lds, requested from inside the product streams, awaited before the step's one barrier).  Each SIMD
 // carries a score wave (68 products of 16x16x32) and a gradient wave (18 of 32x32x16).
@@ -316,8 +317,8 @@ __device__ __forceinline__ void query_gradient_walk(
     constexpr int Q_STEPS = WIDTH / 32;   // 18
     constexpr int O_STEPS = RANK / 32;    // 16
     constexpr int AHEAD = 6;
-    constexpr int LATENT_BLOCKS = 8;      // per gradient wave
-    constexpr int BLOCKS = LATENT_BLOCKS + 1;
+    constexpr int LATENT_BLOCKS = 4;      // per gradient wave, of each row tile
+    constexpr int HELD = LATENT_BLOCKS + 1;   // fragments per 16-key step: the latent blocks and the rope block
     constexpr int ROWS_PER_WAVE = TILE / 8;   // key rows of the wide tile a wave requests
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -404,19 +405,24 @@ __device__ __forceinline__ void query_gradient_walk(
         row_token = statistics.token;
     }
 
-    // gradient waves: row tile `row_tile` of the two, latent column blocks 8*half .. +7 and rope block half
-    const int row_tile = (wave % 4) / 2;
-    const int half = wave % 2;
-    const TransposedAt<RANK> wide_columns(lane, 512 * half);
-    const int rope_columns_low = (int)Narrow::Read::transposed(0, half, lane);
-    const int rope_columns_high = (int)Narrow::Read::transposed(1, half, lane);
-    f32x16 dq_acc[BLOCKS];
-    bf16x8 held[2 * BLOCKS];   // the column fragments of the key tile before the one in LDS (zero before the first)
+    // gradient waves: latent column blocks 4*v .. +3 of both row tiles, rope block v % 2 of row tile v / 2
+    const int v = wave % 4;
+    const int rope_tile = v / 2;
+    const int rope_block = v % 2;
+    const TransposedAt<RANK> wide_columns(lane, 256 * v);
+    const int rope_columns_low = (int)Narrow::Read::transposed(0, rope_block, lane);
+    const int rope_columns_high = (int)Narrow::Read::transposed(1, rope_block, lane);
+    f32x16 dq_acc[2][LATENT_BLOCKS], rope_acc;
+    bf16x8 held[2 * HELD];   // the column fragments of the key tile before the one in LDS (zero before the first)
     if constexpr (!SCORES) {
 #pragma unroll
-        for (int j = 0; j < BLOCKS; ++j) clear(dq_acc[j]);
+        for (int j = 0; j < LATENT_BLOCKS; ++j) {
+            clear(dq_acc[0][j]);
+            clear(dq_acc[1][j]);
+        }
+        clear(rope_acc);
 #pragma unroll
-        for (int f = 0; f < 2 * BLOCKS; ++f) held[f] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+        for (int f = 0; f < 2 * HELD; ++f) held[f] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
     }
 
     // (keys x rows) quadrants of 16 x 16, lane holds row l16 and keys 4*quad .. +3 of each key half.  A key fragment
@@ -461,29 +467,34 @@ __device__ __forceinline__ void query_gradient_walk(
         }
     };
 
-    // dQ^T += K^T dS^T: the held fragments (key tile t - 1) meet dS of that tile, and each gives way to the same
-    // fragment of tile t in `buffer`
+    // dQ^T += K^T dS^T: the held fragments (key tile t - 1) meet dS of that tile (of both row tiles), and each
+    // gives way to the same fragment of tile t in `buffer`
     auto add_tile = [&](const unsigned char* buffer, const unsigned char* exchange, bool any) {
         const unsigned char* k_latent = buffer + L::K_LATENT;
         const unsigned char* k_rope = buffer + L::K_ROPE;
-        bf16x8 dsf[2];
+        bf16x8 dsf[2][2];   // [row tile][16-key step]
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            dsf[n] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
-            if (any) dsf[n] = exchange_fragment(exchange, lq, g, n);
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                dsf[t][n] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+                if (any) dsf[t][n] = exchange_fragment(exchange + t * EXCHANGE_BYTES, lq, g, n);
+            }
         }
-        static_for<0, 2 * BLOCKS>([&](auto tag) {
+        static_for<0, 2 * HELD>([&](auto tag) {
             constexpr int I = decltype(tag)::value;
-            constexpr int N = I / BLOCKS;
-            constexpr int F = I % BLOCKS;
-            dq_acc[F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(held[I], dsf[N], dq_acc[F], 0, 0, 0);
+            constexpr int N = I / HELD;
+            constexpr int F = I % HELD;
             if constexpr (F < LATENT_BLOCKS) {
-                held[I] = transposed_fragment(k_latent, wide_columns.low[F % 4], wide_columns.high[F % 4],
-                                              N * 16 * Wide::ROW + 256 * (F / 4));
+                dq_acc[0][F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(held[I], dsf[0][N], dq_acc[0][F], 0, 0, 0);
+                dq_acc[1][F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(held[I], dsf[1][N], dq_acc[1][F], 0, 0, 0);
+                held[I] = transposed_fragment(k_latent, wide_columns.low[F], wide_columns.high[F], N * 16 * Wide::ROW);
             } else {
+                const bf16x8 own = rope_tile == 0 ? dsf[0][N] : dsf[1][N];
+                rope_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(held[I], own, rope_acc, 0, 0, 0);
                 held[I] = transposed_fragment(k_rope, rope_columns_low, rope_columns_high, N * 16 * Narrow::ROW);
             }
-            if constexpr (I % 4 == 0) request(std::integral_constant<int, I / 4>{});
+            if constexpr (I % 2 == 0) request(std::integral_constant<int, I / 2>{});
             __builtin_amdgcn_sched_barrier(0);
         });
     };
@@ -504,31 +515,33 @@ __device__ __forceinline__ void query_gradient_walk(
                            lds + L::EXCHANGE + parity * L::EXCHANGE_PAIR + (wave / 2) * EXCHANGE_BYTES, tile * TILE);
             }
         } else {
-            add_tile(lds + parity * L::BUFFER_BYTES,
-                     lds + L::EXCHANGE + (parity ^ 1) * L::EXCHANGE_PAIR + row_tile * EXCHANGE_BYTES, tile > 0);
+            add_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + (parity ^ 1) * L::EXCHANGE_PAIR, tile > 0);
         }
         wait_vector_memory<0>();
         workgroup_barrier();   // tile t has been read, its dS and tile t + 1 are in place
     }
 
-    // gradient waves: lane holds row lq of the row tile and columns 32*block + 8*(i/4) + 4*g + i%4
+    // gradient waves: lane holds row lq of a row tile and columns 32*block + 8*(i/4) + 4*g + i%4
     if constexpr (!SCORES) {
-        const long long row = row0 + TILE * row_tile + lq;
-        if (row < rows) {
-#pragma unroll
-            for (int j = 0; j < BLOCKS; ++j) {
+        auto store_block = [&](const f32x16& sums, long long row, bf16_t* gradient, int width, int column0) {
+            if (row < rows) {
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     u32x2 packed;
-                    packed.x = pack_bf16(dq_acc[j][4 * i4 + 0], dq_acc[j][4 * i4 + 1]);
-                    packed.y = pack_bf16(dq_acc[j][4 * i4 + 2], dq_acc[j][4 * i4 + 3]);
-                    bf16_t* destination = j < LATENT_BLOCKS
-                        ? query_latent_gradient + (batch_row0 + row) * RANK + 32 * (LATENT_BLOCKS * half + j) + 8 * i4 + 4 * g
-                        : query_rope_gradient + (batch_row0 + row) * ROPE + 32 * half + 8 * i4 + 4 * g;
-                    *reinterpret_cast<u32x2*>(destination) = packed;
+                    packed.x = pack_bf16(sums[4 * i4 + 0], sums[4 * i4 + 1]);
+                    packed.y = pack_bf16(sums[4 * i4 + 2], sums[4 * i4 + 3]);
+                    *reinterpret_cast<u32x2*>(gradient + (batch_row0 + row) * width + column0 + 8 * i4 + 4 * g) = packed;
                 }
             }
+        };
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int j = 0; j < LATENT_BLOCKS; ++j) {
+                store_block(dq_acc[t][j], row0 + TILE * t + lq, query_latent_gradient, RANK, 32 * (LATENT_BLOCKS * v + j));
+            }
         }
+        store_block(rope_acc, row0 + TILE * rope_tile + lq, query_rope_gradient, ROPE, 32 * rope_block);
     }
 }
 
