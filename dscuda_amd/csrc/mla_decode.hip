@@ -612,6 +612,10 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     // The first three units and the query rows.  In the middle of a kernel one round trip brings them all.  At the
     // start of the kernel (`cold`) every workgroup asks at once and the answers come at the rate of the memory, not
     // of its latency: then only what the first scores need is asked for first, the rest once that has arrived.
+    // The query rows are asked for before the page ids of the cursor, whose wait then covers both round trips
+    // (the ids are needed before the first unit can be requested; the rows before its scores).
+    bf16x8 qf[KSTEPS];
+    load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
     UnitCursor cursor;
     cursor.init(keys, unit_begin, last_token);
     if constexpr (PREFILL) cursor.contiguous = false;   // latent and rope parts come from tensors of their own
@@ -622,8 +626,6 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     const UnitSource second = cursor.next(lds, keys, last_token, wave, unit_end);
     const UnitSource third = cursor.next(lds, keys, last_token, wave, unit_end);
     if (!cold) issue_unit(second, offsets, keys, wave);
-    bf16x8 qf[KSTEPS];
-    load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
     if (!cold) issue_unit(third, offsets, keys, wave);
     reset(state);
     UnitReads reads;
@@ -769,6 +771,7 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     int own_workgroups, int own_whole) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ int own_prefix[SELF_PLAN_BATCH + 1];
+    __shared__ int own_lengths[SELF_PLAN_BATCH];   // saves the walk a round trip to memory for its sequence's length
     __shared__ int own_wave_totals[THREADS / 64];
 
     const int tid = threadIdx.x;
@@ -793,7 +796,9 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
     if (own_workgroups > 0) {
         whole_sequences = own_whole != 0;
         overhead = whole_sequences ? 0 : index_math::SEGMENT_OVERHEAD;
-        int value = tid < batch_size ? index_math::positions_of(tiles_of(cache_lengths[tid]), overhead) : 0;
+        const int own_length = tid < batch_size ? cache_lengths[tid] : 0;
+        own_lengths[tid] = own_length;
+        int value = tid < batch_size ? index_math::positions_of(tiles_of(own_length), overhead) : 0;
 #pragma unroll
         for (int offset = 1; offset < 64; offset <<= 1) {
             const int other = __shfl_up(value, offset);
@@ -883,7 +888,7 @@ __global__ __launch_bounds__(THREADS) void mla_decode_split_kernel(
             ++sequence;
             continue;
         }
-        const int tokens = cache_lengths[sequence];
+        const int tokens = own_workgroups > 0 ? __builtin_amdgcn_readfirstlane(own_lengths[sequence]) : cache_lengths[sequence];
         const bool whole = tile_begin == 0 && tile_end == sequence_end - sequence_begin - overhead;
         const bf16_t* query_row = query + ((size_t)sequence * heads + row) * WIDTH;
 

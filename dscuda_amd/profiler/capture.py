@@ -203,17 +203,28 @@ def write_environment(family, suite, profiles, commit, gate):
     try:
         result = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=60)
         # one block per agent: "Name:", "Marketing Name:", ..., "Device Type:"
-        found, name, marketing = [], "", ""
+        # (a GPU's "Compute Unit:" line follows its "Device Type:")
+        found, name, marketing, is_gpu = [], "", "", False
         for line in result.stdout.splitlines():
             text = line.strip()
             if text.startswith("Name:"):
-                name = text.split(":", 1)[1].strip()
+                name, is_gpu = text.split(":", 1)[1].strip(), False
             elif text.startswith("Marketing Name:"):
                 marketing = text.split(":", 1)[1].strip()
-            elif text.startswith("Device Type:") and "GPU" in text:
-                found.append(f"{marketing or 'unnamed'} ({name})")
+            elif text.startswith("Device Type:"):
+                is_gpu = "GPU" in text
+            elif text.startswith("Compute Unit:") and is_gpu:
+                found.append(f"{marketing or 'no marketing name'} ({name}, {text.split(':', 1)[1].strip()} compute units)")
+                is_gpu = False
         gpu = "; ".join(dict.fromkeys(found)) or "unavailable"
     except (OSError, subprocess.TimeoutExpired):
+        pass
+    try:
+        import torch
+        if torch.cuda.is_available():
+            properties = torch.cuda.get_device_properties(0)
+            gpu += f"; as PyTorch names device 0: {properties.name or 'no name'}, {properties.total_memory / 2 ** 30:.0f} GiB"
+    except Exception:   # noqa: BLE001 -- the record is written with or without it
         pass
     version_file = Path("/opt/rocm/.info/version")
     rocm = version_file.read_text().strip() if version_file.exists() else "unavailable"
