@@ -89,7 +89,11 @@ def test_backward_workload_3(cuda):
 
 @pytest.mark.parametrize("batch,tokens,heads", configs.MLA_TEST_PREFILL + configs.MLA_FULL_PREFILL + [(1, 96, 20), (1, 1024, 16),
                                                                                              (1, 256, 128), (2, 160, 128),
-                                                                                             (1, 33, 160), (2, 50, 1)])
+                                                                                             (1, 33, 160), (2, 50, 1),
+                                                                                             # row tiles that start and end inside
+                                                                                             # tokens, workgroups of one wave's rows
+                                                                                             (3, 33, 7), (1, 200, 2), (2, 64, 33),
+                                                                                             (1, 31, 64), (1, 97, 5), (1, 2, 48)])
 def test_absorbed_backward(cuda, batch, tokens, heads):
     """Shapes of benchmarks/mla.py:34-45; dO = 0.2 * N(0,1) as at :108; saved O (bf16) and LSE
     come from the oracle forward as at :68,113-117."""
