@@ -976,11 +976,24 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
         if (first == cut.intervals - 1) return;
         long long slot = batch * cut.items() + cut.items_before(first) + key_block;
         sum = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
-        for (int interval = first + 1; interval < cut.intervals; ++interval) {
-            slot += cut.blocks_in(interval - 1);
-            const f32x4 value = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
+        // eight parts per round trip, added in the order of the intervals (one at a time, a block with 64 parts
+        // waited for 64 round trips in a row)
+        constexpr int TOGETHER = 8;
+        for (int interval = first + 1; interval < cut.intervals; interval += TOGETHER) {
+            f32x4 value[TOGETHER];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sum[e] += value[e];
+            for (int j = 0; j < TOGETHER; ++j) {
+                value[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (interval + j < cut.intervals) {
+                    slot += cut.blocks_in(interval + j - 1);
+                    value[j] = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TOGETHER; ++j) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum[e] += value[j][e];
+            }
         }
     } else {
         const long long per_batch = visits.per_batch();
@@ -993,10 +1006,21 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
         const float* first_slot = partial_slots + (first_range + blockIdx.x) * PARTIAL_FLOATS + 4 * index;
         const int parts = (int)(last_range - first_range) + 1;
         sum = *reinterpret_cast<const f32x4*>(first_slot);
-        for (int part = 1; part < parts; ++part) {
-            const f32x4 value = *reinterpret_cast<const f32x4*>(first_slot + (long long)part * PARTIAL_FLOATS);
+        constexpr int TOGETHER = 8;
+        for (int part = 1; part < parts; part += TOGETHER) {
+            f32x4 value[TOGETHER];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sum[e] += value[e];
+            for (int j = 0; j < TOGETHER; ++j) {
+                value[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (part + j < parts) {
+                    value[j] = *reinterpret_cast<const f32x4*>(first_slot + (long long)(part + j) * PARTIAL_FLOATS);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TOGETHER; ++j) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum[e] += value[j][e];
+            }
         }
     }
     const int key = key_block * TILE + (4 * index) / WIDTH;
