@@ -40,7 +40,7 @@ def profiled_figures(stem, kernel_prefix):
         return None, None
     for line in path.read_text().splitlines():
         line = line.strip()
-        if line.startswith(kernel_prefix) and " :: " in line:
+        if line.startswith(kernel_prefix) and " :: time_us = " in line:   # not the counter lines of the same kernel
             fields = dict(part.strip().split(" = ") for part in line.split(" :: ", 1)[1].split(" ; "))
             nbytes = float(fields.get("fabric_bytes", fields.get("hbm_bytes", "nan")))
             return (None if nbytes != nbytes else nbytes), float(fields["time_us"])

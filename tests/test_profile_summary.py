@@ -66,3 +66,13 @@ def test_kernel_stats_table(tmp_path):
     lines = profile_summary.kernel_stats(path, ["dscuda"])
     assert len(lines) == 2
     assert lines[1].split()[-5:] == ["4", "650.0", "640.0", "700.0", "91.50"]
+
+
+def test_bench_reads_the_committed_forward_profile():
+    """bench.py takes roofline.traffic and profiled_kernel_ms from the forward's summary under profiles/: the line
+    it wants is the machine-readable one, not one of the counter lines that start with the same kernel name."""
+    import bench
+    traffic, microseconds = bench.profiled_figures("mla_prefill_forward_S4096_H128", "attention_forward_pingpong_kernel")
+    assert traffic is not None and 5e8 < traffic < 1e10
+    assert microseconds is not None and 300.0 < microseconds < 2000.0
+    assert bench.profiled_figures("no_such_case", "attention_forward_pingpong_kernel") == (None, None)
