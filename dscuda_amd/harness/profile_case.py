@@ -13,7 +13,9 @@ lengths ~ U[1024, 8192] seed 3), flash (B=1, H=8, S=512, D=64), absorbed (the
 reference's own prefill entry points, forward then backward, B=1, T=S, H heads,
 512 latent + 64 rope), projection (the W_UK absorb and W_UV un-absorb of S tokens x
 H heads), copy (a plain 16-byte-per-lane copy of 1 GiB, the calibration kernel for
-FETCH_SIZE / WRITE_SIZE).
+FETCH_SIZE / WRITE_SIZE).  ``--data zero`` fills every input with zeros: the kernels
+execute the same instructions, only the operands stop toggling, which separates what a
+workload loses to the chip's power limit (the clock it is given) from what its schedule loses.
 """
 
 from __future__ import annotations
@@ -33,6 +35,7 @@ def main():
     parser.add_argument("--steps", type=int, default=3)
     parser.add_argument("--seq", type=int, default=4096)
     parser.add_argument("--heads", type=int, default=128)
+    parser.add_argument("--data", choices=("random", "zero"), default="random")
     args = parser.parse_args()
 
     import torch
@@ -43,6 +46,8 @@ def main():
     generator = torch.Generator(device=device).manual_seed(1)
 
     def randn(shape, factor):
+        if args.data == "zero":
+            return torch.zeros(shape, device=device, dtype=torch.bfloat16)
         return (torch.randn(shape, device=device, generator=generator) * factor).bfloat16()
 
     if args.workload in ("forward", "backward"):

@@ -121,6 +121,11 @@ def metric_cases(suite):
             ["attention_forward"], "--seq", 16384)
         add("mla_prefill_backward_S16384_H128", "MLA prefill backward B=1 S=16384 H=128 192/128", "backward", 8, 4,
             ["attention_backward", "attention_key_value", "attention_query"], "--seq", 16384)
+        # the same launches on all-zero inputs: same instruction streams, operands that do not toggle
+        add("mla_prefill_forward_S4096_H128_zero_inputs", "MLA prefill forward B=1 S=4096 H=128 192/128, all inputs zero",
+            "forward", 160, 60, ["attention_forward"], "--data", "zero")
+        add("mla_prefill_backward_S4096_H128_zero_inputs", "MLA prefill backward B=1 S=4096 H=128 192/128, all inputs zero",
+            "backward", 80, 30, ["attention_backward", "attention_key_value", "attention_query"], "--data", "zero")
     return cases
 
 
