@@ -126,6 +126,8 @@ def metric_cases(suite):
             "forward", 160, 60, ["attention_forward"], "--data", "zero")
         add("mla_prefill_backward_S4096_H128_zero_inputs", "MLA prefill backward B=1 S=4096 H=128 192/128, all inputs zero",
             "backward", 80, 30, ["attention_backward", "attention_key_value", "attention_query"], "--data", "zero")
+        add("mla_decode_B64_H128_zero_inputs", "absorbed MLA decode B=64 H=128 lengths U[1024,8192] seed 3, query and cache zero",
+            "decode", 300, 100, ["mla_decode"], "--data", "zero")
     return cases
 
 
