@@ -726,6 +726,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attention_query_gradient_kernel(
 
     int bh, rank;
     xcd_order(blockIdx.x, gridDim.x / query_blocks, query_blocks, bh, rank);
+    // the heads in the reverse of the order in which the first pass wrote their dS blocks: what it wrote last is
+    // still in the memory-side cache
+    bh = gridDim.x / query_blocks - 1 - bh;
     const int jb = query_blocks - 1 - rank;   // heaviest (last) query blocks first
     const int local_pair = bh;                // position of this pair's dS blocks in the workspace
     bh += first_pair;
