@@ -261,11 +261,13 @@ constexpr int STREAM_RING = 6;                            // fragments read ahea
 static_assert(UNIT_LOADS * THREADS == UNIT * CHUNKS, "unit loads must divide evenly");
 
 struct UnitSource {
-    const bf16_t* base;      // first row of the unit (contiguous form only)
+    const bf16_t* base;      // first row of the unit (contiguous form; split form: of its latent part)
+    const bf16_t* rope_base; // split form: first row of the unit's rope part
     unsigned lds_base;       // LDS byte offset of this wave's 9 KB of the unit's slot
     int key0;
     int row_limit;           // rows above it repeat it (>= 0: the unit holds a visible token)
     bool contiguous;         // the unit is one run of rows: no paging, or pages that hold whole units
+    bool split;              // no paging, latent and rope parts in tensors of their own, offsets that fit 32 bits
     bool full;               // all 32 rows are visible tokens: the per-lane offsets are the same for every such unit
     bool enabled;
 };
@@ -285,6 +287,7 @@ struct UnitCursor {
     int ids;
     bool paged;
     bool contiguous;
+    bool split;
 
     // Waits for the ids on the spot (the empty asm statement is their first use): a wait left to the
     // first lane read would sit on the path of every step and wait for the unit requests as well.
@@ -297,6 +300,7 @@ struct UnitCursor {
     __device__ __forceinline__ void init(const KeyStream& keys, int first_unit, int last_token) {
         paged = keys.block_table != nullptr;
         contiguous = !paged || (keys.page_size % UNIT == 0);
+        split = false;
         unit = __builtin_amdgcn_readfirstlane(first_unit);
         page = within = units_per_page = first_page = last_page = ids = 0;
         if (paged && contiguous) {
@@ -312,6 +316,7 @@ struct UnitCursor {
                                                int unit_end) {
         UnitSource source;
         source.contiguous = contiguous;
+        source.split = split;
         source.enabled = unit < unit_end;
         source.key0 = unit * UNIT;
         source.row_limit = last_token - source.key0;
@@ -319,6 +324,11 @@ struct UnitCursor {
         source.lds_base = __builtin_amdgcn_readfirstlane(lds_offset_of(lds) + ((unsigned)unit % UNIT_SLOTS) * UNIT_BYTES +
                                                          wave * (UNIT_LOADS * 1024));
         source.base = keys.latent;
+        source.rope_base = keys.rope;
+        if (split) {
+            source.base = keys.latent + (size_t)source.key0 * keys.latent_stride;
+            source.rope_base = keys.rope + (size_t)source.key0 * keys.rope_stride;
+        }
         if (source.enabled && contiguous) {
             long long physical = source.key0;
             if (paged) {
@@ -359,6 +369,29 @@ __device__ __forceinline__ void issue_unit_load(const UnitSource& source, const 
     direct_load_16_offset_streaming(source.base, offset, source.lds_base + i * 1024);   // the cache is read once per call
 }
 
+// Load I of a unit whose latent and rope parts lie in tensors of their own, unpaged (`split`): a wave instruction
+// covers at most two rows of the unit (compile-time boundary), and a lane's 16 bytes come from the one tensor or the
+// other.  Row strides stay below 2^24 elements (the caller saw to that).
+template <int I>
+__device__ __forceinline__ void issue_split_load(const UnitSource& source, const KeyStream& keys, int wave, int lane) {
+    constexpr int FIRST_ROW = (64 * I) / CHUNKS;                 // of the wave's eight rows: the row of lane 0
+    constexpr int BOUNDARY = CHUNKS * (FIRST_ROW + 1) - 64 * I;   // first lane of the next row (64 or more: none)
+    // what depends on the row is the same for all lanes of a row: two candidates, wave-uniform
+    const int row = (UNIT / 4) * wave + FIRST_ROW;
+    const int swizzle[2] = {swizzle_of_row(row), swizzle_of_row(row + 1)};
+    const unsigned row_here[2] = {(unsigned)min(row, source.row_limit), (unsigned)min(row + 1, source.row_limit)};
+    const bool second = BOUNDARY < 64 && lane >= BOUNDARY;
+    const int position = lane + (64 * I - CHUNKS * FIRST_ROW) - (second ? CHUNKS : 0);
+    const int chunk = position ^ (second ? swizzle[1] : swizzle[0]);
+    const bool rope = chunk >= RANK / 8;
+    // bytes from the first row of the unit's part in the lane's tensor (the bases of the source hold key0 * stride)
+    const unsigned row_bytes = __umul24(second ? row_here[1] : row_here[0],
+                                        rope ? 2u * (unsigned)keys.rope_stride : 2u * (unsigned)keys.latent_stride);
+    const unsigned bytes = row_bytes + 16u * (unsigned)chunk - (rope ? 2u * RANK : 0u);
+    const unsigned char* part = reinterpret_cast<const unsigned char*>(rope ? source.rope_base : source.base);
+    direct_load_16(part + bytes, source.lds_base + I * 1024);
+}
+
 // All nine loads of a unit at once: the first units of a walk, and every unit of the
 // general form (per-lane page lookup, or latent and rope parts in tensors of their own).
 __device__ __forceinline__ void issue_unit(const UnitSource& source, const FullUnitOffsets& offsets, const KeyStream& keys,
@@ -368,6 +401,10 @@ __device__ __forceinline__ void issue_unit(const UnitSource& source, const FullU
     if (source.contiguous) {
 #pragma unroll
         for (int i = 0; i < UNIT_LOADS; ++i) issue_unit_load(source, offsets, wave, i, lane);
+        return;
+    }
+    if (source.split) {
+        unrolled<0, UNIT_LOADS>([&](auto tag) { issue_split_load<decltype(tag)::value>(source, keys, wave, lane); });
         return;
     }
     const bool paged = keys.block_table != nullptr;
@@ -567,7 +604,7 @@ __device__ __forceinline__ void unit_step(RowState& state, f32x16& scores, f32x1
     if constexpr (!HAS_NEXT) {
         unrolled<0, 33>(softmax_piece);   // the last unit: no score products to hide it behind
     }
-    if (request.enabled && !request.contiguous) issue_unit(request, offsets, keys, wave);
+    if (request.enabled && !request.contiguous && !request.split) issue_unit(request, offsets, keys, wave);
 
     unrolled<0, COUNT>([&](auto tag) {
         constexpr int I = decltype(tag)::value;
@@ -589,6 +626,7 @@ __device__ __forceinline__ void unit_step(RowState& state, f32x16& scores, f32x1
         // the requests go between the output MFMAs, which leave more issue slots free than the score MFMAs
         if constexpr (HAS_NEXT && I >= SCORE_MFMAS && (I - SCORE_MFMAS) % 3 == 1 && (I - SCORE_MFMAS) / 3 < UNIT_LOADS) {
             if (request.enabled && request.contiguous) issue_unit_load(request, offsets, wave, (I - SCORE_MFMAS) / 3, lane);
+            if (request.enabled && request.split) issue_split_load<(I - SCORE_MFMAS) / 3>(request, keys, wave, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
     });
@@ -618,7 +656,12 @@ __device__ __forceinline__ void walk_units(RowState& state, const bf16_t* query_
     load_query(qf, query_latent_row, query_rope_row, valid, (tid % 64) / 32);
     UnitCursor cursor;
     cursor.init(keys, unit_begin, last_token);
-    if constexpr (PREFILL) cursor.contiguous = false;   // latent and rope parts come from tensors of their own
+    if constexpr (PREFILL) {
+        cursor.contiguous = false;   // latent and rope parts come from tensors of their own
+        // 32 rows of a unit times the row stride, in bytes, as a 32-bit lane offset
+        cursor.split = keys.block_table == nullptr && keys.latent_stride < ((size_t)1 << 24) &&
+                       keys.rope_stride < ((size_t)1 << 24);
+    }
     const int visible = PREFILL ? row_tokens : tokens;   // keys the lane's row sees
     FullUnitOffsets offsets;
     offsets.init(wave, fresh_lane_id());
