@@ -268,11 +268,13 @@ struct KeyVisits {
     }
 };
 
-DSCUDA_HOST_DEVICE inline KeyVisits key_visits(int sequence_length, int heads) {
+// `key_tiles`: key blocks of 32 * key_tiles keys.  Such a block is seen from the tile of row 32 * key_tiles * kb * heads
+// on, which is what blocks of 32 keys and key_tiles * heads heads give: `heads` holds that product.
+DSCUDA_HOST_DEVICE inline KeyVisits key_visits(int sequence_length, int heads, int key_tiles = 1) {
     KeyVisits visits;
-    visits.key_blocks = (sequence_length + 31) / 32;
+    visits.key_blocks = (sequence_length + 32 * key_tiles - 1) / (32 * key_tiles);
     visits.row_tiles = (int)(((long long)sequence_length * heads + 31) / 32);
-    visits.heads = heads;
+    visits.heads = heads * key_tiles;
     return visits;
 }
 
@@ -324,11 +326,11 @@ struct KeyIntervals {
     }
 };
 
-DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int heads, int length) {
+DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int heads, int length, int key_tiles = 1) {
     KeyIntervals cut;
     cut.length = length;
-    cut.heads = heads;
-    cut.key_blocks = (sequence_length + 31) / 32;
+    cut.heads = heads * key_tiles;   // as in key_visits
+    cut.key_blocks = (sequence_length + 32 * key_tiles - 1) / (32 * key_tiles);
     cut.row_tiles = (int)(((long long)sequence_length * heads + 31) / 32);
     cut.intervals = (cut.row_tiles + length - 1) / length;
     return cut;

@@ -954,6 +954,408 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
     }
 }
 
+// ---- key gradients of inputs that outgrow the caches: 64 keys per workgroup ------
+//
+// There the kernel above is bound by what it moves: a row tile of 68 KB meets 32 keys, one tile in flight, drained at
+// every barrier.  This one holds 64 keys, so every row fetched does twice the work, and keeps two requests of rows in
+// flight across the barriers.  The gradient sums of 64 keys fill 288 registers of a gradient wave, which leaves no room
+// to hold a tile's column fragments back; instead the rows come in half tiles of 16 that stay in LDS for four steps:
+//
+//     step h:   half tile h is scored (waves 0, 1)  |  half tile h - 1 is multiplied into the sums (waves 2, 3)
+//               half tiles h + 1 and h + 2 are arriving (h + 2 requested during this step)
+//
+// Four buffers of 16 rows take the room of the two 32-row buffers above.  A wave waits at the end of step h until at most
+// the requests it issued during that step are outstanding, i.e. for its share of half tile h + 1.
+// Score wave w takes all 16 rows against keys 32w .. 32w + 31 (the keys as register operands, each row fragment feeds
+// both halves of them); gradient wave 2 + c holds, for all 64 keys, column blocks 8c .. 8c + 7 of the latent part:
+// every column fragment it reads feeds two products.  Those are 256 registers of sums, all the accumulation registers
+// a wave has (with more the compiler moves sums between the two register files inside the loop and waits for every
+// product it moves), so the rope columns are summed by the score waves, which have registers to spare: wave w
+// multiplies dS of its own 32 keys, read back from the exchange tile it wrote them to, with the two rope column
+// blocks, one step later.
+struct KeyPairLayout {
+    static constexpr int HALF_ROWS = 16;
+    static constexpr int KEYS = 64;
+    static constexpr int Q_LATENT = 0;                                          // [16 rows][512]
+    static constexpr int DO_ROWS = Q_LATENT + HALF_ROWS * Tile32<RANK>::ROW;    // [16 rows][512]
+    static constexpr int Q_ROPE = DO_ROWS + HALF_ROWS * Tile32<RANK>::ROW;      // [16 rows][64]
+    static constexpr int STATS = Q_ROPE + HALF_ROWS * Tile32<ROPE>::ROW;        // [16] lse, [16] delta, [16] token
+    static constexpr int BUFFER_BYTES = STATS + 3 * HALF_ROWS * 4;
+    static constexpr int BUFFERS = 4;
+    static constexpr int EXCHANGE = BUFFERS * BUFFER_BYTES;
+    static constexpr int PITCH = 2 * HALF_ROWS + 8;          // of a key's 16 values: 8-byte accesses of 32 lanes fall into different banks
+    static constexpr int EXCHANGE_PART = KEYS * PITCH;       // P (or dS) of a half tile: [64 keys][16 rows]
+    static constexpr int EXCHANGE_PAIR = 2 * EXCHANGE_PART;
+    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_PAIR;   // of the half tile being scored and the one before
+};
+static_assert(KeyPairLayout::BUFFER_BYTES % 16 == 0 && KeyPairLayout::LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
+
+template <bool SCORES>
+__device__ __forceinline__ void key_pair_walk(
+    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
+    const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
+    const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
+    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
+    int interval_length, float scale) {
+    using L = KeyPairLayout;
+    using Wide = Tile32<RANK>;
+    using Narrow = Tile32<ROPE>;
+    constexpr int Q_STEPS = WIDTH / 32;    // 18
+    constexpr int O_STEPS = RANK / 32;     // 16
+    constexpr int AHEAD = 6;
+    constexpr int LATENT_BLOCKS = 8;       // per gradient wave
+    constexpr int FRAGMENTS = 2 * LATENT_BLOCKS;       // column fragments of a half tile per gradient wave
+    constexpr int ROWS_PER_WAVE = L::HALF_ROWS / 4;
+    constexpr int KEY_TILES = L::KEYS / TILE;
+    // per wave and half tile: four rows of the two wide tiles, then one more request (waves 0, 1: half of the rope
+    // tile; wave 2: the rows' log-sum-exp and delta; wave 3: none)
+    constexpr int REQUESTS = 2 * ROWS_PER_WAVE + 1;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int tid = threadIdx.x;
+    __builtin_assume(tid >= 0 && tid < THREADS);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int lane = tid % 64;
+    const int lq = lane % 32;
+    const int g = lane / 32;
+    const int T = sequence_length;
+    const long long rows = (long long)T * heads;
+    const float c = scale * LOG2E;
+    const int half = wave % 2;             // score waves: keys 32*half .. +31; gradient waves: column blocks 8*half .. +7, 16 + half
+    const int l16 = lane % 16;
+    const int quad = lane / 16;
+    const QuadrantAt<RANK> wide_quadrant(lane, 0);
+    const QuadrantAt<ROPE> narrow_quadrant(lane, 0);
+    const TransposedAt<RANK> wide_columns(lane, 512 * half);
+    const TransposedAt<ROPE> rope_columns(lane, 0);
+
+    const unsigned lds_base = lds_offset_of(lds);
+    unsigned wide_part[ROWS_PER_WAVE];
+#pragma unroll
+    for (int j = 0; j < ROWS_PER_WAVE; ++j) {
+        wide_part[j] = 16u * (unsigned)(lane ^ index_math::tile_swizzle<Wide::ROW>(ROWS_PER_WAVE * wave + j));
+    }
+    const int narrow_row = 8 * half + lane / 8;
+    const unsigned narrow_part = 16u * (unsigned)((lane % 8) ^ index_math::tile_swizzle<Narrow::ROW>(narrow_row));
+
+    // the workgroup's item: the tiles of one key block inside one interval
+    const index_math::KeyVisits visits = index_math::key_visits(T, heads, KEY_TILES);
+    const index_math::KeyIntervals cut = index_math::key_intervals(T, heads, interval_length, KEY_TILES);
+    const long long items = cut.items();
+    const long long item = blockIdx.x;
+    const int batch = (int)(item / items);
+    int interval, key_block;
+    cut.locate(item - batch * items, interval, key_block);
+    const int first_tile = max(interval * interval_length, visits.first_tile(key_block));
+    const int end_tile = cut.end_of(interval);
+    const bool whole = first_tile == visits.first_tile(key_block) && end_tile == visits.row_tiles;
+
+    const int k0 = key_block * L::KEYS;
+    const long long batch_row0 = (long long)batch * rows;
+    const bf16_t* ql = query_latent + batch_row0 * RANK;
+    const bf16_t* qr = query_rope + batch_row0 * ROPE;
+    const bf16_t* dout = output_gradient + batch_row0 * RANK;
+    const bf16_t* latent = kv_latent + (size_t)batch * T * RANK;
+    const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
+    const float* lse_batch = logsumexp + (size_t)batch * heads * T;
+
+    // score waves: the wave's keys as B operands (column = key 32*half + 16*kh + l16)
+    bf16x8 kf[2][Q_STEPS];
+    if constexpr (SCORES) {
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
+            const int own_key = k0 + 32 * half + 16 * kh + l16;
+            const size_t k = own_key < T ? own_key : 0;
+            fetch_quadrant_operand(kf[kh], latent + k * RANK, rope + k * ROPE, own_key < T, quad);
+        }
+    }
+    f32x16 latent_acc[KEY_TILES][LATENT_BLOCKS];   // gradient waves
+    f32x16 rope_acc[ROPE / 32];                    // score waves: keys 32*half .. +31
+    if constexpr (SCORES) {
+#pragma unroll
+        for (int b = 0; b < ROPE / 32; ++b) clear(rope_acc[b]);
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < KEY_TILES; ++kt) {
+#pragma unroll
+            for (int j = 0; j < LATENT_BLOCKS; ++j) clear(latent_acc[kt][j]);
+        }
+    }
+
+    // Half tile u holds rows 16u .. 16u + 15.  One past the last row of the batch element (the second half of a
+    // last tile of at most 16 rows) is requested as the half tile before it, with tokens of -1: such rows see no key.
+    const int last_half_tile = (int)((rows - 1) / L::HALF_ROWS);
+    struct {
+        const bf16_t* latent;
+        const bf16_t* gradient;
+        const bf16_t* rope;
+        int last_valid;     // rows past it repeat it
+        unsigned buffer;
+    } arriving;
+    auto begin_requests = [&](int half_tile, int buffer) {
+        const int fetched = min(half_tile, last_half_tile);
+        const long long row0 = (long long)fetched * L::HALF_ROWS;
+        arriving.latent = ql + row0 * RANK;
+        arriving.gradient = dout + row0 * RANK;
+        arriving.rope = qr + row0 * ROPE;
+        arriving.last_valid = (int)min(rows - row0, (long long)L::HALF_ROWS) - 1;
+        arriving.buffer = lds_base + buffer * L::BUFFER_BYTES;
+        if constexpr (!SCORES) {
+            if (wave == 2 && lane < 2 * L::HALF_ROWS) {
+                // the statistics of its rows: lanes 0 .. 15 bring the log-sum-exp, lanes 16 .. 31 the delta, straight
+                // into LDS (a load into registers would make the compiler wait for the requests issued after it)
+                const int r = min(lane % L::HALF_ROWS, arriving.last_valid);
+                int token, head;
+                if (rows <= 0x7fffffffLL) {
+                    const unsigned row = (unsigned)row0 + (unsigned)r;
+                    token = (int)(row / (unsigned)heads);
+                    head = (int)(row % (unsigned)heads);
+                } else {
+                    token = (int)((row0 + r) / heads);
+                    head = (int)((row0 + r) % heads);
+                }
+                const float* source = lane < L::HALF_ROWS ? lse_batch + (size_t)head * T + token
+                                                          : delta_of_rows + (batch_row0 + row0 + r) * DELTA_STRIDE;
+                direct_load_4(source, arriving.buffer + L::STATS);
+                if (lane < L::HALF_ROWS) {
+                    const bool exists = fetched == half_tile && lane <= arriving.last_valid;
+                    reinterpret_cast<int*>(lds + buffer * L::BUFFER_BYTES + L::STATS)[2 * L::HALF_ROWS + lane] = exists ? token : -1;
+                }
+            }
+        }
+    };
+    auto request = [&](auto tag) {
+        constexpr int R = decltype(tag)::value;
+        if constexpr (R < 2 * ROWS_PER_WAVE) {
+            constexpr int J = R / 2;
+            const int row = ROWS_PER_WAVE * wave + J;
+            const unsigned source = wide_part[J] + (unsigned)(min(row, arriving.last_valid) * Wide::ROW);
+            if constexpr (R % 2 == 0) {
+                direct_load_16_offset(arriving.latent, source, arriving.buffer + L::Q_LATENT + row * Wide::ROW);
+            } else {
+                direct_load_16_offset(arriving.gradient, source, arriving.buffer + L::DO_ROWS + row * Wide::ROW);
+            }
+        } else if constexpr (R == 2 * ROWS_PER_WAVE && SCORES) {
+            direct_load_16_offset(arriving.rope, narrow_part + (unsigned)(min(narrow_row, arriving.last_valid) * Narrow::ROW),
+                                  arriving.buffer + L::Q_ROPE + 8 * half * Narrow::ROW);
+        }
+    };
+    // until the wave's requests of the steps before this one have arrived
+    auto await_earlier_requests = [&]() {
+        if (wave == 3) wait_vector_memory<REQUESTS - 1>(); else wait_vector_memory<REQUESTS>();
+    };
+
+    // scores of a half tile: (rows x keys) blocks of 16 x 16, lane holds key 32*half + 16*kh + l16 and rows 4*quad .. +3
+    auto score_half_tile = [&](const unsigned char* buffer, unsigned char* exchange) {
+        const unsigned char* q_latent = buffer + L::Q_LATENT;
+        const unsigned char* q_rope = buffer + L::Q_ROPE;
+        const unsigned char* do_rows = buffer + L::DO_ROWS;
+        const float* lse_of = reinterpret_cast<const float*>(buffer + L::STATS);
+        const float* delta = lse_of + L::HALF_ROWS;
+        const int* token_of = reinterpret_cast<const int*>(delta + L::HALF_ROWS);
+        f32x4 s_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        f32x4 dp_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        bf16x8 ring[AHEAD];
+        auto row_fragment = [&](auto tag) {
+            constexpr int I = decltype(tag)::value;
+            if constexpr (I >= 2 * O_STEPS) {
+                return quadrant_fragment<I - 2 * O_STEPS>(q_rope, narrow_quadrant);
+            } else if constexpr (I % 2 == 0) {
+                return quadrant_fragment<I / 2>(q_latent, wide_quadrant);
+            } else {
+                return quadrant_fragment<I / 2>(do_rows, wide_quadrant);
+            }
+        };
+        fill_ring(ring, row_fragment);
+        fragment_stream<Q_STEPS + O_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int I = decltype(tag)::value;
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                if constexpr (I >= 2 * O_STEPS) {
+                    s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I - O_STEPS], s_acc[kh], 0, 0, 0);
+                } else if constexpr (I % 2 == 0) {
+                    s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], s_acc[kh], 0, 0, 0);
+                } else {
+                    dp_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], dp_acc[kh], 0, 0, 0);
+                }
+            }
+            if constexpr (I % 4 == 0) request(std::integral_constant<int, I / 4>{});
+        });
+        const int local = 4 * quad;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_of + local);
+        const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
+        const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
+            const int key = 32 * half + 16 * kh + l16;
+            float p[4], ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[kh][i], c, -lse4[i] * LOG2E));
+                if (k0 + key > (int)token4[i]) probability = 0.f;
+                p[i] = probability;
+                ds[i] = probability * (dp_acc[kh][i] - delta4[i]) * scale;
+            }
+            u32x2 packed;
+            packed.x = pack_bf16(p[0], p[1]);
+            packed.y = pack_bf16(p[2], p[3]);
+            *reinterpret_cast<u32x2*>(exchange + key * L::PITCH + 2 * local) = packed;          // [key][row]
+            packed.x = pack_bf16(ds[0], ds[1]);
+            packed.y = pack_bf16(ds[2], ds[3]);
+            *reinterpret_cast<u32x2*>(exchange + L::EXCHANGE_PART + key * L::PITCH + 2 * local) = packed;
+        }
+    };
+
+    // the rope columns of the half tile scored one step before: dS of the wave's keys (lane: key 32*half + lq, rows
+    // {4g .. +3, 8 + 4g .. +3}) times the two rope column blocks
+    auto add_rope = [&](const unsigned char* buffer, const unsigned char* exchange) {
+        const unsigned char* at = exchange + L::EXCHANGE_PART + (32 * half + lq) * L::PITCH + 2 * (4 * g);
+        const u32x2 ds_low = *reinterpret_cast<const u32x2*>(at);
+        const u32x2 ds_high = *reinterpret_cast<const u32x2*>(at + 16);
+        const bf16x8 dsf = __builtin_bit_cast(bf16x8, u32x4{ds_low.x, ds_low.y, ds_high.x, ds_high.y});
+#pragma unroll
+        for (int b = 0; b < ROPE / 32; ++b) {
+            const bf16x8 fragment = transposed_fragment(buffer + L::Q_ROPE, rope_columns.low[b], rope_columns.high[b], 0);
+            rope_acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf, fragment, rope_acc[b], 0, 0, 0);
+        }
+    };
+
+    // A gradient wave's step: the column fragments of a half tile (its eight latent blocks of the query rows with dS,
+    // its eight blocks of the dO rows with P), both key halves one after the other: neighbouring products go to
+    // different sums.
+    auto add_half_tile = [&](const unsigned char* buffer, const unsigned char* exchange) {
+        const unsigned char* q_latent = buffer + L::Q_LATENT;
+        const unsigned char* do_rows = buffer + L::DO_ROWS;
+        bf16x8 pf[KEY_TILES], dsf[KEY_TILES];
+#pragma unroll
+        for (int kt = 0; kt < KEY_TILES; ++kt) {
+            // lane: key 32*kt + lq, rows {4g .. +3, 8 + 4g .. +3}
+            const unsigned char* at = exchange + (32 * kt + lq) * L::PITCH + 2 * (4 * g);
+            const u32x2 p_low = *reinterpret_cast<const u32x2*>(at);
+            const u32x2 p_high = *reinterpret_cast<const u32x2*>(at + 16);
+            const u32x2 ds_low = *reinterpret_cast<const u32x2*>(at + L::EXCHANGE_PART);
+            const u32x2 ds_high = *reinterpret_cast<const u32x2*>(at + L::EXCHANGE_PART + 16);
+            pf[kt] = __builtin_bit_cast(bf16x8, u32x4{p_low.x, p_low.y, p_high.x, p_high.y});
+            dsf[kt] = __builtin_bit_cast(bf16x8, u32x4{ds_low.x, ds_low.y, ds_high.x, ds_high.y});
+        }
+        bf16x8 ring[AHEAD];
+        auto column_fragment = [&](auto tag) {
+            constexpr int F = decltype(tag)::value;
+            if constexpr (F < LATENT_BLOCKS) {
+                return transposed_fragment(q_latent, wide_columns.low[F % 4], wide_columns.high[F % 4], 256 * (F / 4));
+            } else {
+                constexpr int J = F - LATENT_BLOCKS;
+                return transposed_fragment(do_rows, wide_columns.low[J % 4], wide_columns.high[J % 4], 256 * (J / 4));
+            }
+        };
+        fill_ring(ring, column_fragment);
+        fragment_stream<FRAGMENTS>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int F = decltype(tag)::value;
+#pragma unroll
+            for (int kt = 0; kt < KEY_TILES; ++kt) {
+                if constexpr (F < LATENT_BLOCKS) {
+                    latent_acc[kt][F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[kt], fragment, latent_acc[kt][F], 0, 0, 0);
+                } else {
+                    constexpr int J = F - LATENT_BLOCKS;
+                    latent_acc[kt][J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[kt], fragment, latent_acc[kt][J], 0, 0, 0);
+                }
+            }
+            if constexpr (F % 2 == 0) request(std::integral_constant<int, F / 2>{});
+        });
+    };
+
+    // half tiles first .. first + count - 1; one more step lets the gradient waves catch up
+    const int first = 2 * first_tile;
+    const int count = 2 * (end_tile - first_tile);
+    begin_requests(first, 0);
+    static_for<0, REQUESTS>(request);
+    begin_requests(first + 1, 1);
+    static_for<0, REQUESTS>(request);
+    wait_vector_memory<0>();
+    workgroup_barrier();
+
+    for (int h = 0; h <= count; ++h) {
+        // past the item's last half tile that one is requested again, into a buffer nobody reads: the streams stay
+        // free of branches
+        begin_requests(first + min(h + 2, count - 1), (h + 2) % L::BUFFERS);
+        if constexpr (SCORES) {
+            if (h > 0) {
+                add_rope(lds + ((h - 1) % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + ((h - 1) & 1) * L::EXCHANGE_PAIR);
+            }
+            if (h < count) {
+                score_half_tile(lds + (h % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + (h & 1) * L::EXCHANGE_PAIR);
+            }
+        } else {
+            if (h > 0) {
+                add_half_tile(lds + ((h - 1) % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + ((h - 1) & 1) * L::EXCHANGE_PAIR);
+            } else {
+                static_for<0, REQUESTS>(request);
+            }
+        }
+        await_earlier_requests();
+        workgroup_barrier();   // half tile h has been scored, h - 1 read for the last time, h + 1 has arrived
+    }
+    wait_vector_memory<0>();
+
+    // lane holds column (block, lq) and keys (first of the 32) + 8*(i/4) + 4*g + i%4: the gradient waves of both key
+    // halves and their eight latent blocks, score wave w of keys 32w .. +31 and the two rope blocks
+    float* slot = partial_slots + item * (KEY_TILES * PARTIAL_FLOATS);   // [64 keys][576]
+    if constexpr (SCORES) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = 32 * half + 8 * (i / 4) + 4 * g + i % 4;
+            if (whole) {
+                if (k0 + key < T) {
+                    __bf16* rope_row = reinterpret_cast<__bf16*>(key_rope_gradient) + ((size_t)batch * T + k0 + key) * ROPE;
+#pragma unroll
+                    for (int b = 0; b < ROPE / 32; ++b) rope_row[32 * b + lq] = (__bf16)rope_acc[b][i];
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < ROPE / 32; ++b) slot[key * WIDTH + RANK + 32 * b + lq] = rope_acc[b][i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < KEY_TILES; ++kt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = TILE * kt + 8 * (i / 4) + 4 * g + i % 4;
+                if (whole) {
+                    if (k0 + key < T) {
+                        __bf16* latent_row = reinterpret_cast<__bf16*>(kv_latent_gradient) + ((size_t)batch * T + k0 + key) * RANK;
+#pragma unroll
+                        for (int j = 0; j < LATENT_BLOCKS; ++j) {
+                            latent_row[32 * (LATENT_BLOCKS * half + j) + lq] = (__bf16)latent_acc[kt][j][i];
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < LATENT_BLOCKS; ++j) {
+                        slot[key * WIDTH + 32 * (LATENT_BLOCKS * half + j) + lq] = latent_acc[kt][j][i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(THREADS) void mla_absorbed_key_pair_gradient_kernel(
+    bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient, float* __restrict__ partial_slots,
+    const float* __restrict__ delta_of_rows, const bf16_t* __restrict__ output_gradient,
+    const float* __restrict__ logsumexp, const bf16_t* __restrict__ query_latent, const bf16_t* __restrict__ query_rope,
+    const bf16_t* __restrict__ kv_latent, const bf16_t* __restrict__ key_rope, int sequence_length, int heads,
+    int interval_length, float scale) {
+    if (threadIdx.x < THREADS / 2) {
+        key_pair_walk<true>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient, logsumexp,
+                            query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
+    } else {
+        key_pair_walk<false>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient, logsumexp,
+                             query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
+    }
+}
+
 // Sums the partial key gradients of every key block whose visits were cut, in range (or interval) order.  Workgroup (x, y)
 // takes the y-th 1/REDUCTION_PARTS of key block x (numbered through the batch elements), a thread four
 // neighbouring columns of one key; a block that one range held whole wrote its gradients itself.
@@ -963,19 +1365,21 @@ static_assert(REDUCTION_PARTS * THREADS * 4 == PARTIAL_FLOATS, "slot size");
 __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
     bf16_t* __restrict__ kv_latent_gradient, bf16_t* __restrict__ key_rope_gradient,
     const float* __restrict__ partial_slots, int sequence_length, int heads, int batch_size, int ranges,
-    int interval_length) {
-    const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
+    int interval_length, int key_tiles) {
+    // key blocks and slots of 32 * key_tiles keys, blockIdx.y up to REDUCTION_PARTS * key_tiles
+    const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads, key_tiles);
+    const long long slot_floats = (long long)key_tiles * PARTIAL_FLOATS;
     const int batch = blockIdx.x / visits.key_blocks;
     const int key_block = blockIdx.x % visits.key_blocks;
     const int index = blockIdx.y * THREADS + threadIdx.x;   // which four floats of the slot
     f32x4 sum;
     if (interval_length > 0) {
         // the block's items: one per interval from the one its first tile lies in, slot = item number
-        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, interval_length);
+        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, interval_length, key_tiles);
         const int first = cut.first_interval(key_block);
         if (first == cut.intervals - 1) return;
         long long slot = batch * cut.items() + cut.items_before(first) + key_block;
-        sum = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
+        sum = *reinterpret_cast<const f32x4*>(partial_slots + slot * slot_floats + 4 * index);
         // eight parts per round trip, added in the order of the intervals (one at a time, a block with 64 parts
         // waited for 64 round trips in a row)
         constexpr int TOGETHER = 8;
@@ -986,7 +1390,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
                 value[j] = f32x4{0.f, 0.f, 0.f, 0.f};
                 if (interval + j < cut.intervals) {
                     slot += cut.blocks_in(interval + j - 1);
-                    value[j] = *reinterpret_cast<const f32x4*>(partial_slots + slot * PARTIAL_FLOATS + 4 * index);
+                    value[j] = *reinterpret_cast<const f32x4*>(partial_slots + slot * slot_floats + 4 * index);
                 }
             }
 #pragma unroll
@@ -1003,7 +1407,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
         const long long first_range = index_math::wide_range_of(total, ranges, begin);
         const long long last_range = index_math::wide_range_of(total, ranges, end - 1);
         if (first_range == last_range) return;
-        const float* first_slot = partial_slots + (first_range + blockIdx.x) * PARTIAL_FLOATS + 4 * index;
+        const float* first_slot = partial_slots + (first_range + blockIdx.x) * slot_floats + 4 * index;
         const int parts = (int)(last_range - first_range) + 1;
         sum = *reinterpret_cast<const f32x4*>(first_slot);
         constexpr int TOGETHER = 8;
@@ -1013,7 +1417,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
             for (int j = 0; j < TOGETHER; ++j) {
                 value[j] = f32x4{0.f, 0.f, 0.f, 0.f};
                 if (part + j < parts) {
-                    value[j] = *reinterpret_cast<const f32x4*>(first_slot + (long long)(part + j) * PARTIAL_FLOATS);
+                    value[j] = *reinterpret_cast<const f32x4*>(first_slot + (long long)(part + j) * slot_floats);
                 }
             }
 #pragma unroll
@@ -1023,7 +1427,7 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_reduction_kernel(
             }
         }
     }
-    const int key = key_block * TILE + (4 * index) / WIDTH;
+    const int key = key_block * TILE * key_tiles + (4 * index) / WIDTH;
     const int column = (4 * index) % WIDTH;
     if (key < sequence_length) {
         u32x2 packed;
@@ -1082,27 +1486,33 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
     prepared.run([] {
         raise_lds_limit(mla_absorbed_query_gradient_kernel, QueryGradLayout::LDS_BYTES);
         raise_lds_limit(mla_absorbed_key_gradient_kernel, KeyGradLayout::LDS_BYTES);
+        raise_lds_limit(mla_absorbed_key_pair_gradient_kernel, KeyPairLayout::LDS_BYTES);
     });
     // scratch memory until the last launch: delta in the rope query gradients, partial key gradients in the latent ones
     float* delta = reinterpret_cast<float*>(query_rope_gradient);
     float* partial_slots = reinterpret_cast<float*>(query_latent_gradient);
     const index_math::KeyVisits visits = index_math::key_visits(sequence_length, heads);
-    const long long blocks = (long long)visits.key_blocks * batch_size;
+    long long blocks = (long long)visits.key_blocks * batch_size;
     const long long total = visits.per_batch() * batch_size;
     const long long scratch_bytes = rows * batch_size * RANK * 2;
     // Rows that outgrow the caches (query and dO rows of a batch element, 2176 bytes per row): the interval cut
+    // with key blocks of 64 keys (mla_absorbed_key_pair_gradient_kernel)
+    constexpr int PAIR = KeyPairLayout::KEYS / TILE;
     int interval_length = 0;
+    int key_tiles = 1;
     long long grid = 0;
     const int forced = forced_interval_tiles();
     if (forced > 0 || rows * (2 * RANK + ROPE) * 2 > LARGE_INPUT_BYTES) {
         const int tiles = forced > 0 ? forced : INTERVAL_TILES;
-        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles);
+        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles, PAIR);
         const long long items = cut.items() * batch_size;
         // enough items to keep every compute unit busy through several rounds, and a slot for each
-        if ((forced > 0 || items >= 4LL * device_compute_units()) && items <= scratch_bytes / index_math::KEY_PARTIAL_BYTES &&
-            items <= 0x7fffffffLL) {
+        if ((forced > 0 || items >= 4LL * device_compute_units()) &&
+            items <= scratch_bytes / (PAIR * index_math::KEY_PARTIAL_BYTES) && items <= 0x7fffffffLL) {
             interval_length = tiles;
+            key_tiles = PAIR;
             grid = items;
+            blocks = (long long)cut.key_blocks * batch_size;
         }
     }
     long long ranges = 0;
@@ -1114,15 +1524,22 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
     hipLaunchKernelGGL(mla_absorbed_row_statistics_kernel, dim3((unsigned)(row_blocks * batch_size)), dim3(THREADS), 0,
                        stream, delta, output_gradient, output, rows * batch_size);
     HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)grid), dim3(THREADS), KeyGradLayout::LDS_BYTES,
-                       stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta, output_gradient, logsumexp,
-                       query_latent, query_rope, kv_latent, key_rope, batch_size, sequence_length, heads, (int)ranges,
-                       interval_length, scale);
+    if (interval_length > 0) {
+        hipLaunchKernelGGL(mla_absorbed_key_pair_gradient_kernel, dim3((unsigned)grid), dim3(THREADS),
+                           KeyPairLayout::LDS_BYTES, stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta,
+                           output_gradient, logsumexp, query_latent, query_rope, kv_latent, key_rope, sequence_length,
+                           heads, interval_length, scale);
+    } else {
+        hipLaunchKernelGGL(mla_absorbed_key_gradient_kernel, dim3((unsigned)grid), dim3(THREADS), KeyGradLayout::LDS_BYTES,
+                           stream, kv_latent_gradient, key_rope_gradient, partial_slots, delta, output_gradient, logsumexp,
+                           query_latent, query_rope, kv_latent, key_rope, batch_size, sequence_length, heads, (int)ranges,
+                           0, scale);
+    }
     HIP_CHECK(hipGetLastError());
     if (ranges > 0 || interval_length > 0) {
-        hipLaunchKernelGGL(mla_absorbed_key_reduction_kernel, dim3((unsigned)blocks, REDUCTION_PARTS), dim3(THREADS), 0,
-                           stream, kv_latent_gradient, key_rope_gradient, partial_slots, sequence_length, heads,
-                           batch_size, (int)ranges, interval_length);
+        hipLaunchKernelGGL(mla_absorbed_key_reduction_kernel, dim3((unsigned)blocks, REDUCTION_PARTS * key_tiles),
+                           dim3(THREADS), 0, stream, kv_latent_gradient, key_rope_gradient, partial_slots, sequence_length,
+                           heads, batch_size, (int)ranges, interval_length, key_tiles);
         HIP_CHECK(hipGetLastError());
     }
     const long long query_blocks = (rows + QUERY_ROWS - 1) / QUERY_ROWS;

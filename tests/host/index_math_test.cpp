@@ -350,10 +350,15 @@ void check_key_intervals() {
     for (int heads : {1, 3, 8, 16, 128}) {
         for (int tokens : {1, 33, 257, 512, 1000}) {
             if ((long long)heads * tokens > 70000) continue;
-            for (int length : {1, 2, 7, 64, 100000}) {
-                const KeyIntervals cut = key_intervals(tokens, heads, length);
-                const KeyVisits visits = key_visits(tokens, heads);
+            for (int length : {1, 2, 7, 64, 100000}) for (int key_tiles : {1, 2}) {
+                const KeyIntervals cut = key_intervals(tokens, heads, length, key_tiles);
+                const KeyVisits visits = key_visits(tokens, heads, key_tiles);
                 EXPECT(cut.key_blocks == visits.key_blocks && cut.row_tiles == visits.row_tiles, "counts");
+                EXPECT(cut.key_blocks == (tokens + 32 * key_tiles - 1) / (32 * key_tiles), "key blocks");
+                for (int kb = 0; kb < cut.key_blocks; ++kb) {
+                    // the first tile that holds a row of the block's first token
+                    EXPECT(visits.first_tile(kb) == (int)((long long)32 * key_tiles * kb * heads / 32), "first tile");
+                }
                 std::vector<int> seen((size_t)cut.key_blocks * cut.row_tiles, 0), parts(cut.key_blocks, 0);
                 long long item = 0;
                 for (int i = 0; i < cut.intervals; ++i) {
