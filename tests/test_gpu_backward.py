@@ -167,6 +167,9 @@ def test_backward_in_chunks_of_pairs(cuda, batch, seq, heads, budget_pairs, expe
     (2, 160, 128, 100),   # two batch elements, a short last interval, interval ends inside key blocks
     (1, 512, 8, 7),       # many short intervals
     (2, 257, 4, 1000),    # one interval: every key block whole
+    (1, 95, 3, 4),        # 285 rows: the last half tile of 16 rows holds 13
+    (1, 50, 1, 1),        # 50 rows: the last row tile holds 18, its second half tile two; one key block, cut in two
+    (3, 77, 5, 3),        # 385 rows: one row in the last tile, whose second half tile is past the end
 ])
 def test_absorbed_backward_interval_cut(cuda, batch, tokens, heads, interval_tiles):
     """The cut of the key gradients for inputs that outgrow the caches (items of one interval of row tiles and one
