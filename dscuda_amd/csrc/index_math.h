@@ -338,6 +338,26 @@ DSCUDA_HOST_DEVICE inline KeyIntervals key_intervals(int sequence_length, int he
 
 constexpr long long KEY_PARTIAL_BYTES = 32LL * 576 * 4;   // one slot: [32 keys][576] fp32
 
+// Interval length (row tiles) of the cut into items: the shortest of the ladder 24, 32, 48, 64, 96, ... whose items,
+// over `batch` batch elements, number at most twelve rounds of the compute units and have a slot each (shorter
+// intervals give more, shorter items: a fuller last round, as long as the slots last).  0: even that many items
+// are fewer than two rounds, or no length of the ladder fits; equal ranges balance the units better then.
+DSCUDA_HOST_DEVICE inline int key_interval_choice(int sequence_length, int heads, long long batch, long long slots,
+                                                  int compute_units, int key_tiles) {
+    const long long rounds = 12LL * compute_units;
+    const long long most = rounds < slots ? rounds : slots;
+    const long long row_tiles = ((long long)sequence_length * heads + 31) / 32;
+    for (long long base = 8; ; base *= 2) {
+        for (int multiple = 3; multiple <= 4; ++multiple) {
+            const long long tiles = base * multiple;
+            if (tiles >= (1 << 24)) return 0;
+            const long long items = key_intervals(sequence_length, heads, (int)tiles, key_tiles).items() * batch;
+            if (items <= most) return items >= 2LL * compute_units ? (int)tiles : 0;
+            if (tiles >= row_tiles) return 0;
+        }
+    }
+}
+
 // How many ranges the list is cut into when `scratch_bytes` are there for the slots: one per compute unit if the
 // slots allow.  0: every key block is one range and writes its result itself (too few slots for a cut whose
 // longest range is shorter than the longest key block, `row_tiles` visits).

@@ -1447,7 +1447,6 @@ void raise_lds_limit(Kernel kernel, int bytes) {
 }
 
 constexpr long long LARGE_INPUT_BYTES = 64LL << 20;   // per batch element, against 32 MB of L2 and 256 MB behind it
-constexpr int INTERVAL_TILES = 192;                   // 13 MB of rows; T=4096, H=128: 2 795 items, 8.13 ms against 8.64 with 256 (2 080 items, the last round a ninth full)
 
 // mla_absorbed_backward_set_key_interval_tiles (> 0) forces the interval cut with that many row tiles per interval at
 // any size the slots allow; 0 gives the choice back to the dispatch below.
@@ -1503,12 +1502,14 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
     long long grid = 0;
     const int forced = forced_interval_tiles();
     if (forced > 0 || rows * (2 * RANK + ROPE) * 2 > LARGE_INPUT_BYTES) {
-        const int tiles = forced > 0 ? forced : INTERVAL_TILES;
-        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles, PAIR);
+        const long long slots = scratch_bytes / (PAIR * index_math::KEY_PARTIAL_BYTES);
+        const int tiles = forced > 0 ? forced
+                                     : index_math::key_interval_choice(sequence_length, heads, batch_size, slots,
+                                                                       device_compute_units(), PAIR);
+        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles > 0 ? tiles : 1, PAIR);
         const long long items = cut.items() * batch_size;
-        // enough items to keep every compute unit busy through several rounds, and a slot for each
-        if ((forced > 0 || items >= 4LL * device_compute_units()) &&
-            items <= scratch_bytes / (PAIR * index_math::KEY_PARTIAL_BYTES) && items <= 0x7fffffffLL) {
+        // a slot for each item
+        if (tiles > 0 && items <= slots && items <= 0x7fffffffLL) {
             interval_length = tiles;
             key_tiles = PAIR;
             grid = items;

@@ -387,6 +387,34 @@ void check_key_intervals() {
     }
 }
 
+// the interval length the dispatch picks by itself: known cases at 256 compute units (slots = rows * batch * 1024 bytes
+// over 147456), and the bounds it promises wherever it picks one
+void check_key_interval_choice() {
+    struct { int tokens, heads, batch, expected; } known[] = {
+        {4096, 128, 1, 192}, {2048, 128, 1, 96}, {1024, 128, 1, 48}, {512, 128, 1, 0}, {8192, 32, 1, 384},
+        {2048, 16, 1, 0}, {4096, 128, 2, 384}, {16384, 16, 1, 768}, {1024, 128, 4, 48}, {300, 128, 8, 24}, {300, 128, 5, 24},
+    };
+    for (const auto& c : known) {
+        const long long slots = (long long)c.tokens * c.heads * c.batch * 1024 / (2 * KEY_PARTIAL_BYTES);
+        const int tiles = key_interval_choice(c.tokens, c.heads, c.batch, slots, 256, 2);
+        EXPECT(tiles == c.expected, "interval choice T=%d H=%d B=%d: %d, expected %d", c.tokens, c.heads, c.batch, tiles, c.expected);
+    }
+    for (int heads : {1, 8, 16, 128}) {
+        for (int tokens : {64, 1000, 4096, 20000}) {
+            for (int batch : {1, 3}) {
+                for (int units : {8, 256}) {
+                    const long long slots = (long long)tokens * heads * batch * 1024 / (2 * KEY_PARTIAL_BYTES);
+                    const int tiles = key_interval_choice(tokens, heads, batch, slots, units, 2);
+                    if (tiles == 0) continue;
+                    const long long items = key_intervals(tokens, heads, tiles, 2).items() * batch;
+                    EXPECT(items <= slots && items <= 12LL * units && items >= 2LL * units, "items %lld of T=%d H=%d B=%d units %d", items,
+                           tokens, heads, batch, units);
+                }
+            }
+        }
+    }
+}
+
 // ---- decode: the ranges partition the list of positions, their lengths differ by at most one, every tile of every
 // sequence is computed by exactly one range, and (range, sequence) pairs that hold part of a sequence own distinct slots
 void check_decode_ranges() {
@@ -530,6 +558,7 @@ int main() {
     check_decode_loads<32>();
     check_key_visits();
     check_key_intervals();
+    check_key_interval_choice();
     check_decode_ranges();
     check_decode_layout();
     if (failures) {

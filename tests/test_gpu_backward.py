@@ -181,6 +181,13 @@ def test_absorbed_backward_interval_cut(cuda, batch, tokens, heads, interval_til
         ops.mla_backward_set_key_interval_tiles(0)
 
 
+def test_absorbed_backward_interval_cut_chosen_by_the_library(cuda):
+    """B=5, T=300, H=128: 38 400 rows of 2176 bytes per batch element are above the library's own bound for the
+    interval cut, and on 256 compute units it cuts into intervals of 24 row tiles (725 items; the choice itself is
+    pinned on the host, tests/host/index_math_test.cpp)."""
+    _absorbed_case(cuda, 5, 300, 128, seed=79, dout_factor=0.05)
+
+
 def test_backward_workspace_is_bounded(cuda):
     """Workload 5 (S=16384, H=128) asks for less than 4 GiB; workload 3 still fits one launch."""
     long_case = ops.mla_prefill_backward_workspace_elements(1, 16384, 128, 192, 128)
