@@ -159,14 +159,6 @@ __device__ __forceinline__ void direct_load_16(const void* source, unsigned lds_
                  : "memory", "m0");
 }
 
-// four bytes per lane: lane l's value lands at lds_base + 4 * l (lanes switched off leave their place alone)
-__device__ __forceinline__ void direct_load_4(const void* source, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
-                 :
-                 : "v"(source), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
-}
-
 // source = uniform 64-bit base + per-lane 32-bit byte offset; lds_base wave-uniform
 __device__ __forceinline__ void direct_load_16_offset(const void* uniform_base, unsigned byte_offset, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"

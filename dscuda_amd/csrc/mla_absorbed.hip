@@ -956,39 +956,30 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_gradient_kernel(
 
 // ---- key gradients of inputs that outgrow the caches: 64 keys per workgroup ------
 //
-// There the kernel above is bound by what it moves: a row tile of 68 KB meets 32 keys, one tile in flight, drained at
-// every barrier.  This one holds 64 keys, so every row fetched does twice the work, and keeps two requests of rows in
-// flight across the barriers.  The gradient sums of 64 keys fill 288 registers of a gradient wave, which leaves no room
-// to hold a tile's column fragments back; instead the rows come in half tiles of 16 that stay in LDS for four steps:
-//
-//     step h:   half tile h is scored (waves 0, 1)  |  half tile h - 1 is multiplied into the sums (waves 2, 3)
-//               half tiles h + 1 and h + 2 are arriving (h + 2 requested during this step)
-//
-// Four buffers of 16 rows take the room of the two 32-row buffers above.  A wave waits at the end of step h until at most
-// the requests it issued during that step are outstanding, i.e. for its share of half tile h + 1.
-// Score wave w takes all 16 rows against keys 32w .. 32w + 31 (the keys as register operands, each row fragment feeds
-// both halves of them); gradient wave 2 + c holds, for all 64 keys, column blocks 8c .. 8c + 7 of the latent part:
-// every column fragment it reads feeds two products.  Those are 256 registers of sums, all the accumulation registers
-// a wave has (with more the compiler moves sums between the two register files inside the loop and waits for every
-// product it moves), so the rope columns are summed by the score waves, which have registers to spare: wave w
-// multiplies dS of its own 32 keys, read back from the exchange tile it wrote them to, with the two rope column
-// blocks, one step later.
+// There the kernel above is bound by what it moves: a row tile of 68 KB meets 32 keys.  This one has the same layout
+// (score waves, gradient waves one tile behind that hold the tile's column fragments in registers, two 32-row
+// buffers, one barrier a step) with 64 keys, so every row fetched does twice the work and a step carries twice the
+// products for the same barrier, first reads and wait for the rows.  The gradient waves hold the latent sums of all
+// 64 keys, 256 registers: all the accumulation registers a wave has (with more the compiler keeps sums in both
+// register files and moves them inside the loop, waiting for every product it moves), besides 128 registers of held
+// fragments.  The rope columns are therefore summed by the score waves.  Score wave w takes all 32 rows against keys
+// 32w .. 32w + 31 (the keys as register operands, 144 registers; with the rows split instead each wave would hold all
+// 64 keys, 288, and spill), so dS of its keys over the whole tile are its own: it reads them back from the exchange
+// tile behind its own stores, which the LDS keeps in order, and multiplies them with the rope column blocks.
+// Only the interval cut uses it: a workgroup walks one item.
 struct KeyPairLayout {
-    static constexpr int HALF_ROWS = 16;
     static constexpr int KEYS = 64;
-    static constexpr int Q_LATENT = 0;                                          // [16 rows][512]
-    static constexpr int DO_ROWS = Q_LATENT + HALF_ROWS * Tile32<RANK>::ROW;    // [16 rows][512]
-    static constexpr int Q_ROPE = DO_ROWS + HALF_ROWS * Tile32<RANK>::ROW;      // [16 rows][64]
-    static constexpr int STATS = Q_ROPE + HALF_ROWS * Tile32<ROPE>::ROW;        // [16] lse, [16] delta, [16] token
-    static constexpr int BUFFER_BYTES = STATS + 3 * HALF_ROWS * 4;
-    static constexpr int BUFFERS = 4;
-    static constexpr int EXCHANGE = BUFFERS * BUFFER_BYTES;
-    static constexpr int PITCH = 2 * HALF_ROWS + 8;          // of a key's 16 values: 8-byte accesses of 32 lanes fall into different banks
-    static constexpr int EXCHANGE_PART = KEYS * PITCH;       // P (or dS) of a half tile: [64 keys][16 rows]
+    static constexpr int Q_LATENT = 0;                                   // [32 rows][512]
+    static constexpr int DO_ROWS = Q_LATENT + Tile32<RANK>::BYTES;       // [32 rows][512]
+    static constexpr int Q_ROPE = DO_ROWS + Tile32<RANK>::BYTES;         // [32 rows][64]
+    static constexpr int STATS = Q_ROPE + Tile32<ROPE>::BYTES;
+    static constexpr int BUFFER_BYTES = STATS + 3 * TILE * 4;
+    static constexpr int EXCHANGE = 2 * BUFFER_BYTES;                    // the tile in use and the one arriving
+    static constexpr int EXCHANGE_PART = (KEYS / TILE) * EXCHANGE_BYTES; // P (or dS) of a tile: [64 keys][32 rows]
     static constexpr int EXCHANGE_PAIR = 2 * EXCHANGE_PART;
-    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_PAIR;   // of the half tile being scored and the one before
+    static constexpr int LDS_BYTES = EXCHANGE + 2 * EXCHANGE_PAIR;       // of the tile being scored and the one before
 };
-static_assert(KeyPairLayout::BUFFER_BYTES % 16 == 0 && KeyPairLayout::LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
+static_assert(KeyPairLayout::LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
 
 template <bool SCORES>
 __device__ __forceinline__ void key_pair_walk(
@@ -1003,12 +994,10 @@ __device__ __forceinline__ void key_pair_walk(
     constexpr int Q_STEPS = WIDTH / 32;    // 18
     constexpr int O_STEPS = RANK / 32;     // 16
     constexpr int AHEAD = 6;
-    constexpr int LATENT_BLOCKS = 8;       // per gradient wave
-    constexpr int FRAGMENTS = 2 * LATENT_BLOCKS;       // column fragments of a half tile per gradient wave
-    constexpr int ROWS_PER_WAVE = L::HALF_ROWS / 4;
     constexpr int KEY_TILES = L::KEYS / TILE;
-    // per wave and half tile: four rows of the two wide tiles, then one more request (waves 0, 1: half of the rope
-    // tile; wave 2: the rows' log-sum-exp and delta; wave 3: none)
+    constexpr int LATENT_BLOCKS = 8;       // per gradient wave
+    constexpr int PER_STEP = 2 * LATENT_BLOCKS;   // column fragments per 16-row step of a gradient wave
+    constexpr int ROWS_PER_WAVE = TILE / 4;
     constexpr int REQUESTS = 2 * ROWS_PER_WAVE + 1;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -1022,7 +1011,7 @@ __device__ __forceinline__ void key_pair_walk(
     const int T = sequence_length;
     const long long rows = (long long)T * heads;
     const float c = scale * LOG2E;
-    const int half = wave % 2;             // score waves: keys 32*half .. +31; gradient waves: column blocks 8*half .. +7, 16 + half
+    const int half = wave % 2;             // score waves: keys 32*half .. +31; gradient waves: column blocks 8*half .. +7
     const int l16 = lane % 16;
     const int quad = lane / 16;
     const QuadrantAt<RANK> wide_quadrant(lane, 0);
@@ -1036,7 +1025,7 @@ __device__ __forceinline__ void key_pair_walk(
     for (int j = 0; j < ROWS_PER_WAVE; ++j) {
         wide_part[j] = 16u * (unsigned)(lane ^ index_math::tile_swizzle<Wide::ROW>(ROWS_PER_WAVE * wave + j));
     }
-    const int narrow_row = 8 * half + lane / 8;
+    const int narrow_row = ROWS_PER_WAVE * wave + lane / 8;
     const unsigned narrow_part = 16u * (unsigned)((lane % 8) ^ index_math::tile_swizzle<Narrow::ROW>(narrow_row));
 
     // the workgroup's item: the tiles of one key block inside one interval
@@ -1060,8 +1049,9 @@ __device__ __forceinline__ void key_pair_walk(
     const bf16_t* rope = key_rope + (size_t)batch * T * ROPE;
     const float* lse_batch = logsumexp + (size_t)batch * heads * T;
 
-    // score waves: the wave's keys as B operands (column = key 32*half + 16*kh + l16)
+    // score waves: the wave's 32 keys as B operands (column = key 32*half + 16*kh + l16), and their rope sums
     bf16x8 kf[2][Q_STEPS];
+    f32x16 rope_acc[ROPE / 32];
     if constexpr (SCORES) {
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) {
@@ -1069,43 +1059,43 @@ __device__ __forceinline__ void key_pair_walk(
             const size_t k = own_key < T ? own_key : 0;
             fetch_quadrant_operand(kf[kh], latent + k * RANK, rope + k * ROPE, own_key < T, quad);
         }
-    }
-    f32x16 latent_acc[KEY_TILES][LATENT_BLOCKS];   // gradient waves
-    f32x16 rope_acc[ROPE / 32];                    // score waves: keys 32*half .. +31
-    if constexpr (SCORES) {
 #pragma unroll
         for (int b = 0; b < ROPE / 32; ++b) clear(rope_acc[b]);
-    } else {
+    }
+    // gradient waves: latent column blocks 8*half + j of both key tiles, and the column fragments of the tile before
+    // the one in LDS (zero before the first: its products add nothing)
+    f32x16 latent_acc[KEY_TILES][LATENT_BLOCKS];
+    bf16x8 held[2 * PER_STEP];
+    if constexpr (!SCORES) {
 #pragma unroll
         for (int kt = 0; kt < KEY_TILES; ++kt) {
 #pragma unroll
             for (int j = 0; j < LATENT_BLOCKS; ++j) clear(latent_acc[kt][j]);
         }
+#pragma unroll
+        for (int f = 0; f < 2 * PER_STEP; ++f) held[f] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
     }
 
-    // Half tile u holds rows 16u .. 16u + 15.  One past the last row of the batch element (the second half of a
-    // last tile of at most 16 rows) is requested as the half tile before it, with tokens of -1: such rows see no key.
-    const int last_half_tile = (int)((rows - 1) / L::HALF_ROWS);
     struct {
         const bf16_t* latent;
         const bf16_t* gradient;
         const bf16_t* rope;
-        int last_valid;     // rows past it repeat it
+        int last_valid;
         unsigned buffer;
     } arriving;
-    auto begin_requests = [&](int half_tile, int buffer) {
-        const int fetched = min(half_tile, last_half_tile);
-        const long long row0 = (long long)fetched * L::HALF_ROWS;
+    RowStatistics statistics = {0.f, 0.f, -1};
+    auto begin_requests = [&](int tile, int parity) {
+        const long long row0 = (long long)tile * TILE;
         arriving.latent = ql + row0 * RANK;
         arriving.gradient = dout + row0 * RANK;
         arriving.rope = qr + row0 * ROPE;
-        arriving.last_valid = (int)min(rows - row0, (long long)L::HALF_ROWS) - 1;
-        arriving.buffer = lds_base + buffer * L::BUFFER_BYTES;
-        if constexpr (!SCORES) {
-            if (wave == 2 && lane < 2 * L::HALF_ROWS) {
-                // the statistics of its rows: lanes 0 .. 15 bring the log-sum-exp, lanes 16 .. 31 the delta, straight
-                // into LDS (a load into registers would make the compiler wait for the requests issued after it)
-                const int r = min(lane % L::HALF_ROWS, arriving.last_valid);
+        arriving.last_valid = (int)min(rows - row0, (long long)TILE) - 1;
+        arriving.buffer = lds_base + parity * L::BUFFER_BYTES;
+        // the statistics of its rows: one lane per row, in a gradient wave (the score waves have more to do)
+        if (tid >= 2 * 64 && tid < 2 * 64 + TILE) {
+            const int r = tid - 2 * 64;
+            statistics = {0.f, 0.f, -1};
+            if (r <= arriving.last_valid) {
                 int token, head;
                 if (rows <= 0x7fffffffLL) {
                     const unsigned row = (unsigned)row0 + (unsigned)r;
@@ -1115,13 +1105,9 @@ __device__ __forceinline__ void key_pair_walk(
                     token = (int)((row0 + r) / heads);
                     head = (int)((row0 + r) % heads);
                 }
-                const float* source = lane < L::HALF_ROWS ? lse_batch + (size_t)head * T + token
-                                                          : delta_of_rows + (batch_row0 + row0 + r) * DELTA_STRIDE;
-                direct_load_4(source, arriving.buffer + L::STATS);
-                if (lane < L::HALF_ROWS) {
-                    const bool exists = fetched == half_tile && lane <= arriving.last_valid;
-                    reinterpret_cast<int*>(lds + buffer * L::BUFFER_BYTES + L::STATS)[2 * L::HALF_ROWS + lane] = exists ? token : -1;
-                }
+                statistics.lse = lse_batch[(size_t)head * T + token];
+                statistics.delta = delta_of_rows[(batch_row0 + row0 + r) * DELTA_STRIDE];
+                statistics.token = token;
             }
         }
     };
@@ -1136,175 +1122,182 @@ __device__ __forceinline__ void key_pair_walk(
             } else {
                 direct_load_16_offset(arriving.gradient, source, arriving.buffer + L::DO_ROWS + row * Wide::ROW);
             }
-        } else if constexpr (R == 2 * ROWS_PER_WAVE && SCORES) {
+        } else if constexpr (R == 2 * ROWS_PER_WAVE) {
             direct_load_16_offset(arriving.rope, narrow_part + (unsigned)(min(narrow_row, arriving.last_valid) * Narrow::ROW),
-                                  arriving.buffer + L::Q_ROPE + 8 * half * Narrow::ROW);
+                                  arriving.buffer + L::Q_ROPE + ROWS_PER_WAVE * wave * Narrow::ROW);
         }
     };
-    // until the wave's requests of the steps before this one have arrived
-    auto await_earlier_requests = [&]() {
-        if (wave == 3) wait_vector_memory<REQUESTS - 1>(); else wait_vector_memory<REQUESTS>();
+    auto place_statistics = [&](int parity) {
+        if (tid >= 2 * 64 && tid < 2 * 64 + TILE) {
+            const int r = tid - 2 * 64;
+            float* lse2 = reinterpret_cast<float*>(lds + parity * L::BUFFER_BYTES + L::STATS);
+            lse2[r] = statistics.lse * LOG2E;
+            lse2[TILE + r] = statistics.delta;
+            reinterpret_cast<int*>(lse2)[2 * TILE + r] = statistics.token;
+        }
     };
 
-    // scores of a half tile: (rows x keys) blocks of 16 x 16, lane holds key 32*half + 16*kh + l16 and rows 4*quad .. +3
-    auto score_half_tile = [&](const unsigned char* buffer, unsigned char* exchange) {
+    // scores of one tile: (rows x keys) blocks of 16 x 16, lane holds key 32*half + 16*kh + l16 and rows 16*r + 4*quad .. +3;
+    // the two halves of the rows one after the other, every row fragment serves both key blocks
+    auto score_tile = [&](const unsigned char* buffer, unsigned char* exchange) {
         const unsigned char* q_latent = buffer + L::Q_LATENT;
         const unsigned char* q_rope = buffer + L::Q_ROPE;
         const unsigned char* do_rows = buffer + L::DO_ROWS;
-        const float* lse_of = reinterpret_cast<const float*>(buffer + L::STATS);
-        const float* delta = lse_of + L::HALF_ROWS;
-        const int* token_of = reinterpret_cast<const int*>(delta + L::HALF_ROWS);
-        f32x4 s_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-        f32x4 dp_acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        const float* lse2 = reinterpret_cast<const float*>(buffer + L::STATS);
+        const float* delta = lse2 + TILE;
+        const int* token_of = reinterpret_cast<const int*>(delta + TILE);
+        f32x4 s_acc[2][2], dp_acc[2][2];   // [half of the rows][key block]
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) s_acc[r][kh] = dp_acc[r][kh] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        constexpr int PER_HALF = Q_STEPS + O_STEPS;
         bf16x8 ring[AHEAD];
         auto row_fragment = [&](auto tag) {
-            constexpr int I = decltype(tag)::value;
+            constexpr int R = decltype(tag)::value / PER_HALF;
+            constexpr int I = decltype(tag)::value % PER_HALF;
             if constexpr (I >= 2 * O_STEPS) {
-                return quadrant_fragment<I - 2 * O_STEPS>(q_rope, narrow_quadrant);
+                return quadrant_fragment<I - 2 * O_STEPS>(q_rope + R * 16 * Narrow::ROW, narrow_quadrant);
             } else if constexpr (I % 2 == 0) {
-                return quadrant_fragment<I / 2>(q_latent, wide_quadrant);
+                return quadrant_fragment<I / 2>(q_latent + R * 16 * Wide::ROW, wide_quadrant);
             } else {
-                return quadrant_fragment<I / 2>(do_rows, wide_quadrant);
+                return quadrant_fragment<I / 2>(do_rows + R * 16 * Wide::ROW, wide_quadrant);
             }
         };
         fill_ring(ring, row_fragment);
-        fragment_stream<Q_STEPS + O_STEPS>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
-            constexpr int I = decltype(tag)::value;
+        fragment_stream<2 * PER_HALF>(ring, row_fragment, [&](auto tag, const bf16x8& fragment) {
+            constexpr int R = decltype(tag)::value / PER_HALF;
+            constexpr int I = decltype(tag)::value % PER_HALF;
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh) {
                 if constexpr (I >= 2 * O_STEPS) {
-                    s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I - O_STEPS], s_acc[kh], 0, 0, 0);
+                    s_acc[R][kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I - O_STEPS], s_acc[R][kh], 0, 0, 0);
                 } else if constexpr (I % 2 == 0) {
-                    s_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], s_acc[kh], 0, 0, 0);
+                    s_acc[R][kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], s_acc[R][kh], 0, 0, 0);
                 } else {
-                    dp_acc[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], dp_acc[kh], 0, 0, 0);
+                    dp_acc[R][kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fragment, kf[kh][I / 2], dp_acc[R][kh], 0, 0, 0);
                 }
             }
-            if constexpr (I % 4 == 0) request(std::integral_constant<int, I / 4>{});
+            if constexpr (decltype(tag)::value % 4 == 0) request(std::integral_constant<int, decltype(tag)::value / 4>{});
         });
-        const int local = 4 * quad;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_of + local);
-        const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
-        const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+        // the rope columns of the tile's rows, for the rope products below
+        bf16x8 rope_columns_of_rows[2][ROPE / 32];
 #pragma unroll
-        for (int kh = 0; kh < 2; ++kh) {
-            const int key = 32 * half + 16 * kh + l16;
-            float p[4], ds[4];
+        for (int n = 0; n < 2; ++n) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[kh][i], c, -lse4[i] * LOG2E));
-                if (k0 + key > (int)token4[i]) probability = 0.f;
-                p[i] = probability;
-                ds[i] = probability * (dp_acc[kh][i] - delta4[i]) * scale;
+            for (int b = 0; b < ROPE / 32; ++b) {
+                rope_columns_of_rows[n][b] = transposed_fragment(q_rope, rope_columns.low[b], rope_columns.high[b], n * 16 * Narrow::ROW);
             }
-            u32x2 packed;
-            packed.x = pack_bf16(p[0], p[1]);
-            packed.y = pack_bf16(p[2], p[3]);
-            *reinterpret_cast<u32x2*>(exchange + key * L::PITCH + 2 * local) = packed;          // [key][row]
-            packed.x = pack_bf16(ds[0], ds[1]);
-            packed.y = pack_bf16(ds[2], ds[3]);
-            *reinterpret_cast<u32x2*>(exchange + L::EXCHANGE_PART + key * L::PITCH + 2 * local) = packed;
         }
-    };
-
-    // the rope columns of the half tile scored one step before: dS of the wave's keys (lane: key 32*half + lq, rows
-    // {4g .. +3, 8 + 4g .. +3}) times the two rope column blocks
-    auto add_rope = [&](const unsigned char* buffer, const unsigned char* exchange) {
-        const unsigned char* at = exchange + L::EXCHANGE_PART + (32 * half + lq) * L::PITCH + 2 * (4 * g);
-        const u32x2 ds_low = *reinterpret_cast<const u32x2*>(at);
-        const u32x2 ds_high = *reinterpret_cast<const u32x2*>(at + 16);
-        const bf16x8 dsf = __builtin_bit_cast(bf16x8, u32x4{ds_low.x, ds_low.y, ds_high.x, ds_high.y});
 #pragma unroll
-        for (int b = 0; b < ROPE / 32; ++b) {
-            const bf16x8 fragment = transposed_fragment(buffer + L::Q_ROPE, rope_columns.low[b], rope_columns.high[b], 0);
-            rope_acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf, fragment, rope_acc[b], 0, 0, 0);
+        for (int r = 0; r < 2; ++r) {
+            const int local = 16 * r + 4 * quad;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse2 + local);
+            const f32x4 delta4 = *reinterpret_cast<const f32x4*>(delta + local);
+            const u32x4 token4 = *reinterpret_cast<const u32x4*>(token_of + local);
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                const int own_key = k0 + 32 * half + 16 * kh + l16;
+                float p[4], ds[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float probability = __builtin_amdgcn_exp2f(fmaf(s_acc[r][kh][i], c, -lse4[i]));
+                    if (own_key > (int)token4[i]) probability = 0.f;
+                    p[i] = probability;
+                    ds[i] = probability * (dp_acc[r][kh][i] - delta4[i]) * scale;
+                }
+                // [key][row], the wave's 32 keys are one part of EXCHANGE_BYTES
+                exchange_store(exchange + half * EXCHANGE_BYTES, 16 * kh + l16, local, p);
+                exchange_store(exchange + L::EXCHANGE_PART + half * EXCHANGE_BYTES, 16 * kh + l16, local, ds);
+            }
+        }
+        // dK_rope += dS^T Q_rope for the wave's keys: their dS of all 32 rows were written by this wave
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const bf16x8 gradient = exchange_fragment(exchange + L::EXCHANGE_PART + half * EXCHANGE_BYTES, lq, g, n);
+#pragma unroll
+            for (int b = 0; b < ROPE / 32; ++b) {
+                rope_acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gradient, rope_columns_of_rows[n][b], rope_acc[b], 0, 0, 0);
+            }
         }
     };
 
-    // A gradient wave's step: the column fragments of a half tile (its eight latent blocks of the query rows with dS,
-    // its eight blocks of the dO rows with P), both key halves one after the other: neighbouring products go to
-    // different sums.
-    auto add_half_tile = [&](const unsigned char* buffer, const unsigned char* exchange) {
+    // One step of a gradient wave: the held fragments (tile t - 1) meet P and dS of that tile, both key tiles one after
+    // the other, and each gives way to the same fragment of tile t in `buffer`.  Per 16-row step n: the query columns
+    // of the wave's eight latent blocks (with dS), then the dO columns of the same blocks (with P).
+    auto add_tile = [&](const unsigned char* buffer, const unsigned char* exchange, bool any) {
         const unsigned char* q_latent = buffer + L::Q_LATENT;
         const unsigned char* do_rows = buffer + L::DO_ROWS;
-        bf16x8 pf[KEY_TILES], dsf[KEY_TILES];
+        bf16x8 pf[KEY_TILES][2], dsf[KEY_TILES][2];
 #pragma unroll
         for (int kt = 0; kt < KEY_TILES; ++kt) {
-            // lane: key 32*kt + lq, rows {4g .. +3, 8 + 4g .. +3}
-            const unsigned char* at = exchange + (32 * kt + lq) * L::PITCH + 2 * (4 * g);
-            const u32x2 p_low = *reinterpret_cast<const u32x2*>(at);
-            const u32x2 p_high = *reinterpret_cast<const u32x2*>(at + 16);
-            const u32x2 ds_low = *reinterpret_cast<const u32x2*>(at + L::EXCHANGE_PART);
-            const u32x2 ds_high = *reinterpret_cast<const u32x2*>(at + L::EXCHANGE_PART + 16);
-            pf[kt] = __builtin_bit_cast(bf16x8, u32x4{p_low.x, p_low.y, p_high.x, p_high.y});
-            dsf[kt] = __builtin_bit_cast(bf16x8, u32x4{ds_low.x, ds_low.y, ds_high.x, ds_high.y});
-        }
-        bf16x8 ring[AHEAD];
-        auto column_fragment = [&](auto tag) {
-            constexpr int F = decltype(tag)::value;
-            if constexpr (F < LATENT_BLOCKS) {
-                return transposed_fragment(q_latent, wide_columns.low[F % 4], wide_columns.high[F % 4], 256 * (F / 4));
-            } else {
-                constexpr int J = F - LATENT_BLOCKS;
-                return transposed_fragment(do_rows, wide_columns.low[J % 4], wide_columns.high[J % 4], 256 * (J / 4));
-            }
-        };
-        fill_ring(ring, column_fragment);
-        fragment_stream<FRAGMENTS>(ring, column_fragment, [&](auto tag, const bf16x8& fragment) {
-            constexpr int F = decltype(tag)::value;
 #pragma unroll
-            for (int kt = 0; kt < KEY_TILES; ++kt) {
-                if constexpr (F < LATENT_BLOCKS) {
-                    latent_acc[kt][F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[kt], fragment, latent_acc[kt][F], 0, 0, 0);
-                } else {
-                    constexpr int J = F - LATENT_BLOCKS;
-                    latent_acc[kt][J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[kt], fragment, latent_acc[kt][J], 0, 0, 0);
+            for (int n = 0; n < 2; ++n) {
+                pf[kt][n] = dsf[kt][n] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+                if (any) {
+                    pf[kt][n] = exchange_fragment(exchange + kt * EXCHANGE_BYTES, lq, g, n);
+                    dsf[kt][n] = exchange_fragment(exchange + L::EXCHANGE_PART + kt * EXCHANGE_BYTES, lq, g, n);
                 }
             }
-            if constexpr (F % 2 == 0) request(std::integral_constant<int, F / 2>{});
+        }
+        static_for<0, 2 * PER_STEP>([&](auto tag) {
+            constexpr int I = decltype(tag)::value;
+            constexpr int N = I / PER_STEP;
+            constexpr int F = I % PER_STEP;
+            if constexpr (F < LATENT_BLOCKS) {
+#pragma unroll
+                for (int kt = 0; kt < KEY_TILES; ++kt) {
+                    latent_acc[kt][F] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[kt][N], held[I], latent_acc[kt][F], 0, 0, 0);
+                }
+                held[I] = transposed_fragment(q_latent, wide_columns.low[F % 4], wide_columns.high[F % 4],
+                                              N * 16 * Wide::ROW + 256 * (F / 4));
+            } else {
+                constexpr int J = F - LATENT_BLOCKS;
+#pragma unroll
+                for (int kt = 0; kt < KEY_TILES; ++kt) {
+                    latent_acc[kt][J] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[kt][N], held[I], latent_acc[kt][J], 0, 0, 0);
+                }
+                held[I] = transposed_fragment(do_rows, wide_columns.low[J % 4], wide_columns.high[J % 4],
+                                              N * 16 * Wide::ROW + 256 * (J / 4));
+            }
+            if constexpr (I % 2 == 0) request(std::integral_constant<int, I / 2>{});
+            if constexpr (I + 1 == 2 * PER_STEP) request(std::integral_constant<int, PER_STEP>{});
+            __builtin_amdgcn_sched_barrier(0);
         });
     };
 
-    // half tiles first .. first + count - 1; one more step lets the gradient waves catch up
-    const int first = 2 * first_tile;
-    const int count = 2 * (end_tile - first_tile);
-    begin_requests(first, 0);
-    static_for<0, REQUESTS>(request);
-    begin_requests(first + 1, 1);
+    // Step t: tile t is in buffer t % 2 (scored there, and picked up by the gradient waves for step t + 1), tile
+    // t + 1 arrives in the other buffer.  One more step after the last tile lets the gradient waves catch up.
+    begin_requests(first_tile, 0);
     static_for<0, REQUESTS>(request);
     wait_vector_memory<0>();
+    place_statistics(0);
     workgroup_barrier();
 
-    for (int h = 0; h <= count; ++h) {
-        // past the item's last half tile that one is requested again, into a buffer nobody reads: the streams stay
-        // free of branches
-        begin_requests(first + min(h + 2, count - 1), (h + 2) % L::BUFFERS);
+    for (int tile = first_tile; tile <= end_tile; ++tile) {
+        const int parity = (tile - first_tile) & 1;
+        const bool more = tile + 1 < end_tile;
+        begin_requests(more ? tile + 1 : end_tile - 1, parity ^ 1);
         if constexpr (SCORES) {
-            if (h > 0) {
-                add_rope(lds + ((h - 1) % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + ((h - 1) & 1) * L::EXCHANGE_PAIR);
-            }
-            if (h < count) {
-                score_half_tile(lds + (h % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + (h & 1) * L::EXCHANGE_PAIR);
+            if (tile < end_tile) {
+                score_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + parity * L::EXCHANGE_PAIR);
             }
         } else {
-            if (h > 0) {
-                add_half_tile(lds + ((h - 1) % L::BUFFERS) * L::BUFFER_BYTES, lds + L::EXCHANGE + ((h - 1) & 1) * L::EXCHANGE_PAIR);
-            } else {
-                static_for<0, REQUESTS>(request);
-            }
+            add_tile(lds + parity * L::BUFFER_BYTES, lds + L::EXCHANGE + (parity ^ 1) * L::EXCHANGE_PAIR, tile > first_tile);
         }
-        await_earlier_requests();
-        workgroup_barrier();   // half tile h has been scored, h - 1 read for the last time, h + 1 has arrived
+        wait_vector_memory<0>();
+        place_statistics(parity ^ 1);
+        workgroup_barrier();   // tile t has been read, P and dS of it and tile t + 1 are in place
     }
-    wait_vector_memory<0>();
 
-    // lane holds column (block, lq) and keys (first of the 32) + 8*(i/4) + 4*g + i%4: the gradient waves of both key
-    // halves and their eight latent blocks, score wave w of keys 32w .. +31 and the two rope blocks
+    // lane holds column (block, lq) and keys (first of the 32) + 8*(i/4) + 4*g + i%4: score wave w of keys 32w .. +31 and
+    // the two rope blocks, the gradient waves of both key tiles and their eight latent blocks
     float* slot = partial_slots + item * (KEY_TILES * PARTIAL_FLOATS);   // [64 keys][576]
     if constexpr (SCORES) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int key = 32 * half + 8 * (i / 4) + 4 * g + i % 4;
+            const int key = TILE * half + 8 * (i / 4) + 4 * g + i % 4;
             if (whole) {
                 if (k0 + key < T) {
                     __bf16* rope_row = reinterpret_cast<__bf16*>(key_rope_gradient) + ((size_t)batch * T + k0 + key) * ROPE;
@@ -1349,10 +1342,10 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_key_pair_gradient_kernel
     int interval_length, float scale) {
     if (threadIdx.x < THREADS / 2) {
         key_pair_walk<true>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient, logsumexp,
-                            query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
+                                 query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
     } else {
         key_pair_walk<false>(kv_latent_gradient, key_rope_gradient, partial_slots, delta_of_rows, output_gradient, logsumexp,
-                             query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
+                                  query_latent, query_rope, kv_latent, key_rope, sequence_length, heads, interval_length, scale);
     }
 }
 
