@@ -229,7 +229,8 @@ __device__ __forceinline__ void fetch_quadrant_operand(bf16x8 (&operand)[STEPS],
 // query-gradient kernel, the last of the call, overwrites after it has read the delta of its own rows).
 constexpr int DELTA_STRIDE = ROPE / 2;   // in floats
 
-// Eight threads share a row and 64 columns each; rows of all batch elements are numbered through.
+// Eight threads share a row: thread `part` takes the 16 bytes at 16 * part of each of the row's eight 128-byte
+// pieces, so that an instruction of the eight reads 128 bytes in a row; rows of all batch elements are numbered through.
 __global__ __launch_bounds__(THREADS) void mla_absorbed_row_statistics_kernel(
     float* delta, const bf16_t* __restrict__ output_gradient, const bf16_t* __restrict__ output, long long rows) {
     const int tid = threadIdx.x;
@@ -237,12 +238,12 @@ __global__ __launch_bounds__(THREADS) void mla_absorbed_row_statistics_kernel(
     const long long row = (long long)blockIdx.x * TILE + tid / 8;
     float sum = 0.f;
     if (row < rows) {
-        const bf16_t* a_row = output_gradient + row * RANK + 64 * part;
-        const bf16_t* b_row = output + row * RANK + 64 * part;
+        const bf16_t* a_row = output_gradient + row * RANK + 8 * part;
+        const bf16_t* b_row = output + row * RANK + 8 * part;
 #pragma unroll
         for (int v = 0; v < 8; ++v) {
-            const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + 8 * v);
-            const u32x4 b = *reinterpret_cast<const u32x4*>(b_row + 8 * v);
+            const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + 64 * v);
+            const u32x4 b = *reinterpret_cast<const u32x4*>(b_row + 64 * v);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 sum += bf16_bits_to_float(a[j] & 0xffffu) * bf16_bits_to_float(b[j] & 0xffffu);
