@@ -1497,17 +1497,33 @@ void mla_absorbed_backward_dispatch(bf16_t* query_latent_gradient, bf16_t* query
     const int forced = forced_interval_tiles();
     if (forced > 0 || rows * (2 * RANK + ROPE) * 2 > LARGE_INPUT_BYTES) {
         const long long slots = scratch_bytes / (PAIR * index_math::KEY_PARTIAL_BYTES);
-        const int tiles = forced > 0 ? forced
-                                     : index_math::key_interval_choice(sequence_length, heads, batch_size, slots,
-                                                                       device_compute_units(), PAIR);
-        const index_math::KeyIntervals cut = index_math::key_intervals(sequence_length, heads, tiles > 0 ? tiles : 1, PAIR);
-        const long long items = cut.items() * batch_size;
+        // (the choice walks the intervals of several lengths: remembered for the shape a thread asked about last)
+        struct Choice {
+            int sequence_length = -1, heads = -1, batch_size = -1, units = -1, forced = -1, tiles = 0;
+            long long items = 0;
+            int key_blocks = 0;
+        };
+        static thread_local Choice last;
+        const int units = device_compute_units();
+        if (last.sequence_length != sequence_length || last.heads != heads || last.batch_size != batch_size ||
+            last.units != units || last.forced != forced) {
+            last = Choice{sequence_length, heads, batch_size, units, forced, 0, 0, 0};
+            last.tiles = forced > 0 ? forced
+                                    : index_math::key_interval_choice(sequence_length, heads, batch_size, slots, units, PAIR);
+            if (last.tiles > 0) {
+                const index_math::KeyIntervals chosen = index_math::key_intervals(sequence_length, heads, last.tiles, PAIR);
+                last.items = chosen.items() * batch_size;
+                last.key_blocks = chosen.key_blocks;
+            }
+        }
+        const int tiles = last.tiles;
+        const long long items = last.items;
         // a slot for each item
         if (tiles > 0 && items <= slots && items <= 0x7fffffffLL) {
             interval_length = tiles;
             key_tiles = PAIR;
             grid = items;
-            blocks = (long long)cut.key_blocks * batch_size;
+            blocks = (long long)last.key_blocks * batch_size;
         }
     }
     long long ranges = 0;
